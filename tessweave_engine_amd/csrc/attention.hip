@@ -1,0 +1,428 @@
+// Attention over the paged cache, grouped-query, for float32 and bfloat16.
+//
+//   keys   [pages][kv_heads][page_size][head_dim]
+//   values [pages][kv_heads][head_dim][page_size]   (transposed inside a page)
+//   block_table[seq][b] = physical page of logical block b, or -1 if not held
+//
+// A query at absolute position t of a sequence with kv_len cached keys sees key
+// p iff p <= t, p < kv_len and (window == 0 or p > t - window). Scores are
+// q.k * scale; softmax statistics, probabilities and the output sum are float32.
+// Masked scores are SELECTED to -inf and keys outside the sequence are loaded
+// as zeros, so whatever an unowned or reused page holds (NaN included) never
+// reaches a result.
+//
+// The unit of work is a wave with a tile of 16 query ROWS that share one kv
+// head; a row is a (token, query head of the group) pair. Per 16 keys the wave
+// computes S^T = K Q^T on the MFMA units (accumulator element j of lane
+// (r, g) is the score of row r against key 4g + j), does the online-softmax
+// update per row, and feeds the probabilities, still in accumulator layout, as
+// the B operand of O^T += V^T P^T. Values are stored transposed in the page so
+// that the A operand of that product is one aligned load of 4 consecutive keys.
+//
+//   attn_decode_kernel   rows = the group's heads of ONE token; the sequence's
+//                        keys are split over workgroups (and over the 4 waves
+//                        of each); partial results are merged in a fixed order.
+//   attn_prefill_kernel  rows = (token, head) pairs of a prompt portion; each
+//                        wave walks the keys its rows can see.
+#include "tw_common.h"
+
+template <typename T> __device__ __forceinline__ float tw_exp(float v);
+template <> __device__ __forceinline__ float tw_exp<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ float tw_exp<bf16_t>(float v) { return __expf(v); }
+
+template <typename T> struct KeyQuad;          // 4 consecutive keys of one d (A operand of the PV product)
+template <> struct KeyQuad<float> { typedef f32x4 Type; };
+template <> struct KeyQuad<bf16_t> { typedef bf16x4 Type; };
+
+template <typename T, int DTMAX> struct AttnShape {
+  static constexpr int EPF = Elem<T>::kPerFrag;
+  static constexpr int NSMAX = (DTMAX * 16 / EPF + 3) / 4;    // MFMA steps over head_dim
+};
+
+struct AttnArgs {
+  const void* q;          // [rows][ldq], head h of row n at q + n*ldq + h*head_dim
+  long ldq;
+  const void* keys;
+  const void* values;
+  const int* block_table;
+  int table_stride;
+  const int* q_start;     // [n_seqs + 1] first token row of each sequence
+  const int* kv_len;      // [n_seqs] keys cached, this step's tokens included
+  int seq0;               // first sequence this launch covers
+  void* out;              // [rows][ldo]
+  long ldo;
+  float* part_o;          // decode partials [seq - seq0][q_heads][splits][head_dim]
+  float* part_ml;         // [seq - seq0][q_heads][splits][2]  (max, sum)
+  int q_heads, kv_heads, head_dim, page_size, window;
+  float scale;
+  int splits;
+};
+
+// Per-wave online-softmax state for one 16-row tile. Lane (r, g) belongs to row r.
+template <typename T, int DTMAX>
+struct RowTile {
+  typedef typename Elem<T>::Frag Frag;
+  typedef typename KeyQuad<T>::Type Quad;
+  static constexpr int EPF = Elem<T>::kPerFrag;
+  static constexpr int NSMAX = AttnShape<T, DTMAX>::NSMAX;
+
+  Frag qf[NSMAX];
+  f32x4 acc[DTMAX];
+  float m, l;
+
+  __device__ __forceinline__ void init(const T* q_row /* null: no such row */, int head_dim, int g) {
+    const int chunks = head_dim / EPF;
+#pragma unroll
+    for (int s = 0; s < NSMAX; ++s) {
+      const int chunk = s * 4 + g;
+      qf[s] = (q_row && chunk < chunks) ? tw_load_frag(q_row + chunk * EPF) : Elem<T>::zero();
+    }
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    m = -INFINITY;
+    l = 0.f;
+  }
+
+  // One tile of 16 keys starting at position p0 (a multiple of 16).
+  // t_row: position of this lane's row (-1: no such row). lo_load: keys below it are never loaded.
+  __device__ __forceinline__ void key_tile(const AttnArgs& a, const int* table, int kvh, int p0, int kv_len,
+                                           int t_row, int lo_load, int r, int g) {
+    const T* keys = (const T*)a.keys;
+    const T* values = (const T*)a.values;
+    const int D = a.head_dim, P = a.page_size;
+    const int chunks = D / EPF, dts = D / 16;
+    // ---- S^T = K Q^T ------------------------------------------------------
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    {
+      const int p = p0 + r;                       // this lane loads key p's fragments
+      int page = -1;
+      if (p < kv_len && p >= lo_load) page = table[p / P];
+      const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh) * P + p % P) * D;
+#pragma unroll
+      for (int st = 0; st < NSMAX; ++st) {
+        const int chunk = st * 4 + g;
+        if (st * 4 < chunks) {
+          const Frag kf = (page >= 0 && chunk < chunks) ? tw_load_frag(k_row + chunk * EPF) : Elem<T>::zero();
+          tw_mma16(s, kf, qf[st]);
+        }
+      }
+    }
+    // ---- mask, online softmax (this lane: row r, keys p0 + 4g + j) ------------
+    const int lo_row = a.window > 0 ? t_row - a.window + 1 : 0;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int p = p0 + 4 * g + j;
+      const bool ok = p < kv_len && p <= t_row && p >= lo_row;
+      s[j] = ok ? s[j] * a.scale : -INFINITY;
+      mx = fmaxf(mx, s[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = tw_exp<T>(m - m_use);
+    f32x4 pr;
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      pr[j] = tw_exp<T>(s[j] - m_use);
+      sum += pr[j];
+    }
+    sum += __shfl_xor(sum, 16, TW_WAVE);
+    sum += __shfl_xor(sum, 32, TW_WAVE);
+    l = l * alpha + sum;
+    m = m_new;
+    // ---- O^T += V^T P^T (this lane loads d = 16 dt + r, keys p0 + 4g .. + 3) ----
+    const int pv = p0 + 4 * g;
+    int vpage = -1;
+    if (pv < kv_len && pv + 3 >= lo_load) vpage = table[pv / P];
+    const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.kv_heads + kvh) * D * P + pv % P;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt) {
+      if (dt < dts) {
+        Quad vq;
+        if (vpage >= 0) {
+          vq = *reinterpret_cast<const Quad*>(v_base + (size_t)(dt * 16 + r) * P);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (pv + j >= kv_len || pv + j < lo_load) vq[j] = tw_from_float<T>(0.f);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) vq[j] = tw_from_float<T>(0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[dt][j] *= alpha;
+        tw_mma16_k4(acc[dt], vq, pr);
+      }
+    }
+  }
+};
+
+// =====================================================================================
+// Decode: one token per sequence. grid = (splits, kv_heads * row_tiles, n_seqs).
+// =====================================================================================
+template <typename T, int DTMAX>
+__global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
+  __shared__ float lds_o[3][16][DTMAX * 16];
+  __shared__ float lds_ml[3][16][2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int G = a.q_heads / a.kv_heads;
+  const int row_tiles = (G + 15) / 16;
+  const int kvh = blockIdx.y / row_tiles, rt = blockIdx.y % row_tiles;
+  const int seq = a.seq0 + blockIdx.z;
+  const int split = blockIdx.x;
+  const int kv_len = a.kv_len[seq];
+  const int token = a.q_start[seq];
+  const int t = kv_len - 1;
+  const int* table = a.block_table + (size_t)seq * a.table_stride;
+  const int D = a.head_dim, dts = D / 16;
+
+  const int hig = rt * 16 + r;                      // head within the group
+  const bool row_ok = hig < G;
+  const int head = kvh * G + hig;
+  RowTile<T, DTMAX> tile;
+  tile.init(row_ok ? (const T*)a.q + (size_t)token * a.ldq + (size_t)head * D : nullptr, D, g);
+
+  const int lo = a.window > 0 ? max(0, t - a.window + 1) : 0;
+  const int tile_lo = lo / 16, tile_hi = (kv_len + 15) / 16;     // key tiles [tile_lo, tile_hi)
+  const int per_split = (tile_hi - tile_lo + a.splits - 1) / a.splits;
+  const int begin = tile_lo + split * per_split;
+  const int end = min(tile_hi, begin + per_split);
+  for (int kt = begin + wave; kt < end; kt += 4)
+    tile.key_tile(a, table, kvh, kt * 16, kv_len, row_ok ? t : -1, lo, r, g);
+
+  // ---- merge the 4 waves (fixed order: wave 0 absorbs 1, 2, 3) -------------------
+  if (wave > 0) {
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) lds_o[wave - 1][r][dt * 16 + 4 * g + j] = tile.acc[dt][j];
+    if (g == 0) {
+      lds_ml[wave - 1][r][0] = tile.m;
+      lds_ml[wave - 1][r][1] = tile.l;
+    }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  float m = tile.m, l = tile.l;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) m = fmaxf(m, lds_ml[w][r][0]);
+  const float m_use = m == -INFINITY ? 0.f : m;
+  const float own = tw_exp<T>(tile.m - m_use);
+  l *= own;
+#pragma unroll
+  for (int dt = 0; dt < DTMAX; ++dt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tile.acc[dt][j] *= own;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    const float f = tw_exp<T>(lds_ml[w][r][0] - m_use);
+    l += lds_ml[w][r][1] * f;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tile.acc[dt][j] += lds_o[w][r][dt * 16 + 4 * g + j] * f;
+  }
+  if (!row_ok) return;
+  if (a.splits == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    T* dst = (T*)a.out + (size_t)token * a.ldo + (size_t)head * D;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = tw_from_float<T>(tile.acc[dt][j] * inv);
+  } else {
+    const size_t slot = ((size_t)blockIdx.z * a.q_heads + head) * a.splits + split;
+    float* dst = a.part_o + slot * D;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = tile.acc[dt][j];
+    if (g == 0) {
+      a.part_ml[slot * 2] = m;
+      a.part_ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
+// Merge the splits of one (sequence, head): grid = (q_heads, n_seqs), one thread per d.
+template <typename T>
+__global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                          const int* __restrict__ q_start, int seq0, T* out, long ldo,
+                                          int q_heads, int head_dim, int splits) {
+  const int head = blockIdx.x, local = blockIdx.y;
+  const size_t slot0 = ((size_t)local * q_heads + head) * splits;
+  float m = -INFINITY;
+  for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+  const float m_use = m == -INFINITY ? 0.f : m;
+  float l = 0.f;
+  for (int s = 0; s < splits; ++s) l += part_ml[(slot0 + s) * 2 + 1] * expf(part_ml[(slot0 + s) * 2] - m_use);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const int token = q_start[seq0 + local];
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < splits; ++s)
+      o += part_o[(slot0 + s) * head_dim + d] * expf(part_ml[(slot0 + s) * 2] - m_use);
+    out[(size_t)token * ldo + (size_t)head * head_dim + d] = tw_from_float<T>(o * inv);
+  }
+}
+
+// =====================================================================================
+// Prefill: q_len tokens of a sequence. grid = (row tiles / 4, kv_heads, n_seqs);
+// each of the 4 waves of a workgroup takes one tile of 16 (token, head) rows.
+// =====================================================================================
+template <typename T, int DTMAX>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int G = a.q_heads / a.kv_heads;
+  const int kvh = blockIdx.y;
+  const int seq = a.seq0 + blockIdx.z;
+  const int kv_len = a.kv_len[seq];
+  const int token0 = a.q_start[seq];
+  const int q_len = a.q_start[seq + 1] - token0;
+  const int rows = q_len * G;
+  const int row0 = (blockIdx.x * 4 + wave) * 16;
+  if (row0 >= rows) return;
+  const int* table = a.block_table + (size_t)seq * a.table_stride;
+  const int D = a.head_dim, dts = D / 16;
+
+  const int row = row0 + r;
+  const bool row_ok = row < rows;
+  const int tok = row / G, hig = row % G;            // token within the portion, head within the group
+  const int head = kvh * G + hig;
+  const int first_pos = kv_len - q_len;              // position of the portion's first token
+  const int t_row = row_ok ? first_pos + tok : -1;
+  RowTile<T, DTMAX> tile;
+  tile.init(row_ok ? (const T*)a.q + (size_t)(token0 + tok) * a.ldq + (size_t)head * D : nullptr, D, g);
+
+  const int t_min = first_pos + row0 / G;
+  const int t_max = first_pos + min(rows - 1, row0 + 15) / G;
+  const int lo = a.window > 0 ? max(0, t_min - a.window + 1) : 0;
+  for (int kt = lo / 16; kt * 16 <= t_max; ++kt)
+    tile.key_tile(a, table, kvh, kt * 16, kv_len, t_row, lo, r, g);
+
+  if (!row_ok) return;
+  const float inv = tile.l > 0.f ? 1.f / tile.l : 0.f;
+  T* dst = (T*)a.out + (size_t)(token0 + tok) * a.ldo + (size_t)head * D;
+#pragma unroll
+  for (int dt = 0; dt < DTMAX; ++dt)
+    if (dt < dts)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = tw_from_float<T>(tile.acc[dt][j] * inv);
+}
+
+// =====================================================================================
+// Host side
+// =====================================================================================
+static int check_common(const AttnArgs& a) {
+  TW_REQUIRE(a.q_heads > 0 && a.kv_heads > 0 && a.q_heads % a.kv_heads == 0);
+  TW_REQUIRE(a.head_dim >= 16 && a.head_dim <= 256 && a.head_dim % 16 == 0);
+  TW_REQUIRE(a.page_size >= 4 && a.page_size % 4 == 0);
+  TW_REQUIRE(a.window >= 0 && a.table_stride > 0);
+  TW_REQUIRE(a.ldq >= (long)a.q_heads * a.head_dim && a.ldo >= (long)a.q_heads * a.head_dim);
+  TW_REQUIRE(a.ldq % 8 == 0 && ((uintptr_t)a.q % 16 == 0));
+  return 0;
+}
+
+extern "C" int tw_attn_decode_splits(int n_seqs, int q_heads, int kv_heads, int max_kv_len) {
+  const int G = q_heads / kv_heads;
+  const int units = n_seqs * kv_heads * ((G + 15) / 16);
+  int splits = tw_div_up(1024, units > 0 ? units : 1);
+  const int by_len = tw_div_up(max_kv_len, 256);
+  if (splits > by_len) splits = by_len;
+  if (splits > 64) splits = 64;
+  return splits < 1 ? 1 : splits;
+}
+
+extern "C" long tw_attn_decode_workspace_floats(int n_seqs, int q_heads, int head_dim, int splits) {
+  return splits > 1 ? (long)n_seqs * q_heads * splits * (head_dim + 2) : 0;
+}
+
+template <typename T>
+static int decode_launch(AttnArgs a, int n_seqs, hipStream_t stream) {
+  const int G = a.q_heads / a.kv_heads;
+  dim3 grid(a.splits, a.kv_heads * ((G + 15) / 16), n_seqs);
+  if (a.head_dim <= 64)
+    attn_decode_kernel<T, 4><<<grid, 256, 0, stream>>>(a);
+  else if (a.head_dim <= 128)
+    attn_decode_kernel<T, 8><<<grid, 256, 0, stream>>>(a);
+  else
+    attn_decode_kernel<T, 16><<<grid, 256, 0, stream>>>(a);
+  int err = TW_LAUNCH_RESULT();
+  if (err || a.splits == 1) return err;
+  const int threads = a.head_dim <= 64 ? 64 : (a.head_dim <= 128 ? 128 : 256);
+  attn_decode_reduce_kernel<T><<<dim3(a.q_heads, n_seqs), threads, 0, stream>>>(
+      a.part_o, a.part_ml, a.q_start, a.seq0, (T*)a.out, a.ldo, a.q_heads, a.head_dim, a.splits);
+  return TW_LAUNCH_RESULT();
+}
+
+// Sequences seq0 .. seq0 + n_seqs - 1 must each have exactly one token in this step.
+// `workspace` holds tw_attn_decode_workspace_floats floats when splits > 1.
+extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* keys, const void* values,
+                              const int* block_table, int table_stride, const int* q_start,
+                              const int* kv_len, int seq0, int n_seqs, void* out, long ldo,
+                              float* workspace, long workspace_floats, int q_heads, int kv_heads,
+                              int head_dim, int page_size, int window, float scale, int splits,
+                              hipStream_t stream) {
+  AttnArgs a;
+  a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
+  a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
+  a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
+  a.page_size = page_size; a.window = window; a.scale = scale; a.splits = splits;
+  a.part_o = nullptr; a.part_ml = nullptr;
+  int err = check_common(a);
+  if (err) return err;
+  TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && splits >= 1 && splits <= 64 && n_seqs <= 65535);
+  if (n_seqs == 0) return 0;
+  if (splits > 1) {
+    TW_REQUIRE(workspace != nullptr);
+    TW_REQUIRE(workspace_floats >= tw_attn_decode_workspace_floats(n_seqs, q_heads, head_dim, splits));
+    a.part_o = workspace;
+    a.part_ml = workspace + (size_t)n_seqs * q_heads * splits * head_dim;
+  }
+  if (dtype == TW_DTYPE_F32) return decode_launch<float>(a, n_seqs, stream);
+  if (dtype == TW_DTYPE_BF16) return decode_launch<bf16_t>(a, n_seqs, stream);
+  return TW_ERR_BAD_ARGUMENT;
+}
+
+template <typename T>
+static int prefill_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
+  const int G = a.q_heads / a.kv_heads;
+  const long rows = (long)max_q_len * G;
+  dim3 grid(tw_div_up(rows, 64), a.kv_heads, n_seqs);
+  if (a.head_dim <= 64)
+    attn_prefill_kernel<T, 4><<<grid, 256, 0, stream>>>(a);
+  else if (a.head_dim <= 128)
+    attn_prefill_kernel<T, 8><<<grid, 256, 0, stream>>>(a);
+  else
+    attn_prefill_kernel<T, 16><<<grid, 256, 0, stream>>>(a);
+  return TW_LAUNCH_RESULT();
+}
+
+// Sequences seq0 .. seq0 + n_seqs - 1 with any number of tokens (at most max_q_len) each.
+extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* keys, const void* values,
+                               const int* block_table, int table_stride, const int* q_start,
+                               const int* kv_len, int seq0, int n_seqs, int max_q_len, void* out,
+                               long ldo, int q_heads, int kv_heads, int head_dim, int page_size,
+                               int window, float scale, hipStream_t stream) {
+  AttnArgs a;
+  a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
+  a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
+  a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
+  a.page_size = page_size; a.window = window; a.scale = scale; a.splits = 1;
+  a.part_o = nullptr; a.part_ml = nullptr;
+  int err = check_common(a);
+  if (err) return err;
+  TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && max_q_len >= 1 && n_seqs <= 65535);
+  if (n_seqs == 0) return 0;
+  if (dtype == TW_DTYPE_F32) return prefill_launch<float>(a, n_seqs, max_q_len, stream);
+  if (dtype == TW_DTYPE_BF16) return prefill_launch<bf16_t>(a, n_seqs, max_q_len, stream);
+  return TW_ERR_BAD_ARGUMENT;
+}

@@ -1,0 +1,203 @@
+// Row kernels: embedding gather, RMS norm, rotary tables, rotation + cache
+// write, SiLU-multiply. Statistics, angles and products are float32; storage
+// is float32 or bfloat16. The residual stream is float32 in both precisions.
+#include "tw_common.h"
+
+// ---- embedding: x[n, :] = float(E[ids[n], :]) ------------------------------------
+template <typename T>
+__global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                    float* __restrict__ out, int hidden, int vocab) {
+  const int n = blockIdx.x;
+  int id = ids[n];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // ids are validated on the host; never read outside
+  const T* row = table + (size_t)id * hidden;
+  float* dst = out + (size_t)n * hidden;
+  for (int h = threadIdx.x; h < hidden; h += blockDim.x) dst[h] = tw_to_float(row[h]);
+}
+
+extern "C" int tw_embed_gather(int dtype, const int* ids, const void* table, float* out, int n,
+                               int hidden, int vocab, hipStream_t stream) {
+  TW_REQUIRE(n >= 0 && hidden > 0 && vocab > 0);
+  if (n == 0) return 0;
+  if (dtype == TW_DTYPE_F32)
+    embed_gather_kernel<float><<<n, 256, 0, stream>>>(ids, (const float*)table, out, hidden, vocab);
+  else if (dtype == TW_DTYPE_BF16)
+    embed_gather_kernel<bf16_t><<<n, 256, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- RMS norm -------------------------------------------------------------------------
+// y = x * rsqrt(mean(x^2) + eps) * w, statistics and products in float32, one
+// rounding to the output type. `rows` (optional) picks the input row of each
+// output row. If `add` is given the input row is x + sum_s add[s] and that sum
+// is written back to x first (split-K partial sums of the layer before).
+template <typename T>
+__global__ void rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ w, T* __restrict__ out,
+                               const int* __restrict__ rows, int hidden, float eps,
+                               const float* __restrict__ add, int add_splits, size_t add_stride) {
+  __shared__ float lds[16];
+  const int o = blockIdx.x;
+  const int r = rows ? rows[o] : o;
+  float* src = x + (size_t)r * hidden;
+  float ss = 0.f;
+  if (add) {
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+      float v = src[h];
+      for (int s = 0; s < add_splits; ++s) v += add[s * add_stride + (size_t)r * hidden + h];
+      src[h] = v;
+      ss += v * v;
+    }
+  } else {
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+      const float v = src[h];
+      ss += v * v;
+    }
+  }
+  ss = tw_block_sum(ss, lds);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+  T* dst = out + (size_t)o * hidden;
+  for (int h = threadIdx.x; h < hidden; h += blockDim.x)
+    dst[h] = tw_from_float<T>(src[h] * scale * w[h]);
+}
+
+extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, const int* rows,
+                          int n_out, int hidden, float eps, const float* add, int add_splits,
+                          long add_stride, hipStream_t stream) {
+  TW_REQUIRE(n_out >= 0 && hidden > 0 && eps > 0.f);
+  TW_REQUIRE(add == nullptr || (rows == nullptr && add_splits > 0));
+  if (n_out == 0) return 0;
+  const int threads = hidden >= 2048 ? 512 : 256;
+  if (out_dtype == TW_DTYPE_F32)
+    rmsnorm_kernel<float><<<n_out, threads, 0, stream>>>(x, w, (float*)out, rows, hidden, eps, add,
+                                                         add_splits, (size_t)add_stride);
+  else if (out_dtype == TW_DTYPE_BF16)
+    rmsnorm_kernel<bf16_t><<<n_out, threads, 0, stream>>>(x, w, (bf16_t*)out, rows, hidden, eps, add,
+                                                          add_splits, (size_t)add_stride);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- rotary tables: cos/sin[n, j] of angle = float(position[n]) * inv_freq[j] -----
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float* __restrict__ cos_out, float* __restrict__ sin_out, int n, int half) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * half) return;
+  const int t = i / half, j = i % half;
+  const float angle = (float)positions[t] * inv_freq[j];
+  cos_out[i] = cosf(angle);
+  sin_out[i] = sinf(angle);
+}
+
+extern "C" int tw_rope_table(const int* positions, const float* inv_freq, float* cos_out, float* sin_out,
+                             int n, int half, hipStream_t stream) {
+  TW_REQUIRE(n >= 0 && half > 0);
+  if (n == 0) return 0;
+  rope_table_kernel<<<tw_div_up((long)n * half, 256), 256, 0, stream>>>(positions, inv_freq, cos_out,
+                                                                       sin_out, n, half);
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- rotation of q and k, and the cache write ----------------------------------------------
+// qkv[n] = [q heads | k heads | v heads], head-major, `ld` elements per row.
+// Pair j of a head is (x[j], x[j + rot/2]) for j < rot/2 (rotate-half); elements
+// from `rot` on are not rotated. q is rotated in place. Rotated k goes to
+//   keys  [page][kv_head][offset][d]      and raw v to
+//   values[page][kv_head][d][offset]      (transposed inside the page),
+// slot = page * page_size + offset; a negative slot writes nothing.
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* __restrict__ cos_t,
+                                     const float* __restrict__ sin_t, const int* __restrict__ slots,
+                                     T* __restrict__ keys, T* __restrict__ values, int q_heads,
+                                     int kv_heads, int head_dim, int rot, int page_size, int write_cache) {
+  const int n = blockIdx.x;
+  const int half = rot / 2;
+  T* row = qkv + (size_t)n * ld;
+  const float* c = cos_t + (size_t)n * half;
+  const float* s = sin_t + (size_t)n * half;
+  const int slot = write_cache ? slots[n] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  const int rot_heads = q_heads + kv_heads;
+  // rotated part: one thread per pair
+  for (int i = threadIdx.x; i < rot_heads * half; i += blockDim.x) {
+    const int head = i / half, j = i % half;
+    T* x = row + (size_t)head * head_dim;
+    const float lo = tw_to_float(x[j]), hi = tw_to_float(x[j + half]);
+    const float cj = c[j], sj = s[j];
+    const T out_lo = tw_from_float<T>(lo * cj - hi * sj);
+    const T out_hi = tw_from_float<T>(hi * cj + lo * sj);
+    if (head < q_heads) {
+      x[j] = out_lo;
+      x[j + half] = out_hi;
+    } else if (slot >= 0) {
+      const int kh = head - q_heads;
+      T* dst = keys + (((size_t)page * kv_heads + kh) * page_size + off) * head_dim;
+      dst[j] = out_lo;
+      dst[j + half] = out_hi;
+    }
+  }
+  if (slot < 0) return;
+  // unrotated tail of the keys
+  const int tail = head_dim - rot;
+  for (int i = threadIdx.x; i < kv_heads * tail; i += blockDim.x) {
+    const int kh = i / tail, d = rot + i % tail;
+    keys[(((size_t)page * kv_heads + kh) * page_size + off) * head_dim + d] =
+        row[(size_t)(q_heads + kh) * head_dim + d];
+  }
+  // values, transposed inside the page
+  const T* v = row + (size_t)(q_heads + kv_heads) * head_dim;
+  for (int i = threadIdx.x; i < kv_heads * head_dim; i += blockDim.x) {
+    const int kh = i / head_dim, d = i % head_dim;
+    values[(((size_t)page * kv_heads + kh) * head_dim + d) * page_size + off] = v[i];
+  }
+}
+
+extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_t, const float* sin_t,
+                                const int* slots, void* keys, void* values, int n, int q_heads,
+                                int kv_heads, int head_dim, int rot, int page_size, int write_cache,
+                                hipStream_t stream) {
+  TW_REQUIRE(n >= 0 && q_heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0);
+  TW_REQUIRE(rot >= 0 && rot <= head_dim && rot % 2 == 0);
+  TW_REQUIRE(ld >= (long)(q_heads + 2 * kv_heads) * head_dim);
+  TW_REQUIRE(!write_cache || (slots && keys && values));
+  if (n == 0) return 0;
+  if (dtype == TW_DTYPE_F32)
+    rope_kv_write_kernel<float><<<n, 256, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
+                                                       (float*)values, q_heads, kv_heads, head_dim, rot,
+                                                       page_size, write_cache);
+  else if (dtype == TW_DTYPE_BF16)
+    rope_kv_write_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots,
+                                                        (bf16_t*)keys, (bf16_t*)values, q_heads, kv_heads,
+                                                        head_dim, rot, page_size, write_cache);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- SiLU-multiply: out[n, i] = silu(gu[n, i]) * gu[n, inter + i] -------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int inter) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * inter) return;
+  const long row = i / inter;
+  const int col = (int)(i % inter);
+  const float g = tw_to_float(gu[row * 2 * inter + col]);
+  const float u = tw_to_float(gu[row * 2 * inter + inter + col]);
+  out[i] = tw_from_float<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int tw_silu_mul(int dtype, const void* gu, void* out, int n, int inter, hipStream_t stream) {
+  TW_REQUIRE(n >= 0 && inter > 0);
+  if (n == 0) return 0;
+  const int blocks = tw_div_up((long)n * inter, 256);
+  if (dtype == TW_DTYPE_F32)
+    silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, n, inter);
+  else if (dtype == TW_DTYPE_BF16)
+    silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, inter);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}

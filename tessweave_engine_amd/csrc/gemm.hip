@@ -1,0 +1,359 @@
+// Linear layers: C[M, N] = A[M, K] * W[N, K]^T (+ bias[N]) (+ residual[M, N]).
+// A and W are both contiguous along K (the checkpoint's [out, in] layout), in
+// float32 or bfloat16; accumulation is float32 on the MFMA units (true float32
+// MFMA for float32 inputs, no reduced-precision matrix mode). Three kernels:
+//   gemm_tiled   - many rows (prompt portions): LDS-staged 32x32 MFMA tiles
+//   gemm_skinny  - few rows (decode): weights streamed once from HBM straight
+//                  into 16x16 MFMA fragments, split over K when N is small
+//   gemm_generic - any K (rows not 16-byte aligned): one output per thread
+#include "tw_common.h"
+
+// =====================================================================================
+// Tiled kernel. Workgroup = 4 waves in a 2x2 grid, wave tile (32*WM) x (32*WN).
+// One stage holds 128 bytes of K per row (64 bf16 / 32 f32), rows padded to 144
+// bytes in LDS so that 16-byte fragment reads of 8 consecutive lanes hit
+// distinct banks. Two stages: the next stage's global loads are in flight
+// while the current one is multiplied.
+// =====================================================================================
+#define TW_LDS_ROW 144
+
+template <typename T, typename OutT, int WM, int WN>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A, long lda,
+                                                         const T* __restrict__ W, long ldw,
+                                                         const float* __restrict__ bias,
+                                                         const float* residual, long ldr, OutT* C,
+                                                         long ldc, int M, int N, int K, int tiles_m,
+                                                         int n_blocks) {
+  typedef typename Elem<T>::Frag Frag;
+  constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr int BK = 8 * EPF;
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int A_LOADS = BM / 32, W_LOADS = BN / 32;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+
+  // Blocks are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
+  // of tiles so that neighbours sharing a weight tile share an L2.
+  const int per_xcd = gridDim.x / 8;
+  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (logical >= n_blocks) return;
+  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave >> 1) * 32 * WM, wn0 = (wave & 1) * 32 * WN;
+  const int r = lane & 31, g = lane >> 5;
+
+  constexpr int STAGE = (BM + BN) * TW_LDS_ROW;            // bytes of one stage: A rows then W rows
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  Frag a_reg[A_LOADS], w_reg[W_LOADS];
+  const int k_tiles = (K + BK - 1) / BK;
+
+  auto load_global = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
+      const int gm = m0 + row, gk = kt * BK + kc * EPF;
+      a_reg[i] = (gm < M && gk < K) ? tw_load_frag(A + (size_t)gm * lda + gk) : Elem<T>::zero();
+    }
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
+      const int gn = n0 + row, gk = kt * BK + kc * EPF;
+      w_reg[i] = (gn < N && gk < K) ? tw_load_frag(W + (size_t)gn * ldw + gk) : Elem<T>::zero();
+    }
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
+      *reinterpret_cast<Frag*>(lds + buf * STAGE + row * TW_LDS_ROW + kc * 16) = a_reg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
+      *reinterpret_cast<Frag*>(lds + buf * STAGE + (BM + row) * TW_LDS_ROW + kc * 16) = w_reg[i];
+    }
+  };
+
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < k_tiles) load_global(kt + 1);
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      Frag af[WM], wf[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+        af[i] = *reinterpret_cast<const Frag*>(lds + buf * STAGE + (wm0 + i * 32 + r) * TW_LDS_ROW + (2 * cc + g) * 16);
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+        wf[j] = *reinterpret_cast<const Frag*>(lds + buf * STAGE + (BM + wn0 + j * 32 + r) * TW_LDS_ROW + (2 * cc + g) * 16);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[i], wf[j]);
+    }
+    if (kt + 1 < k_tiles) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      const int col = n0 + wn0 + j * 32 + r;
+      if (col >= N) continue;
+      const float b = bias ? bias[col] : 0.f;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm0 + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
+        if (row >= M) continue;
+        float v = acc[i][j][e] + b;
+        if (residual) v += residual[(size_t)row * ldr + col];
+        C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
+      }
+    }
+}
+
+// =====================================================================================
+// Skinny kernel: M <= 16*MT rows. Each wave owns 16 output columns (16 rows of
+// W) and one K range; it loads weight fragments straight from global memory
+// (every weight byte is read by exactly one wave, 64 contiguous bytes per row
+// per load instruction) and the matching activation fragments from L2.
+// SPLITS == 1: the epilogue runs here. SPLITS > 1: float32 partial sums go to
+// `partial[split][M][N]` and `splitk_reduce_kernel` finishes, always in the
+// same order, so results do not depend on timing.
+// =====================================================================================
+template <typename T, typename OutT, int MT>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const T* __restrict__ A, long lda,
+                                                          const T* __restrict__ W, long ldw,
+                                                          const float* __restrict__ bias,
+                                                          const float* residual, long ldr, OutT* C,
+                                                          long ldc, float* __restrict__ partial, int M,
+                                                          int N, int K, int n_tiles, int splits) {
+  typedef typename Elem<T>::Frag Frag;
+  constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr int U = 4;                       // MFMA steps per loop iteration
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int unit = blockIdx.x * 4 + wave;
+  if (unit >= n_tiles * splits) return;
+  const int tile = unit % n_tiles, split = unit / n_tiles;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = tile * 16;
+
+  const int chunks = K / EPF;                              // 16-byte chunks per row
+  const int steps = (chunks + 3) / 4;                      // MFMA steps over all of K
+  const int steps_per_split = (steps + splits - 1) / splits;
+  const int step_begin = split * steps_per_split;
+  const int step_end = min(steps, step_begin + steps_per_split);
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const bool w_row_ok = n0 + r < N;
+  const T* w_row = W + (size_t)(w_row_ok ? n0 + r : 0) * ldw;
+  const T* a_row[MT];
+  bool a_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    a_ok[mt] = mt * 16 + r < M;
+    a_row[mt] = A + (size_t)(a_ok[mt] ? mt * 16 + r : 0) * lda;
+  }
+
+  for (int s0 = step_begin; s0 < step_end; s0 += U) {
+    Frag wf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int chunk = (s0 + u) * 4 + g;
+      const bool ok = w_row_ok && (s0 + u) < step_end && chunk < chunks;
+      wf[u] = ok ? tw_load_frag(w_row + (size_t)chunk * EPF) : Elem<T>::zero();
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int chunk = (s0 + u) * 4 + g;
+      const bool in_k = (s0 + u) < step_end && chunk < chunks;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const Frag af = (a_ok[mt] && in_k) ? tw_load_frag(a_row[mt] + (size_t)chunk * EPF) : Elem<T>::zero();
+        tw_mma16(acc[mt], wf[u], af);
+      }
+    }
+  }
+
+  // acc[mt][j] = sum_k W[n0 + 4g + j][k] * A[16 mt + r][k]
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int row = mt * 16 + r;
+    if (row >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + 4 * g + j;
+      if (col >= N) continue;
+      if (splits > 1) {
+        partial[((size_t)split * M + row) * N + col] = acc[mt][j];
+      } else {
+        float v = acc[mt][j] + (bias ? bias[col] : 0.f);
+        if (residual) v += residual[(size_t)row * ldr + col];
+        C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
+      }
+    }
+  }
+}
+
+template <typename OutT>
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, int splits,
+                                     const float* __restrict__ bias, const float* residual, long ldr,
+                                     OutT* C, long ldc, int M, int N) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)M * N) return;
+  const int row = (int)(i / N), col = (int)(i % N);
+  float v = 0.f;
+  for (int s = 0; s < splits; ++s) v += partial[(size_t)s * M * N + i];
+  if (bias) v += bias[col];
+  if (residual) v += residual[(size_t)row * ldr + col];
+  C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
+}
+
+// =====================================================================================
+// Generic kernel: any K. One thread per output element, float32 accumulation.
+// =====================================================================================
+template <typename T, typename OutT>
+__global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* __restrict__ W, long ldw,
+                                    const float* __restrict__ bias, const float* residual, long ldr,
+                                    OutT* C, long ldc, int M, int N, int K) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)M * N) return;
+  const int row = (int)(i / N), col = (int)(i % N);
+  const T* a = A + (size_t)row * lda;
+  const T* w = W + (size_t)col * ldw;
+  float v = 0.f;
+  for (int k = 0; k < K; ++k) v = fmaf(tw_to_float(a[k]), tw_to_float(w[k]), v);
+  if (bias) v += bias[col];
+  if (residual) v += residual[(size_t)row * ldr + col];
+  C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
+}
+
+// =====================================================================================
+// Host side
+// =====================================================================================
+template <typename T, typename OutT, int WM, int WN>
+static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
+                        const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
+                        hipStream_t stream) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
+  const long n_blocks = (long)tiles_m * tiles_n;
+  TW_REQUIRE(n_blocks < (1L << 30));
+  const int grid = (int)((n_blocks + 7) / 8 * 8);
+  const size_t lds_bytes = 2 * (size_t)(BM + BN) * TW_LDS_ROW;
+  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN>;
+  static bool attribute_set = false;   // per instantiation
+  if (!attribute_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    attribute_set = true;
+  }
+  kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m,
+                                           (int)n_blocks);
+  return TW_LAUNCH_RESULT();
+}
+
+// How many K ranges the skinny kernel uses for an [N, K] weight: enough waves
+// to fill 256 CUs several times over, each range at least 32 MFMA steps long.
+// The choice depends on N and K only, never on the rows of a batch.
+static int skinny_splits(int N, int K, int epf) {
+  const int n_tiles = tw_div_up(N, 16);
+  const int steps = tw_div_up(K / epf, 4);
+  int splits = tw_div_up(2048, n_tiles);
+  const int max_by_k = steps / 32 > 0 ? steps / 32 : 1;
+  if (splits > max_by_k) splits = max_by_k;
+  if (splits > 16) splits = 16;
+  return splits < 1 ? 1 : splits;
+}
+
+extern "C" long tw_linear_workspace_bytes(int dtype, int max_rows, int N, int K) {
+  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
+  if (K % epf) return 0;
+  const int rows = max_rows < 64 ? max_rows : 64;
+  const int splits = skinny_splits(N, K, epf);
+  return splits > 1 ? (long)splits * rows * N * 4 : 0;
+}
+
+template <typename T, typename OutT, int MT>
+static int launch_skinny(const T* A, long lda, const T* W, long ldw, const float* bias,
+                         const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                         long partial_bytes, int M, int N, int K, hipStream_t stream) {
+  constexpr int EPF = Elem<T>::kPerFrag;
+  const int n_tiles = tw_div_up(N, 16);
+  int splits = skinny_splits(N, K, EPF);
+  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) splits = 1;
+  const int units = n_tiles * splits;
+  gemm_skinny_kernel<T, OutT, MT><<<tw_div_up(units, 4), 256, 0, stream>>>(
+      A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, n_tiles, splits);
+  int err = TW_LAUNCH_RESULT();
+  if (err || splits == 1) return err;
+  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
+                                                                             ldr, C, ldc, M, N);
+  return TW_LAUNCH_RESULT();
+}
+
+template <typename T, typename OutT>
+static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const float* bias,
+                           const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                           long partial_bytes, int M, int N, int K, int force, hipStream_t stream) {
+  constexpr int EPF = Elem<T>::kPerFrag;
+  const bool aligned = K % EPF == 0 && lda % EPF == 0 && ldw % EPF == 0 &&
+                       ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  // force: 0 = choose, 1 = generic, 2 = skinny, 3 = tiled 128x128, 4 = tiled 128x256
+  if (force == 1 || !aligned) {
+    TW_REQUIRE(force <= 1);
+    gemm_generic_kernel<T, OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(A, lda, W, ldw, bias, residual,
+                                                                               ldr, C, ldc, M, N, K);
+    return TW_LAUNCH_RESULT();
+  }
+  if (force == 2 || (force == 0 && M <= 64)) {
+    TW_REQUIRE(M <= 64);
+    if (M <= 16) return launch_skinny<T, OutT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    if (M <= 32) return launch_skinny<T, OutT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    if (M <= 48) return launch_skinny<T, OutT, 3>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny<T, OutT, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  }
+  if (force == 4 || (force == 0 && M > 1024 && N >= 4096))
+    return launch_tiled<T, OutT, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+  return launch_tiled<T, OutT, 2, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+}
+
+// C = A W^T (+bias) (+residual). out_f32 != 0: C is float32 whatever the input
+// type (residual stream, logits); else C has the input type. `residual` may be
+// C itself. `partial` is scratch for split-K (tw_linear_workspace_bytes).
+extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const void* W, long ldw,
+                         const float* bias, const float* residual, long ldr, void* C, long ldc,
+                         float* partial, long partial_bytes, int M, int N, int K, int force,
+                         hipStream_t stream) {
+  TW_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K && ldw >= K && ldc >= N);
+  TW_REQUIRE(residual == nullptr || (ldr >= N && out_f32));
+  if (M == 0) return 0;
+  if (dtype == TW_DTYPE_F32)
+    return linear_dispatch<float, float>((const float*)A, lda, (const float*)W, ldw, bias, residual, ldr,
+                                         (float*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
+  if (dtype == TW_DTYPE_BF16) {
+    if (out_f32)
+      return linear_dispatch<bf16_t, float>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, residual, ldr,
+                                            (float*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
+    return linear_dispatch<bf16_t, bf16_t>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, residual, ldr,
+                                           (bf16_t*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
+  }
+  return TW_ERR_BAD_ARGUMENT;
+}

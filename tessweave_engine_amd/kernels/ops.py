@@ -1,0 +1,245 @@
+"""Checked Python entry points of the HIP kernels.
+
+Every function checks on the host that operand shapes, types and strides are
+what its kernel and grid assume, then launches on torch's current stream.
+Tensors are torch CUDA tensors used as plain device memory; nothing here falls
+back to a library routine.
+"""
+from __future__ import annotations
+
+import torch
+
+from .lib import library, check
+
+F32, BF16 = 0, 1
+_DTYPE_ID = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond, text):
+    if not cond:
+        raise ValueError(text)
+
+
+def _dev(t, dtype=None, name="tensor"):
+    _need(isinstance(t, torch.Tensor) and t.is_cuda, f"{name} must be a CUDA tensor")
+    if dtype is not None:
+        _need(t.dtype == dtype, f"{name} must be {dtype}, is {t.dtype}")
+    return t.data_ptr()
+
+
+def _rows(t, name):
+    """(rows, cols, leading dimension) of a 2-D tensor whose rows are contiguous."""
+    _need(t.dim() == 2 and (t.shape[1] == 1 or t.stride(1) == 1), f"{name} must be 2-D with contiguous rows")
+    ld = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    _need(ld >= t.shape[1], f"{name} has overlapping rows")
+    return t.shape[0], t.shape[1], ld
+
+
+def dtype_id(dtype):
+    _need(dtype in _DTYPE_ID, f"unsupported dtype {dtype}; float32 and bfloat16 are built")
+    return _DTYPE_ID[dtype]
+
+
+def embed_gather(ids, table, out):
+    """out[n, :] = float32(table[ids[n], :])."""
+    n = ids.numel()
+    vocab, hidden = table.shape
+    _need(table.is_contiguous() and out.is_contiguous(), "embedding operands must be contiguous")
+    _need(tuple(out.shape) == (n, hidden), "embedding output has the wrong shape")
+    check(library().tw_embed_gather(dtype_id(table.dtype), _dev(ids, torch.int32, "ids"), _dev(table),
+                                    _dev(out, torch.float32, "out"), n, hidden, vocab, _stream()),
+          "embed_gather")
+    return out
+
+
+def rmsnorm(x, weight, eps, out, rows=None, add=None):
+    """out = x * rsqrt(mean(x^2) + eps) * weight per row; x float32, weight float32.
+
+    rows: int32 indices choosing the input row of each output row.
+    add: float32 [splits, n, hidden] partial sums first added into x (x is updated).
+    """
+    _need(x.dim() == 2 and x.is_contiguous(), "rmsnorm input must be contiguous [n, hidden]")
+    n, hidden = x.shape
+    n_out = rows.numel() if rows is not None else n
+    _need(out.is_contiguous() and tuple(out.shape) == (n_out, hidden), "rmsnorm output has the wrong shape")
+    _need(weight.numel() == hidden, "rmsnorm weight has the wrong size")
+    add_ptr, splits, stride = None, 0, 0
+    if add is not None:
+        _need(rows is None, "rmsnorm cannot gather rows and add partial sums at once")
+        _need(add.dim() == 3 and add.is_contiguous() and tuple(add.shape[1:]) == (n, hidden),
+              "rmsnorm partial sums must be [splits, n, hidden]")
+        add_ptr, splits, stride = _dev(add, torch.float32, "add"), add.shape[0], n * hidden
+    check(library().tw_rmsnorm(dtype_id(out.dtype), _dev(x, torch.float32, "x"),
+                               _dev(weight, torch.float32, "weight"), _dev(out),
+                               _dev(rows, torch.int32, "rows") if rows is not None else None,
+                               n_out, hidden, float(eps), add_ptr, splits, stride, _stream()), "rmsnorm")
+    return out
+
+
+def rope_table(positions, inv_freq, cos, sin):
+    """cos/sin[n, j] of float32(positions[n]) * inv_freq[j]."""
+    n, half = positions.numel(), inv_freq.numel()
+    _need(cos.is_contiguous() and sin.is_contiguous() and tuple(cos.shape) == (n, half)
+          and tuple(sin.shape) == (n, half), "rotary tables must be [n, rot/2]")
+    check(library().tw_rope_table(_dev(positions, torch.int32, "positions"),
+                                  _dev(inv_freq, torch.float32, "inv_freq"),
+                                  _dev(cos, torch.float32, "cos"), _dev(sin, torch.float32, "sin"),
+                                  n, half, _stream()), "rope_table")
+
+
+def rope_kv_write(qkv, cos, sin, slots, keys, values, q_heads, kv_heads, head_dim, page_size,
+                  write_cache=True):
+    """Rotate q (in place) and k of qkv[n] = [q | k | v]; write rotated k and v to the pages.
+
+    keys [pages, kv_heads, page_size, head_dim]; values hold the same number of
+    elements and are written as [pages, kv_heads, head_dim, page_size].
+    """
+    n, width, ld = _rows(qkv, "qkv")
+    _need(width == (q_heads + 2 * kv_heads) * head_dim, "qkv width does not match the head counts")
+    half = cos.shape[1] if cos is not None else 0
+    rot = 2 * half
+    _need(rot <= head_dim, "rotary dimension exceeds head_dim")
+    if rot:
+        _need(tuple(cos.shape) == (n, half) and tuple(sin.shape) == (n, half) and cos.is_contiguous()
+              and sin.is_contiguous(), "rotary tables must be [n, rot/2]")
+    if write_cache:
+        _need(keys.dtype == qkv.dtype and values.dtype == qkv.dtype, "cache and qkv types differ")
+        _need(keys.is_contiguous() and values.is_contiguous(), "cache tensors must be contiguous")
+        _need(tuple(keys.shape[1:]) == (kv_heads, page_size, head_dim), "keys must be [pages, kv_heads, page_size, head_dim]")
+        _need(values.numel() == keys.numel(), "keys and values differ in size")
+        _need(slots.numel() == n, "one cache slot per token is needed")
+    dummy = qkv
+    check(library().tw_rope_kv_write(
+        dtype_id(qkv.dtype), _dev(qkv), ld,
+        _dev(cos, torch.float32, "cos") if rot else _dev(dummy), _dev(sin, torch.float32, "sin") if rot else _dev(dummy),
+        _dev(slots, torch.int32, "slots") if write_cache else None,
+        _dev(keys) if write_cache else None, _dev(values) if write_cache else None,
+        n, q_heads, kv_heads, head_dim, rot, page_size, 1 if write_cache else 0, _stream()), "rope_kv_write")
+
+
+def silu_mul(gate_up, out):
+    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, inter + i]."""
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gate_up must be contiguous [n, 2*inter]")
+    n, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    _need(out.is_contiguous() and tuple(out.shape) == (n, inter) and out.dtype == gate_up.dtype,
+          "silu_mul output has the wrong shape or type")
+    check(library().tw_silu_mul(dtype_id(gate_up.dtype), _dev(gate_up), _dev(out), n, inter, _stream()), "silu_mul")
+    return out
+
+
+def linear_workspace_bytes(dtype, max_rows, n, k):
+    return int(library().tw_linear_workspace_bytes(dtype_id(dtype), int(max_rows), int(n), int(k)))
+
+
+GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE = 0, 1, 2, 3, 4
+
+
+def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_AUTO):
+    """out = x @ weight.T (+ bias) (+ residual).
+
+    x [m, k] and weight [n, k] share a type (float32 or bfloat16); out is float32
+    (required with a residual; the residual may be `out` itself) or that type.
+    bias is float32 [n]; workspace is a float32/byte scratch tensor for split-K.
+    """
+    m, k, lda = _rows(x, "x")
+    n, k2, ldw = _rows(weight, "weight")
+    mo, no, ldc = _rows(out, "out")
+    _need(k == k2 and mo == m and no == n, f"linear shapes do not agree: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    _need(x.dtype == weight.dtype, "x and weight types differ")
+    out_f32 = out.dtype == torch.float32
+    _need(out_f32 or out.dtype == x.dtype, "out must be float32 or the input type")
+    ldr = 0
+    if residual is not None:
+        _need(out_f32, "a residual needs a float32 output")
+        mr, nr, ldr = _rows(residual, "residual")
+        _need((mr, nr) == (m, n), "residual shape differs from the output")
+    if bias is not None:
+        _need(bias.numel() == n and bias.is_contiguous(), "bias has the wrong size")
+    ws_ptr, ws_bytes = None, 0
+    if workspace is not None:
+        ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
+    check(library().tw_linear(dtype_id(x.dtype), 1 if out_f32 else 0, _dev(x), lda, _dev(weight), ldw,
+                              _dev(bias, torch.float32, "bias") if bias is not None else None,
+                              _dev(residual, torch.float32, "residual") if residual is not None else None, ldr,
+                              _dev(out), ldc, ws_ptr, ws_bytes, m, n, k, int(force), _stream()), "linear")
+    return out
+
+
+def attn_decode_splits(n_seqs, q_heads, kv_heads, max_kv_len):
+    return int(library().tw_attn_decode_splits(n_seqs, q_heads, kv_heads, max_kv_len))
+
+
+def attn_decode_workspace_floats(n_seqs, q_heads, head_dim, splits):
+    return int(library().tw_attn_decode_workspace_floats(n_seqs, q_heads, head_dim, splits))
+
+
+def _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim):
+    nq, wq, ldq = _rows(q, "q")
+    no, wo, ldo = _rows(out, "out")
+    _need(wq >= q_heads * head_dim and wo == q_heads * head_dim and no == nq, "attention q/out shapes do not agree")
+    _need(out.dtype == q.dtype == keys.dtype == values.dtype, "attention operand types differ")
+    _need(keys.dim() == 4 and keys.is_contiguous() and values.is_contiguous() and values.numel() == keys.numel(),
+          "keys must be contiguous [pages, kv_heads, page_size, head_dim] and values the same size")
+    _need(keys.shape[1] == kv_heads and keys.shape[3] == head_dim, "cache shape does not match the head sizes")
+    _need(head_dim % 16 == 0 and 16 <= head_dim <= 256, "head_dim must be a multiple of 16 between 16 and 256")
+    _need(keys.shape[2] % 4 == 0, "page_size must be a multiple of 4")
+    _need(q_heads % kv_heads == 0, "q_heads must be a multiple of kv_heads")
+    _need(block_table.dim() == 2 and block_table.stride(1) == 1, "block_table must be 2-D")
+    _need(q_start.numel() >= kv_len.numel() + 1, "q_start needs one more entry than kv_len")
+    return ldq, ldo
+
+
+def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out, q_heads, kv_heads,
+                head_dim, scale, window=0, splits=1, workspace=None):
+    """Attention of sequences seq0..seq0+n_seqs-1, each with ONE query token, over their pages."""
+    ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
+    _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
+    ws_ptr, ws_floats = None, 0
+    if splits > 1:
+        _need(workspace is not None and workspace.dtype == torch.float32, "split decode attention needs a float32 workspace")
+        ws_ptr, ws_floats = _dev(workspace), workspace.numel()
+    check(library().tw_attn_decode(dtype_id(q.dtype), _dev(q), ldq, _dev(keys), _dev(values),
+                                   _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
+                                   _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
+                                   seq0, n_seqs, _dev(out), ldo, ws_ptr, ws_floats, q_heads, kv_heads, head_dim,
+                                   keys.shape[2], int(window or 0), float(scale), int(splits), _stream()),
+          "attn_decode")
+    return out
+
+
+def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_q_len, out, q_heads,
+                 kv_heads, head_dim, scale, window=0):
+    """Attention of sequences seq0..seq0+n_seqs-1 with up to max_q_len query tokens each."""
+    ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
+    _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
+    check(library().tw_attn_prefill(dtype_id(q.dtype), _dev(q), ldq, _dev(keys), _dev(values),
+                                    _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
+                                    _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
+                                    seq0, n_seqs, int(max_q_len), _dev(out), ldo, q_heads, kv_heads, head_dim,
+                                    keys.shape[2], int(window or 0), float(scale), _stream()), "attn_prefill")
+    return out
+
+
+def sampling_uniform(seed, counter):
+    """The uniform number the sampler draws for (seed, counter); host-side, for tests."""
+    return float(library().tw_sampling_uniform(int(seed) & (2 ** 64 - 1), int(counter)))
+
+
+def sample_rows(logits, out, temperature=None, seeds=None, counters=None):
+    """out[r] = greedy (temperature 0 or None) or sampled token of logits[r]."""
+    rows, vocab, ld = _rows(logits, "logits")
+    _need(out.numel() == rows, "one output id per row is needed")
+    if temperature is not None:
+        _need(temperature.numel() == rows and seeds.numel() == rows and counters.numel() == rows,
+              "one temperature, seed and counter per row are needed")
+        _need(seeds.dtype == torch.int64, "seeds must be int64")
+    check(library().tw_sample_rows(_dev(logits, torch.float32, "logits"), ld, rows, vocab,
+                                   _dev(temperature, torch.float32, "temperature") if temperature is not None else None,
+                                   _dev(seeds) if temperature is not None else None,
+                                   _dev(counters, torch.int32, "counters") if temperature is not None else None,
+                                   _dev(out, torch.int32, "out"), _stream()), "sample_rows")
+    return out

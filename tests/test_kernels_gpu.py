@@ -1,0 +1,356 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+import plain_model as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, fp32=(2e-5, 2e-5), bf16=(2e-2, 2e-2)):
+    return dict(zip(("atol", "rtol"), fp32 if dtype == torch.float32 else bf16))
+
+
+@pytest.fixture(scope="module")
+def ops(device):
+    from tessweave_engine_amd.kernels import ops
+    return ops
+
+
+def rand(shape, dtype, device, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(device)
+
+
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_gather(ops, device, dtype):
+    table = rand((389, 72), dtype, device)
+    ids = torch.tensor([0, 388, 5, 5, 17], dtype=torch.int32, device=device)
+    out = torch.empty(5, 72, dtype=torch.float32, device=device)
+    ops.embed_gather(ids, table, out)
+    torch.testing.assert_close(out, table.float()[ids.long()], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,eps", [(64, 1e-6), (200, 1e-5), (3000, 1e-2)])
+def test_rmsnorm(ops, device, dtype, hidden, eps):
+    x = rand((7, hidden), torch.float32, device, 3.0)
+    w = (1 + rand((hidden,), torch.float32, device, 0.1, seed=1))
+    out = torch.empty(7, hidden, dtype=dtype, device=device)
+    ops.rmsnorm(x, w, eps, out)
+    want = plain.rms_norm(x.cpu().double(), w.cpu().double(), eps).float()
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype, (3e-6, 3e-6), (1e-2, 1e-2)))
+    # gathered rows
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=device)
+    out2 = torch.empty(3, hidden, dtype=dtype, device=device)
+    ops.rmsnorm(x, w, eps, out2, rows=rows)
+    torch.testing.assert_close(out2, out[rows.long()], atol=0, rtol=0)
+    # partial sums folded into x first
+    add = rand((3, 7, hidden), torch.float32, device, 1.0, seed=2)
+    x2 = x.clone()
+    out3 = torch.empty(7, hidden, dtype=dtype, device=device)
+    ops.rmsnorm(x2, w, eps, out3, add=add)
+    total = x.cpu().double() + add.cpu().double().sum(0)
+    torch.testing.assert_close(x2.cpu(), total.float(), atol=1e-5, rtol=1e-6)
+    want3 = plain.rms_norm(total, w.cpu().double(), eps).float()
+    torch.testing.assert_close(out3.float().cpu(), want3, **tol(dtype, (3e-6, 3e-6), (1e-2, 1e-2)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,page,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 8, 1e6), (5, 5, 48, 4, 5e5)])
+def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, page, theta):
+    n, pages = 9, 7
+    width = (q_heads + 2 * kv_heads) * head_dim
+    qkv = rand((n, width), dtype, device)
+    positions = torch.tensor([0, 1, 2, 500, 501, 37, 1023, 3, 4], dtype=torch.int32, device=device)
+    half = head_dim // 2
+    inv = (theta ** (-torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim)).to(device)
+    cos = torch.empty(n, half, device=device)
+    sin = torch.empty(n, half, device=device)
+    ops.rope_table(positions, inv, cos, sin)
+    keys = torch.full((pages, kv_heads, page, head_dim), float("nan"), dtype=dtype, device=device)
+    values = torch.full_like(keys, float("nan"))
+    slots = torch.tensor([5 * page + 1, 0, 3 * page + page - 1, -1, 2 * page, 2 * page + 1, 6 * page + 2, 1, 2],
+                         dtype=torch.int32, device=device)
+    before = qkv.clone()
+    ops.rope_kv_write(qkv, cos, sin, slots, keys, values, q_heads, kv_heads, head_dim, page)
+    src = before.float().cpu()
+    pos = positions.cpu()
+    q_want = plain.rope(src[:, :q_heads * head_dim].reshape(n, q_heads, head_dim), pos, theta)
+    k_want = plain.rope(src[:, q_heads * head_dim:(q_heads + kv_heads) * head_dim].reshape(n, kv_heads, head_dim), pos, theta)
+    v_want = src[:, (q_heads + kv_heads) * head_dim:].reshape(n, kv_heads, head_dim)
+    t = tol(dtype, (2e-6, 2e-6), (1e-2, 1e-2))
+    torch.testing.assert_close(qkv[:, :q_heads * head_dim].float().cpu().reshape(n, q_heads, head_dim), q_want, **t)
+    # v columns of qkv untouched
+    torch.testing.assert_close(qkv[:, (q_heads + kv_heads) * head_dim:], before[:, (q_heads + kv_heads) * head_dim:], atol=0, rtol=0)
+    kc = keys.float().cpu()
+    vc = values.float().cpu().reshape(pages, kv_heads, head_dim, page)      # transposed inside the page
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for i, slot in enumerate(slots.tolist()):
+        if slot < 0:
+            continue
+        p, o = divmod(slot, page)
+        written[slot] = True
+        torch.testing.assert_close(kc[p, :, o, :], k_want[i], **t)
+        torch.testing.assert_close(vc[p, :, :, o], v_want[i], atol=0, rtol=0)
+    # nothing else was written
+    kflat = kc.permute(0, 2, 1, 3).reshape(pages * page, -1)
+    assert torch.isnan(kflat[~written]).all()
+    vflat = vc.permute(0, 3, 1, 2).reshape(pages * page, -1)
+    assert torch.isnan(vflat[~written]).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(ops, device, dtype):
+    gu = rand((5, 2 * 70), dtype, device, 2.0)
+    out = torch.empty(5, 70, dtype=dtype, device=device)
+    ops.silu_mul(gu, out)
+    g, u = gu.float().cpu()[:, :70], gu.float().cpu()[:, 70:]
+    torch.testing.assert_close(out.float().cpu(), torch.nn.functional.silu(g) * u, **tol(dtype, (1e-6, 1e-6), (1e-2, 1e-2)))
+
+
+# ---------------------------------------------------------------------------------------
+LINEAR_SHAPES = [  # m, n, k
+    (1, 16, 64), (3, 389, 320), (8, 1000, 1032), (16, 48, 4096), (17, 130, 192), (33, 64, 8200),
+    (64, 256, 512), (65, 200, 136), (130, 389, 64), (300, 520, 776),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
+def test_linear_all_paths(ops, device, dtype, m, n, k):
+    x = rand((m, k), dtype, device, 1.0, seed=1)
+    w = rand((n, k), dtype, device, 0.05, seed=2)
+    bias = rand((n,), torch.float32, device, 0.5, seed=3)
+    res = rand((m, n), torch.float32, device, 1.0, seed=4)
+    want = x.double().cpu() @ w.double().cpu().T
+    ws_bytes = max(ops.linear_workspace_bytes(dtype, m, n, k), 16)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=device)
+    forces = [ops.GEMM_AUTO, ops.GEMM_GENERIC, ops.GEMM_TILED, ops.GEMM_TILED_WIDE]
+    if m <= 64:
+        forces.append(ops.GEMM_SKINNY)
+    scale = math.sqrt(k) * 0.05
+    t = dict(atol=2e-5 * scale, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2 * scale, rtol=2e-2)
+    for force in forces:
+        # plain output in the input type
+        out = torch.full((m, n), float("nan"), dtype=dtype, device=device)
+        ops.linear(x, w, out, workspace=ws, force=force)
+        torch.testing.assert_close(out.double().cpu(), want, **t)
+        # bias + residual into a float32 output that is also the residual
+        acc = res.clone()
+        ops.linear(x, w, acc, bias=bias, residual=acc, workspace=ws, force=force)
+        torch.testing.assert_close(acc.double().cpu(), want + bias.double().cpu() + res.double().cpu(),
+                                   atol=t["atol"] if dtype == torch.float32 else 2e-5 * scale + 1e-5, rtol=1e-5)
+        # without workspace (no split-K)
+        out2 = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+        ops.linear(x, w, out2, bias=bias, force=force)
+        torch.testing.assert_close(out2.double().cpu(), want + bias.double().cpu(),
+                                   atol=t["atol"] if dtype == torch.float32 else 2e-5 * scale + 1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_odd_k_uses_generic(ops, device, dtype):
+    m, n, k = 5, 37, 101
+    x, w = rand((m, k), dtype, device, seed=1), rand((n, k), dtype, device, 0.1, seed=2)
+    out = torch.empty(m, n, dtype=torch.float32, device=device)
+    ops.linear(x, w, out)
+    torch.testing.assert_close(out.double().cpu(), x.double().cpu() @ w.double().cpu().T, atol=1e-4, rtol=1e-5)
+
+
+def test_linear_strided_input_view(ops, device):
+    # the activation may be a column slice of a wider buffer
+    buf = rand((20, 256), torch.bfloat16, device, seed=5)
+    x = buf[:, 64:192]
+    w = rand((48, 128), torch.bfloat16, device, 0.1, seed=6)
+    out = torch.empty(20, 48, dtype=torch.float32, device=device)
+    ops.linear(x, w, out)
+    torch.testing.assert_close(out.double().cpu(), x.double().cpu() @ w.double().cpu().T, atol=1e-4, rtol=1e-5)
+
+
+# ---------------------------------------------------------------------------------------
+def build_paged(k, v, lengths, page, pages_total, device, dtype, seed=0, poison=True):
+    """Scatter per-sequence k, v [len, Hk, D] into shuffled pages; returns keys, values, table."""
+    hk, d = k[0].shape[1], k[0].shape[2]
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(pages_total, generator=g).tolist()
+    fill = float("nan") if poison else 0.0
+    keys = torch.full((pages_total, hk, page, d), fill, dtype=torch.float32)
+    values = torch.full((pages_total, hk, d, page), fill, dtype=torch.float32)
+    width = max(math.ceil(n / page) for n in lengths) + 1
+    table = torch.full((len(lengths), width), -1, dtype=torch.int32)
+    used = 0
+    for s, n in enumerate(lengths):
+        for b in range(math.ceil(n / page)):
+            pg = perm[used]
+            used += 1
+            table[s, b] = pg
+            lo, hi = b * page, min(n, (b + 1) * page)
+            keys[pg, :, :hi - lo, :] = k[s][lo:hi].permute(1, 0, 2)
+            values[pg, :, :, :hi - lo] = v[s][lo:hi].permute(1, 2, 0)
+    return keys.to(dtype).to(device), values.to(dtype).to(device).reshape(pages_total, hk, page, d), table.to(device)
+
+
+ATTN_TOL = {torch.float32: dict(atol=3e-5, rtol=3e-5), torch.bfloat16: dict(atol=.025, rtol=.025)}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("head_dim", [16, 32, 48, 64, 80, 128, 256])
+@pytest.mark.parametrize("heads,kv_heads", [(8, 8), (8, 2), (8, 1), (28, 4), (40, 2)])
+def test_attn_decode_matrix(ops, device, dtype, head_dim, heads, kv_heads):
+    """The reference's kernel gate (tools/validate_cuda.py:25-52): ragged lengths, shuffled pages."""
+    if head_dim in (48, 80) and (heads, kv_heads) not in ((8, 2), (28, 4)):
+        pytest.skip("odd head sizes are run on two head layouts")
+    lengths, page = [1, 17, 65, 257], 16
+    torch.manual_seed(20261008)
+    k = [torch.randn(n, kv_heads, head_dim).to(dtype).float() for n in lengths]
+    v = [torch.randn(n, kv_heads, head_dim).to(dtype).float() for n in lengths]
+    q = torch.randn(len(lengths), heads, head_dim).to(dtype)
+    keys, values, table = build_paged(k, v, lengths, page, 80, device, dtype)
+    want = torch.stack([plain.attention(q[i:i + 1].float(), k[i], v[i], torch.tensor([lengths[i] - 1]))[0]
+                        for i in range(len(lengths))])
+    qd = q.reshape(len(lengths), heads * head_dim).to(device)
+    q_start = torch.arange(len(lengths) + 1, dtype=torch.int32, device=device)
+    kv_len = torch.tensor(lengths, dtype=torch.int32, device=device)
+    for splits in (1, 2, 5):
+        out = torch.full((len(lengths), heads * head_dim), float("nan"), dtype=dtype, device=device)
+        ws = torch.empty(max(1, ops.attn_decode_workspace_floats(len(lengths), heads, head_dim, splits)), device=device)
+        ops.attn_decode(qd, keys, values, table, q_start, kv_len, 0, len(lengths), out, heads, kv_heads,
+                        head_dim, head_dim ** -0.5, splits=splits, workspace=ws)
+        torch.testing.assert_close(out.float().cpu().reshape(len(lengths), heads, head_dim), want, **ATTN_TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_reference_vector_tables(ops, device, dtype):
+    """tests/test_engine.py:288-307 of the reference: tables [[3,1,6],[4,7]], lengths [37,19], 8 q heads on 2."""
+    torch.manual_seed(5)
+    dim, page = 64, 16
+    q = torch.randn(2, 8, dim).to(dtype)
+    kpool = torch.randn(8, page, 2, dim).to(dtype)       # the reference's [pages, page, kv, d] layout
+    vpool = torch.randn(8, page, 2, dim).to(dtype)
+    tables, lengths = [[3, 1, 6], [4, 7]], [37, 19]
+    want = []
+    for i in range(2):
+        kk = kpool[tables[i]].flatten(0, 1)[:lengths[i]].float()
+        vv = vpool[tables[i]].flatten(0, 1)[:lengths[i]].float()
+        want.append(plain.attention(q[i:i + 1].float(), kk, vv, torch.tensor([lengths[i] - 1]))[0])
+    keys = kpool.permute(0, 2, 1, 3).contiguous().to(device)              # [pages, kv, page, d]
+    values = vpool.permute(0, 2, 3, 1).contiguous().to(device).reshape(8, 2, page, dim)   # stored [pages, kv, d, page]
+    table = torch.tensor([[3, 1, 6], [4, 7, -1]], dtype=torch.int32, device=device)
+    out = torch.empty(2, 8 * dim, dtype=dtype, device=device)
+    ops.attn_decode(q.reshape(2, -1).to(device), keys, values, table,
+                    torch.tensor([0, 1, 2], dtype=torch.int32, device=device),
+                    torch.tensor(lengths, dtype=torch.int32, device=device), 0, 2, out, 8, 2, dim, dim ** -0.5)
+    torch.testing.assert_close(out.float().cpu().reshape(2, 8, dim), torch.stack(want),
+                               atol=.015 if dtype == torch.bfloat16 else 3e-5, rtol=.02 if dtype == torch.bfloat16 else 3e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page", [(4, 2, 16, 16), (6, 1, 32, 8), (28, 4, 128, 16), (5, 5, 48, 4)])
+@pytest.mark.parametrize("window", [0, 9])
+def test_attn_prefill_portions(ops, device, dtype, heads, kv_heads, head_dim, page, window):
+    """Portions of prompts at any offset: the query rows are the LAST q_len positions of kv_len keys."""
+    cases = [(5, 5), (17, 3), (33, 33), (70, 2), (130, 64), (40, 1)]       # (kv_len, q_len)
+    torch.manual_seed(11)
+    lengths = [c[0] for c in cases]
+    k = [torch.randn(n, kv_heads, head_dim).to(dtype).float() for n in lengths]
+    v = [torch.randn(n, kv_heads, head_dim).to(dtype).float() for n in lengths]
+    keys, values, table = build_paged(k, v, lengths, page, 64 * 16 // page, device, dtype, seed=3)
+    total_q = sum(c[1] for c in cases)
+    q = torch.randn(total_q, heads, head_dim).to(dtype)
+    q_start, want, row = [0], [], 0
+    for (n, ql), kk, vv in zip(cases, k, v):
+        pos = torch.arange(n - ql, n)
+        want.append(plain.attention(q[row:row + ql].float(), kk, vv, pos, window=window or None))
+        row += ql
+        q_start.append(row)
+    want = torch.cat(want)
+    # q lives inside a wider qkv buffer
+    buf = torch.zeros(total_q, (heads + 2 * kv_heads) * head_dim, dtype=dtype, device=device)
+    buf[:, :heads * head_dim] = q.reshape(total_q, -1).to(device)
+    out = torch.full((total_q, heads * head_dim), float("nan"), dtype=dtype, device=device)
+    ops.attn_prefill(buf, keys, values, table, torch.tensor(q_start, dtype=torch.int32, device=device),
+                     torch.tensor(lengths, dtype=torch.int32, device=device), 0, len(cases), max(c[1] for c in cases),
+                     out, heads, kv_heads, head_dim, head_dim ** -0.5, window=window)
+    torch.testing.assert_close(out.float().cpu().reshape(total_q, heads, head_dim), want, **ATTN_TOL[dtype])
+    # the decode kernel on the one-token sequence must agree with the prefill kernel
+    s = len(cases) - 1
+    out1 = torch.full_like(out, float("nan"))
+    ops.attn_decode(buf, keys, values, table, torch.tensor(q_start, dtype=torch.int32, device=device),
+                    torch.tensor(lengths, dtype=torch.int32, device=device), s, 1, out1, heads, kv_heads, head_dim,
+                    head_dim ** -0.5, window=window)
+    torch.testing.assert_close(out1[q_start[s]].float().cpu().reshape(heads, head_dim), want[q_start[s]], **ATTN_TOL[dtype])
+
+
+def test_attn_far_key_among_hundreds(ops, device):
+    """One far key is made to dominate: a kernel that drops or misplaces it fails by O(1)."""
+    heads, kv_heads, d, page, n = 4, 1, 32, 16, 700
+    torch.manual_seed(3)
+    k = torch.randn(n, kv_heads, d) * 0.1
+    v = torch.randn(n, kv_heads, d)
+    q = torch.randn(1, heads, d) * 0.1
+    far = 37
+    k[far, 0] = q[0, 2] / q[0, 2].norm() * 40.0          # head 2 sees key 37 almost alone
+    q[0, 2] = q[0, 2] / q[0, 2].norm() * 8.0
+    keys, values, table = build_paged([k], [v], [n], page, 64, device, torch.float32, seed=9)
+    want = plain.attention(q, k, v, torch.tensor([n - 1]))
+    assert (want[0, 2] - v[far, 0]).abs().max() < 1e-3
+    for splits in (1, 3):
+        out = torch.empty(1, heads * d, device=device)
+        ws = torch.empty(max(1, ops.attn_decode_workspace_floats(1, heads, d, splits)), device=device)
+        ops.attn_decode(q.reshape(1, -1).to(device), keys, values, table, torch.tensor([0, 1], dtype=torch.int32, device=device),
+                        torch.tensor([n], dtype=torch.int32, device=device), 0, 1, out, heads, kv_heads, d, d ** -0.5,
+                        splits=splits, workspace=ws)
+        torch.testing.assert_close(out.cpu().reshape(1, heads, d), want, atol=3e-5, rtol=3e-5)
+
+
+# ---------------------------------------------------------------------------------------
+def test_sampling_greedy_ties_and_distribution(ops, device):
+    vocab = 389
+    logits = torch.zeros(3, vocab, device=device)
+    logits[0, [5, 200, 388]] = 7.0            # tie: the lowest index wins
+    logits[1, 388] = 1.0
+    logits[2] = -1.0
+    out = torch.empty(3, dtype=torch.int32, device=device)
+    ops.sample_rows(logits, out)
+    assert out.tolist() == [5, 388, 0]
+    # distribution: many seeds on a small vocabulary against softmax(logits / T)
+    torch.manual_seed(0)
+    base = torch.randn(11) * 1.5
+    rows = 20000
+    temp = 0.8
+    lg = base.repeat(rows, 1).to(device)
+    ids = torch.empty(rows, dtype=torch.int32, device=device)
+    ops.sample_rows(lg, ids, temperature=torch.full((rows,), temp, device=device),
+                    seeds=torch.arange(rows, dtype=torch.int64, device=device),
+                    counters=torch.zeros(rows, dtype=torch.int32, device=device))
+    probs = plain.softmax_temperature(base, temp)
+    counts = torch.bincount(ids.long().cpu(), minlength=11).double()
+    chi2 = (((counts - rows * probs.double()) ** 2) / (rows * probs.double())).sum().item()
+    assert chi2 < 40.0, chi2                   # 10 degrees of freedom: P(chi2 > 40) < 2e-5
+    # same (seed, counter) -> same id whatever else is in the batch; other counters differ somewhere
+    ids2 = torch.empty(5, dtype=torch.int32, device=device)
+    ops.sample_rows(lg[:5], ids2, temperature=torch.full((5,), temp, device=device),
+                    seeds=torch.tensor([7, 3, 7, 1, 7], dtype=torch.int64, device=device),
+                    counters=torch.tensor([2, 0, 2, 0, 2], dtype=torch.int32, device=device))
+    assert ids2[0] == ids2[2] == ids2[4]
+    assert ids2[1].item() == ids[3].item() and ids2[3].item() == ids[1].item()
+    # T -> 0+ converges to greedy
+    ids3 = torch.empty(64, dtype=torch.int32, device=device)
+    ops.sample_rows(lg[:64], ids3, temperature=torch.full((64,), 1e-3, device=device),
+                    seeds=torch.arange(64, dtype=torch.int64, device=device),
+                    counters=torch.zeros(64, dtype=torch.int32, device=device))
+    assert (ids3.cpu() == int(base.argmax())).all()
+    # inverse CDF with the generator's own uniform number
+    u = ops.sampling_uniform(12345, 9)
+    cdf = torch.cumsum(probs, 0)
+    want = int((cdf > u * cdf[-1]).nonzero()[0])
+    one = torch.empty(1, dtype=torch.int32, device=device)
+    ops.sample_rows(lg[:1], one, temperature=torch.tensor([temp], device=device),
+                    seeds=torch.tensor([12345], dtype=torch.int64, device=device),
+                    counters=torch.tensor([9], dtype=torch.int32, device=device))
+    assert one.item() == want
