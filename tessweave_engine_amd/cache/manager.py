@@ -13,6 +13,8 @@ from __future__ import annotations
 
 import math
 
+import numpy as np
+
 from .pages import CapacityError, PagePool
 from .spec import CacheLayout
 
@@ -40,8 +42,11 @@ class Sequence:
 
 class CacheManager:
     def __init__(self, layout: CacheLayout, page_size, pages, max_requests, dtype="bfloat16",
-                 device=None, prefix_cache=True):
+                 device=None, prefix_cache=True, max_request_tokens=None):
         """PAGES is one count for every group or a list with one count per group.
+
+        MAX_REQUEST_TOKENS bounds one request's length (default: what the
+        largest pool could hold); it fixes the width of the block tables.
 
         DEVICE None keeps only the host-side accounting (no tensors): the
         allocator, tables and slots can be tested without a GPU.
@@ -56,6 +61,14 @@ class CacheManager:
             raise ValueError("one page count per cache group is needed")
         self.prefix_cache = bool(prefix_cache) and layout.shares_prefixes
         self.pools = [PagePool(n, self.page_size, self.prefix_cache) for n in counts]
+        if max_request_tokens is None:
+            max_request_tokens = max(counts, default=1) * self.page_size
+        self.max_request_tokens = int(max_request_tokens)
+        self.table_width = max(1, math.ceil(self.max_request_tokens / self.page_size))
+        # Block tables as arrays, one row per request slot, kept equal to the
+        # requests' page lists; a step gathers its rows from here.
+        self.table_rows = [np.full((self.max_requests, self.table_width), -1, dtype=np.int32)
+                           for _ in self.pools]
         self.free_state_slots = list(reversed(range(self.max_requests)))
         self.sequences: dict = {}
         self.dtype = dtype
@@ -150,6 +163,7 @@ class CacheManager:
         pool = self.pools[0]
         shared = pool.acquire_prefix(prompt, namespace)
         seq.tables[0] = list(shared)
+        self.table_rows[0][seq.state_slot, :len(shared)] = shared
         seq.computed = seq.cached = len(shared) * self.page_size
         pool.hits += seq.cached
         return seq.cached
@@ -169,6 +183,8 @@ class CacheManager:
         """Hold pages for positions [seq.computed, n_tokens) in every group; all or nothing."""
         if seq.closed:
             raise RuntimeError("request is closed")
+        if n_tokens > self.max_request_tokens:
+            raise ValueError(f"a request may hold at most {self.max_request_tokens} tokens")
         plans = []
         for g, pool in enumerate(self.pools):
             table = seq.tables[g]
@@ -192,6 +208,7 @@ class CacheManager:
             table.extend([-1] * (blocks - len(table)))
             for b, page in zip(missing, pages):
                 table[b] = page
+                self.table_rows[g][seq.state_slot, b] = page
             seq.promised[g] -= from_promise
 
     def advance(self, seq, computed):
@@ -208,6 +225,7 @@ class CacheManager:
                 if table[b] >= 0:
                     pool.release([table[b]])
                     table[b] = -1
+                    self.table_rows[g][seq.state_slot, b] = -1
                     # A reserved request keeps its budget of simultaneous pages:
                     # the page it gave back is promised to it again.
                     if seq.held(g) + seq.promised[g] < seq.budget[g]:
@@ -223,6 +241,7 @@ class CacheManager:
             pool.unpromise(seq.promised[g])
             seq.tables[g] = []
             seq.promised[g] = 0
+            self.table_rows[g][seq.state_slot, :] = -1
         self.free_state_slots.append(seq.state_slot)
         seq.closed = True
         del self.sequences[seq.id]
@@ -257,6 +276,12 @@ class CacheManager:
             promised = sum(seq.promised[g] for seq in self.sequences.values())
             if promised != pool.promised:
                 raise AssertionError(f"group {g}: {pool.promised} pages promised, requests hold promises for {promised}")
+        for seq in self.sequences.values():
+            for g in range(len(self.pools)):
+                row = self.table_rows[g][seq.state_slot]
+                want = seq.tables[g] + [-1] * (self.table_width - len(seq.tables[g]))
+                if row.tolist() != want:
+                    raise AssertionError(f"block table row of request {seq.id!r} differs from its page list")
         slots = [seq.state_slot for seq in self.sequences.values()]
         if len(set(slots)) != len(slots):
             raise AssertionError("two requests share a state slot")

@@ -1,0 +1,264 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+The reference runs two uniform forwards per scheduler turn, a [B,1] decode
+batch and then one [1,T] prompt portion (flow_engine/engine.py:249-260,
+model.py:169), and rebuilds and uploads slot lists per layer
+(model.py:178, cache.py:98,105-107). Here one call takes any mix of prompt
+portions and single decode tokens as ONE flat batch: the metadata of the step
+(token ids, positions, cache slots, block tables, lengths, wanted rows) is
+packed on the host into a single int32 buffer, uploaded once, and every layer
+only reads it. Logits come back in float32 for exactly the rows asked for.
+
+Decode-only steps of a model whose parts are all graph-safe are captured once
+per batch size into a HIP graph and replayed; only the metadata upload differs
+between replays.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+from ..kernels.lib import library, check
+from ..parts.base import GroupStep, StepContext, Workspace
+
+
+@dataclass
+class StepEntry:
+    seq: object                      # cache.Sequence
+    tokens: list                     # the request's next tokens (at least one)
+    want: list = field(default_factory=list)   # indices into tokens whose logits are wanted
+
+
+def _round_up(v, m):
+    return (v + m - 1) // m * m
+
+
+class _Graph:
+    def __init__(self, handle, logits, generation):
+        self.handle, self.logits, self.generation = handle, logits, generation
+
+
+class Stepper:
+    def __init__(self, model, cache, max_step_tokens=256, max_step_seqs=None, use_graphs=True):
+        if model.device is None or model.device.type != "cuda":
+            raise RuntimeError("the model's weights must be on a GPU: there is no CPU path")
+        self.model = model
+        self.cache = cache
+        self.device = model.device
+        self.dtype = model.dtype
+        self.workspace = Workspace(self.device)
+        self.stream = torch.cuda.Stream(device=self.device)
+        self.use_graphs = bool(use_graphs) and model.graph_safe_model
+        self.max_tokens = 0
+        self.max_seqs = 0
+        self._graphs = {}
+        self._warm = set()
+        self._staging = []
+        self._staging_events = []
+        self._staging_next = 0
+        self.steps = 0
+        self.graph_replays = 0
+        self._reserve(max(1, int(max_step_tokens)), int(max_step_seqs or cache.max_requests))
+
+    # ---- metadata buffers ------------------------------------------------------------
+    def _reserve(self, max_tokens, max_seqs):
+        """(Re)allocate the metadata buffers for steps of up to MAX_TOKENS rows and MAX_SEQS requests."""
+        self._drop_graphs()
+        self.max_tokens, self.max_seqs = max_tokens, max_seqs
+        width = self.cache.table_width
+        n_groups = len(self.cache.pools)
+        sections, offset = {}, 0
+
+        def add(name, count):
+            nonlocal offset
+            sections[name] = (offset, count)
+            offset += _round_up(count, 64)
+
+        add("token_ids", max_tokens)
+        add("positions", max_tokens)
+        add("q_start", max_seqs + 1)
+        add("kv_len", max_seqs)
+        add("state_slots", max_seqs)
+        add("logit_rows", max_tokens)
+        for g in range(n_groups):
+            add(f"slots{g}", max_tokens)
+            add(f"table{g}", max_seqs * width)
+        self._sections, self._meta_ints = sections, offset
+        self._meta_dev = torch.zeros(offset, dtype=torch.int32, device=self.device)
+        self._staging = [torch.zeros(offset, dtype=torch.int32, pin_memory=True) for _ in range(4)]
+        self._staging_np = [t.numpy() for t in self._staging]
+        self._staging_events = [None] * 4
+        self._staging_next = 0
+
+    def _dev(self, name, count=None):
+        off, cap = self._sections[name]
+        return self._meta_dev[off:off + (cap if count is None else count)]
+
+    def _drop_graphs(self):
+        if self._graphs:
+            torch.cuda.synchronize(self.device)
+            lib = library()
+            for graph in self._graphs.values():
+                lib.tw_graph_destroy(graph.handle)
+        self._graphs = {}
+        self._warm = set()
+
+    def close(self):
+        self._drop_graphs()
+
+    # ---- the step ----------------------------------------------------------------------
+    def step(self, entries):
+        """Run ENTRIES as one batch; float32 logits [sum(len(e.want)), vocab] in the order of entries and want.
+
+        The returned tensor is scratch memory: read or copy it before the next step.
+        """
+        entries = list(entries)
+        if not entries:
+            return torch.empty(0, self.model.vocab_size, dtype=torch.float32, device=self.device)
+        vocab, seen = self.model.vocab_size, set()
+        for e in entries:
+            if not e.tokens:
+                raise ValueError("a step entry needs at least one token")
+            if id(e.seq) in seen:
+                raise ValueError("a request appears twice in one step")
+            seen.add(id(e.seq))
+            if e.seq.closed:
+                raise ValueError(f"request {e.seq.id!r} is closed")
+            if any(type(t) is not int or t < 0 or t >= vocab for t in e.tokens):
+                raise ValueError(f"request {e.seq.id!r}: token ids must be integers in [0, {vocab})")
+            if any(type(w) is not int or w < 0 or w >= len(e.tokens) for w in e.want):
+                raise ValueError(f"request {e.seq.id!r}: wanted places must index this step's tokens")
+        n_tokens = sum(len(e.tokens) for e in entries)
+        if n_tokens > self.max_tokens or len(entries) > self.max_seqs:
+            self._reserve(max(self.max_tokens, _round_up(n_tokens, 256)), max(self.max_seqs, len(entries)))
+        for e in entries:
+            self.cache.ensure(e.seq, e.seq.computed + len(e.tokens))
+
+        # decode entries (one token) first, then prompt portions; stable
+        order = sorted(range(len(entries)), key=lambda i: len(entries[i].tokens) != 1)
+        ordered = [entries[i] for i in order]
+        n_seqs = len(ordered)
+        q_lens = np.fromiter((len(e.tokens) for e in ordered), dtype=np.int64, count=n_seqs)
+        n_decode = int((q_lens == 1).sum())
+        computed = np.fromiter((e.seq.computed for e in ordered), dtype=np.int64, count=n_seqs)
+        slots_of = np.fromiter((e.seq.state_slot for e in ordered), dtype=np.int64, count=n_seqs)
+        q_start = np.zeros(n_seqs + 1, dtype=np.int64)
+        np.cumsum(q_lens, out=q_start[1:])
+        kv_len = computed + q_lens
+        seq_of_token = np.repeat(np.arange(n_seqs), q_lens)
+        positions = np.arange(n_tokens) - np.repeat(q_start[:-1] - computed, q_lens)
+        if n_decode == n_seqs:
+            token_ids = np.fromiter((e.tokens[0] for e in ordered), dtype=np.int64, count=n_seqs)
+        else:
+            token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in ordered])
+        position_in_order = {orig: pos for pos, orig in enumerate(order)}
+        rows = [int(q_start[position_in_order[i]]) + w for i, e in enumerate(entries) for w in e.want]
+        n_logits = len(rows)
+
+        # pack the metadata into a pinned buffer and upload it once
+        k = self._staging_next
+        self._staging_next = (k + 1) % len(self._staging)
+        if self._staging_events[k] is not None:
+            self._staging_events[k].synchronize()
+        host = self._staging_np[k]
+
+        def put(name, values):
+            off, _ = self._sections[name]
+            host[off:off + len(values)] = values
+
+        put("token_ids", token_ids)
+        put("positions", positions)
+        put("q_start", q_start)
+        put("kv_len", kv_len)
+        put("state_slots", slots_of)
+        put("logit_rows", np.asarray(rows, dtype=np.int64))
+        page = self.cache.page_size
+        width = self.cache.table_width
+        for g in range(len(self.cache.pools)):
+            tables = self.cache.table_rows[g][slots_of]                       # [n_seqs, width]
+            pages = tables[seq_of_token, positions // page]
+            first = self._first_positions(g, computed)
+            live = positions >= np.repeat(first, q_lens)
+            if (pages[live] < 0).any():
+                raise RuntimeError("a token's page is not held; the cache manager and the step disagree")
+            put(f"slots{g}", np.where(pages >= 0, pages * page + positions % page, -1))
+            off, _ = self._sections[f"table{g}"]
+            host[off:off + n_seqs * width] = tables.reshape(-1)
+
+        ctx = StepContext()
+        ctx.device, ctx.dtype = self.device, self.dtype
+        ctx.n_tokens, ctx.n_seqs, ctx.n_decode, ctx.n_logits = n_tokens, n_seqs, n_decode, n_logits
+        ctx.token_ids = self._dev("token_ids", n_tokens)
+        ctx.positions = self._dev("positions", n_tokens)
+        ctx.q_start = self._dev("q_start", n_seqs + 1)
+        ctx.kv_len = self._dev("kv_len", n_seqs)
+        ctx.state_slots = self._dev("state_slots", n_seqs)
+        ctx.logit_rows = self._dev("logit_rows", n_logits)
+        ctx.groups = [GroupStep(self._dev(f"table{g}", n_seqs * width).view(n_seqs, width),
+                                self._dev(f"slots{g}", n_tokens)) for g in range(len(self.cache.pools))]
+        ctx.h_q_start = q_start.tolist()
+        ctx.h_kv_len = kv_len.tolist()
+        ctx.h_state_slots = slots_of.tolist()
+        ctx.max_q_len = int(q_lens[n_decode:].max()) if n_decode < n_seqs else 0
+        ctx.max_kv_len = int(kv_len.max())
+        ctx.kv_capacity = width * page
+        ctx.max_tokens = self.max_tokens
+        ctx.cache, ctx.workspace = self.cache, self.workspace
+
+        graphable = (self.use_graphs and n_decode == n_seqs and n_logits == n_seqs
+                     and rows == list(range(n_seqs)))
+        ctx.capturing = graphable       # fixed launch shapes in warm-up, capture and replay alike
+        caller = torch.cuda.current_stream(self.device)
+        self.stream.wait_stream(caller)
+        with torch.cuda.stream(self.stream):
+            self._meta_dev.copy_(self._staging[k], non_blocking=True)
+            event = torch.cuda.Event()
+            event.record(self.stream)
+            self._staging_events[k] = event
+            if graphable:
+                logits = self._run_graphable(ctx, n_seqs)
+            else:
+                logits = self.model.forward(ctx)
+        caller.wait_stream(self.stream)
+        for e in ordered:
+            self.cache.advance(e.seq, e.seq.computed + len(e.tokens))
+        self.steps += 1
+        return logits
+
+    def _first_positions(self, group, computed):
+        """Per sequence, the first position whose page a windowed group must still hold."""
+        window = self.cache.layout.groups[group].spec.window
+        if window is None:
+            return np.zeros_like(computed)
+        return np.maximum(0, computed - window + 1) // self.cache.page_size * self.cache.page_size
+
+    # ---- HIP graphs for decode-only steps ------------------------------------------------
+    def _run_graphable(self, ctx, n_seqs):
+        graph = self._graphs.get(n_seqs)
+        if graph is not None and graph.generation != self.workspace.generation:
+            self._drop_graphs()
+            graph = None
+        if graph is None:
+            if n_seqs not in self._warm:
+                # First time at this batch size: run eagerly so every scratch buffer exists.
+                self._warm.add(n_seqs)
+                return self.model.forward(ctx)
+            lib = library()
+            generation = self.workspace.generation
+            handle = ctypes.c_void_p()
+            check(lib.tw_graph_begin(self.stream.cuda_stream), "graph capture begin")
+            try:
+                logits = self.model.forward(ctx)
+            finally:
+                code = lib.tw_graph_end(self.stream.cuda_stream, ctypes.byref(handle))
+            check(code, "graph capture end")
+            if self.workspace.generation != generation:
+                lib.tw_graph_destroy(handle)
+                raise RuntimeError("a scratch buffer was allocated during graph capture")
+            graph = self._graphs[n_seqs] = _Graph(handle, logits, generation)
+        check(library().tw_graph_launch(graph.handle, self.stream.cuda_stream), "graph launch")
+        self.graph_replays += 1
+        return graph.logits

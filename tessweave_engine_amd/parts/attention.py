@@ -1,0 +1,80 @@
+"""Grouped-query attention over the paged cache (flow_engine/model.py:36-55,183-201).
+
+q, k, v come from one packed projection (biases optional); q and k are rotated
+by the position part; rotated k and raw v go to this run's cache slot; query
+head h reads kv head h // (q_heads / kv_heads); scores are scaled by
+head_dim^-0.5 unless `scale` says otherwise; the output projection adds into
+the residual stream. Sequences with one token use the split-KV decode kernel,
+the others the prefill kernel; every dense operation runs once over all rows.
+"""
+from __future__ import annotations
+
+from ..cache.spec import CacheNeed, PagedKV
+from ..kernels import ops
+from .base import Mixer
+from .linear import Linear
+
+import torch
+
+
+class GroupedQueryAttention(Mixer):
+    def __init__(self, prefix, hidden, q_heads, kv_heads, head_dim, position, qkv_bias=True,
+                 o_bias=False, window=None, scale=None, packed=True):
+        if q_heads % kv_heads:
+            raise ValueError("q_heads must be a multiple of kv_heads")
+        if head_dim % 16 or not 16 <= head_dim <= 256:
+            raise ValueError("the attention kernels take head sizes in steps of 16 from 16 to 256; "
+                             f"head_dim {head_dim} is refused")
+        self.prefix = prefix
+        self.hidden, self.q_heads, self.kv_heads, self.head_dim = int(hidden), int(q_heads), int(kv_heads), int(head_dim)
+        self.position = position
+        self.window = window
+        self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
+        self.qkv = Linear([prefix + "q_proj", prefix + "k_proj", prefix + "v_proj"], hidden,
+                          [q_heads * head_dim, kv_heads * head_dim, kv_heads * head_dim], bias=qkv_bias, packed=packed)
+        self.o = Linear([prefix + "o_proj"], q_heads * head_dim, [hidden], bias=o_bias)
+
+    def parts(self):
+        return [self.qkv, self.o, self.position]
+
+    def tensor_specs(self):
+        return self.qkv.tensor_specs() + self.o.tensor_specs()
+
+    def bind(self, tensors, dtype, device):
+        self.qkv.bind(tensors, dtype, device)
+        self.o.bind(tensors, dtype, device)
+        self.position.bind(tensors, dtype, device)     # shared by layers; binding again is harmless
+
+    def cache_need(self):
+        return CacheNeed(paged=PagedKV(self.kv_heads, self.head_dim, self.window))
+
+    def forward(self, ctx, run, h, x):
+        n = ctx.n_tokens
+        width = (self.q_heads + 2 * self.kv_heads) * self.head_dim
+        qkv = ctx.scratch("attn.qkv", (n, width))
+        self.qkv.forward(ctx, h, qkv)
+        cos, sin = self.position.tables(ctx)
+        keys, values, g = ctx.cache.keys_values(run.cache_slot)
+        group = ctx.groups[g]
+        ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
+                          self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache)
+        out = ctx.scratch("attn.out", (n, self.q_heads * self.head_dim))
+        window = self.window or 0
+        if ctx.n_decode:
+            # Under graph capture the split count may not depend on this step's lengths.
+            longest = ctx.kv_capacity if ctx.capturing else ctx.max_kv_len
+            if window:
+                longest = min(longest, window)
+            splits = ops.attn_decode_splits(ctx.n_decode, self.q_heads, self.kv_heads, longest)
+            ws = None
+            if splits > 1:
+                floats = ops.attn_decode_workspace_floats(ctx.n_decode, self.q_heads, self.head_dim, splits)
+                ws = ctx.workspace.get("attn.split", (floats,), torch.float32)
+            ops.attn_decode(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode, out,
+                            self.q_heads, self.kv_heads, self.head_dim, self.scale, window=window,
+                            splits=splits, workspace=ws)
+        if ctx.n_seqs > ctx.n_decode:
+            ops.attn_prefill(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode,
+                             ctx.n_seqs - ctx.n_decode, ctx.max_q_len, out, self.q_heads, self.kv_heads,
+                             self.head_dim, self.scale, window=window)
+        self.o.forward(ctx, out, x, residual=x)

@@ -1,0 +1,161 @@
+"""Interfaces of the parts a model is assembled from, and what a part sees of a step.
+
+A model is: a token embedding, a list of blocks, a SCHEDULE (the order in which
+blocks run: data, not code), a final norm and a head. A block arranges a mixer
+(attention here), a feed-forward and norms. Each part gets its sizes and
+constants as constructor parameters and never learns which model it is in.
+
+The reference has none of this: its layers are fixed attributes of one class
+(flow_engine/model.py:88-102) and its forward is one loop (model.py:176-204).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+import math
+
+import torch
+
+
+@dataclass(frozen=True)
+class LayerRun:
+    """One entry of a model's schedule.
+
+    block:        index into the model's blocks (an index may appear more than once)
+    cache_slot:   which cache slot the block's mixer uses in this run
+    writes_cache: False lets the mixer read a slot that another run wrote in this step
+    """
+    block: int
+    cache_slot: int
+    writes_cache: bool = True
+
+
+class Part:
+    """Base of every part: names the checkpoint tensors it owns and takes them over."""
+
+    #: True if `forward` only launches this package's kernels on the current
+    #: stream: no host synchronisation, no allocation once buffers exist. Only
+    #: models whose parts all say so are replayed from HIP graphs.
+    graph_safe = True
+
+    def tensor_specs(self):
+        return []
+
+    def bind(self, tensors, dtype, device):
+        """Take this part's tensors (already on DEVICE, in their device precision) out of TENSORS."""
+
+    def parts(self):
+        """Sub-parts, for walking a model."""
+        return []
+
+
+class Norm(Part):
+    def forward(self, ctx, x, rows=None, add=None):
+        """x float32 [n, hidden] -> normalised rows in the compute type."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Rotary-style encodings hand per-token (cos, sin) tables to the mixers that use them."""
+
+    rotary_dim = 0
+
+    def tables(self, ctx):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self):
+        """A cache.CacheNeed (paged keys/values and/or fixed-size state), or None."""
+        return None
+
+    def forward(self, ctx, run, h, x):
+        """Add the mixer's output for normalised input H into the residual stream X (float32, in place)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, h, x):
+        """Add the feed-forward's output for normalised input H into X (float32, in place)."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, ctx, run, x):
+        raise NotImplementedError
+
+
+class Workspace:
+    """Scratch tensors by tag, allocated once and reused by every step."""
+
+    def __init__(self, device):
+        self.device = device
+        self.buffers = {}
+        self.generation = 0          # changes whenever a buffer is (re)allocated
+
+    def get(self, tag, shape, dtype, capacity=None):
+        """A tensor of SHAPE; the buffer behind it holds CAPACITY rows (default: shape[0])."""
+        shape = tuple(int(v) for v in shape)
+        numel = math.prod(shape)
+        per_row = math.prod(shape[1:]) if shape else 1
+        want = max(numel, per_row * max(capacity or 0, shape[0] if shape else 1), 1)
+        key = (tag, dtype)
+        buf = self.buffers.get(key)
+        if buf is None or buf.numel() < numel:
+            buf = torch.empty(want, dtype=dtype, device=self.device)
+            self.buffers[key] = buf
+            self.generation += 1
+        return buf[:numel].view(shape)
+
+    def bytes(self):
+        return sum(b.numel() * b.element_size() for b in self.buffers.values())
+
+
+class GroupStep:
+    """A cache group's metadata for one step."""
+    __slots__ = ("block_table", "slot_mapping")
+
+    def __init__(self, block_table, slot_mapping):
+        self.block_table = block_table     # int32 [n_seqs, width]; -1 where a block is not held
+        self.slot_mapping = slot_mapping   # int32 [n_tokens]; physical token slot of each new token
+
+
+class StepContext:
+    """Everything a part may read during one step.
+
+    The batch is flat: n_tokens rows, grouped by sequence; sequence s owns rows
+    q_start[s] .. q_start[s+1]-1, at positions kv_len[s]-q_len .. kv_len[s]-1.
+    The first n_decode sequences have exactly one token each.
+    """
+
+    def __init__(self):
+        self.device = None
+        self.dtype = None
+        self.n_tokens = 0
+        self.n_seqs = 0
+        self.n_decode = 0
+        self.token_ids = None        # int32 [n_tokens]
+        self.positions = None        # int32 [n_tokens]
+        self.q_start = None          # int32 [n_seqs + 1]
+        self.kv_len = None           # int32 [n_seqs], this step's tokens included
+        self.state_slots = None      # int32 [n_seqs]
+        self.logit_rows = None       # int32 [n_logits]
+        self.n_logits = 0
+        self.groups = []             # GroupStep per cache group
+        # host copies, for grid sizes and for parts written in plain torch
+        self.h_q_start = []
+        self.h_kv_len = []
+        self.h_state_slots = []
+        self.max_q_len = 0           # over the sequences after the first n_decode
+        self.max_kv_len = 0
+        self.kv_capacity = 0         # most keys a sequence can ever hold (block-table width * page size)
+        self.capturing = False       # launches must not depend on this step's lengths
+        self.max_tokens = 0          # row capacity of per-token scratch buffers
+        self.cache = None            # cache.CacheManager
+        self.workspace = None        # Workspace
+        self.shared = {}             # per-step values shared by layers (rotary tables, ...)
+
+    def scratch(self, tag, shape, dtype=None):
+        """Per-token scratch [n, ...]: the buffer is sized once for the largest step."""
+        return self.workspace.get(tag, tuple(shape), dtype or self.dtype, capacity=self.max_tokens)

@@ -1,0 +1,73 @@
+"""A linear layer over one or several checkpoint matrices with the same input.
+
+Several matrices are packed by exact row concatenation into one weight, as the
+reference packs q,k,v and gate,up (flow_engine/model.py:58-65): 7 matrix
+products per layer become 4. `packed=False` keeps them apart (the reference's
+`--unfused` ablation, cli.py:73); each then writes its own column range.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.spec import MATRIX, VECTOR, NORMAL, TensorSpec
+from .base import Part
+
+
+class Linear(Part):
+    def __init__(self, names, in_features, out_features, bias=False, packed=True):
+        """names[i] is the checkpoint prefix of the i-th matrix ("...q_proj"), out_features[i] its rows."""
+        self.names = list(names)
+        self.in_features = int(in_features)
+        self.out_features = [int(o) for o in out_features]
+        self.has_bias = bool(bias)
+        self.packed = bool(packed)
+        self.weights = []       # one tensor if packed, else one per name
+        self.biases = []
+        self._ws_floats = {}
+
+    @property
+    def total_out(self):
+        return sum(self.out_features)
+
+    def tensor_specs(self):
+        specs = []
+        for name, rows in zip(self.names, self.out_features):
+            specs.append(TensorSpec(name + ".weight", (rows, self.in_features), MATRIX, NORMAL))
+            if self.has_bias:
+                specs.append(TensorSpec(name + ".bias", (rows,), VECTOR, NORMAL))
+        return specs
+
+    def bind(self, tensors, dtype, device):
+        weights = [tensors.pop(name + ".weight") for name in self.names]
+        biases = [tensors.pop(name + ".bias") for name in self.names] if self.has_bias else []
+        if self.packed and len(weights) > 1:
+            self.weights = [torch.cat(weights, 0).contiguous()]
+            self.biases = [torch.cat(biases, 0).contiguous()] if biases else []
+        else:
+            self.weights = [w.contiguous() for w in weights]
+            self.biases = [b.contiguous() for b in biases]
+        del weights, biases
+
+    def weight_bytes(self):
+        return sum(w.numel() * w.element_size() for w in self.weights)
+
+    def forward(self, ctx, x, out, residual=None):
+        """out[:, columns] = x @ W.T (+ bias) (+ residual); out may be float32 or x's type."""
+        col = 0
+        for i, w in enumerate(self.weights):
+            rows = w.shape[0]
+            target = out if len(self.weights) == 1 else out[:, col:col + rows]
+            res = None
+            if residual is not None:
+                res = residual if len(self.weights) == 1 else residual[:, col:col + rows]
+            ws = None
+            if x.shape[0] <= 64:
+                # Split-K scratch, sized once for the largest skinny batch so it never regrows.
+                if i not in self._ws_floats:
+                    self._ws_floats[i] = ops.linear_workspace_bytes(w.dtype, 64, rows, w.shape[1]) // 4
+                if self._ws_floats[i]:
+                    ws = ctx.workspace.get("linear.splitk", (self._ws_floats[i],), torch.float32)
+            ops.linear(x, w, target, bias=self.biases[i] if self.biases else None, residual=res, workspace=ws)
+            col += rows
+        return out

@@ -1,0 +1,30 @@
+"""RMS norm: y = x * rsqrt(mean(x^2) + eps) * weight (flow_engine/model.py:15-23).
+
+The residual stream it reads is float32; statistics and products are float32
+and the result is rounded once to the compute type. The weight is held in
+float32 (exact for a bfloat16 checkpoint).
+"""
+from __future__ import annotations
+
+from ..kernels import ops
+from ..weights.spec import VECTOR, ONE_PLUS_NORMAL, TensorSpec
+from .base import Norm
+
+
+class RMSNorm(Norm):
+    def __init__(self, name, size, eps):
+        self.name = name
+        self.size = int(size)
+        self.eps = float(eps)
+        self.weight = None
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name + ".weight", (self.size,), VECTOR, ONE_PLUS_NORMAL)]
+
+    def bind(self, tensors, dtype, device):
+        self.weight = tensors.pop(self.name + ".weight").contiguous()
+
+    def forward(self, ctx, x, rows=None, add=None, tag="norm.out"):
+        n_out = rows.numel() if rows is not None else x.shape[0]
+        out = ctx.scratch(tag, (n_out, self.size))
+        return ops.rmsnorm(x, self.weight, self.eps, out, rows=rows, add=add)
