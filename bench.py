@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at the Qwen2.5-7B shape on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Default run: the layer sizes of the 7B shape, random weights, bfloat16, a batch
+of 8 requests decoding at a context of 4,096 tokens: each request is given a
+random prompt of 4096 - W - K tokens, then W untimed and K timed decode steps
+run through the scheduler (admission, planning, the step function, greedy
+sampling on the device, commit), so the last timed step reads 4,096 keys per
+request. One JSON line is printed: decoded tokens a second, a 2,048-token
+prefill, the decode step's HBM roofline, and decode at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+QWEN25_7B = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=28, hidden_size=3584,
+    num_attention_heads=28, num_key_value_heads=4, head_dim=128, intermediate_size=18944,
+    vocab_size=152064, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False,
+    use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
+
+HBM_PEAK_GBS = 8000.0
+PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=128)
+    p.add_argument("--warmup", type=int, default=16)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--context", type=int, default=4096)
+    p.add_argument("--layers", type=int, default=0, help="fewer layers than the 7B shape has (0: all 28)")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    p.add_argument("--prefill-tokens", type=int, default=2048)
+    p.add_argument("--points", default="1,64", help="further decode batch sizes to measure")
+    p.add_argument("--no-graphs", action="store_true")
+    p.add_argument("--seed", type=int, default=0)
+    return p.parse_args()
+
+
+def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, seed):
+    """Tokens/s and ms/step of STEPS decode steps at BATCH, ending at CONTEXT keys per request."""
+    from tessweave_engine_amd.config import EngineConfig
+    from tessweave_engine_amd.engine import Engine
+
+    prompt_len = context - steps - warmup
+    assert prompt_len >= 1
+    page = 16
+    blocks = batch * ((context + page - 1) // page + 1)
+    chunk = 2048
+    config = EngineConfig(block_size=page, kv_blocks=blocks, max_context=context + 1, max_active=batch,
+                          max_queue=batch, prefill_chunk=chunk, min_prefill_chunk=16, prefix_cache=False,
+                          dtype=dtype, max_step_tokens=batch + chunk, use_graphs=use_graphs)
+    engine = Engine(model, config)
+    g = torch.Generator().manual_seed(seed)
+    vocab = model.config.vocab_size
+    requests = [engine.submit(torch.randint(0, vocab, (prompt_len,), generator=g).tolist(),
+                              max_tokens=steps + warmup + 1, ignore_eos=True) for _ in range(batch)]
+    # Prompts, untimed: all but the last token of every prompt goes through the step function
+    # directly, so that every request samples its first token in the same step and they decode in lockstep.
+    from tessweave_engine_amd.engine import StepEntry
+    engine._admit()
+    assert len(engine.active) == batch
+    for r in requests:
+        for i in range(0, prompt_len - 1, chunk):
+            engine.stepper.step([StepEntry(r.seq, r.prompt[i:min(prompt_len - 1, i + chunk)], [])])
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert all(len(r.output) == warmup + steps for r in requests), [len(r.output) for r in requests]
+    replays = engine.stepper.graph_replays
+    engine.close()
+    del engine
+    torch.cuda.empty_cache()
+    return batch * steps / elapsed, elapsed / steps * 1000, replays
+
+
+def prefill_run(model, torch, tokens, dtype, seed, repeats=3):
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+
+    page = 16
+    cache = CacheManager(model.cache_layout(), page, tokens // page + 2, 2, dtype=dtype, device=model.device,
+                         prefix_cache=False, max_request_tokens=tokens + page)
+    stepper = Stepper(model, cache, max_step_tokens=tokens, use_graphs=False)
+    g = torch.Generator().manual_seed(seed + 1)
+    ids = torch.randint(0, model.config.vocab_size, (tokens,), generator=g).tolist()
+    best = None
+    for i in range(repeats + 1):
+        seq = cache.open(f"p{i}")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = stepper.step([StepEntry(seq, ids, [tokens - 1])])
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1000
+        assert torch.isfinite(logits).all()
+        cache.close(seq)
+        if i > 0:
+            best = ms if best is None else min(best, ms)
+    stepper.close()
+    return best
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this engine does not run on {args.gpus} GPUs")
+        return 2
+    import torch
+    from tessweave_engine_amd.config import config_from_dict
+    from tessweave_engine_amd.weights import random_model
+
+    cfg = dict(QWEN25_7B)
+    layers_full = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    config = config_from_dict(cfg)
+    model = random_model(config, args.seed, dtype=args.dtype, device="cuda:0")
+    c = config
+    use_graphs = not args.no_graphs
+
+    value, ms_per_step, replays = decode_run(model, torch, args.batch, args.context, args.steps, args.warmup,
+                                             args.dtype, use_graphs, args.seed)
+    element = 2 if args.dtype == "bfloat16" else 4
+    layer_weights = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
+        + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
+    weight_bytes = (c.num_hidden_layers * layer_weights + c.vocab_size * c.hidden_size) * element
+    mean_ctx = args.context - args.steps / 2
+    kv_bytes = args.batch * mean_ctx * c.kv_bytes_per_token(element)
+    achieved = (weight_bytes + kv_bytes) / (ms_per_step / 1000) / 1e9
+
+    t = args.prefill_tokens
+    prefill_ms = prefill_run(model, torch, t, args.dtype, args.seed)
+    linear_flops = 2.0 * t * c.num_hidden_layers * layer_weights + 2.0 * c.vocab_size * c.hidden_size
+    attn_flops = c.num_hidden_layers * 4.0 * c.num_attention_heads * c.head_dim * (t * (t + 1) / 2)
+    prefill_tflops = (linear_flops + attn_flops) / (prefill_ms / 1000) / 1e12
+
+    points = {}
+    for b in [int(v) for v in args.points.split(",") if v]:
+        steps = min(args.steps, 64)
+        tps, _, _ = decode_run(model, torch, b, args.context, steps, 8, args.dtype, use_graphs, args.seed)
+        points[f"decode_b{b}"] = round(tps, 1)
+
+    line = {
+        "metric": "decode tok/s @ batch 8, Qwen2.5-7B shape bf16 (+ prefill tok/s @ 2048, decode @ batch 1/64)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform-random token ids, random weights N(0, 0.02)",
+        "config": {"model": "Qwen2.5-7B shape", "layers": c.num_hidden_layers, "layers_full": layers_full,
+                   "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
+                   "head_dim": c.head_dim, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
+                   "global_batch": args.batch, "seq_len": args.context,
+                   "prompt_len": args.context - args.steps - args.warmup, "page_size": 16,
+                   "parallelism": "single GPU", "hip_graphs": bool(use_graphs and replays > 0),
+                   "sampling": "greedy on device"},
+        "prefill": {"value": round(t / (prefill_ms / 1000), 1), "tokens": t, "ms": round(prefill_ms, 3),
+                    "frac": round(prefill_tflops / PEAK_TFLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

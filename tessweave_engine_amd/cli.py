@@ -1,0 +1,209 @@
+"""Command line and Python entry point, in the manner of the reference's `flow-inference`.
+
+Commands and options keep the reference's names and meanings where it has them
+(flow_engine/cli.py:48-80): `doctor`, `inspect MODEL`, `replay LOG`,
+`generate MODEL --prompt ... --max-tokens N`, and the engine options
+--device --dtype --max-context --kv-blocks --block-size --max-active
+--prefill-chunk --target-step-ms --attention --no-prefix-cache --unfused --log.
+`serve` and the draft options are not built. Added: --prompt-ids/--prompt-file
+(token ids; a tokenizer is only needed for --prompt), --temperature, --seed,
+--ignore-eos, --max-step-tokens, --adaptive-chunk, --no-graphs and
+`random-weights CONFIG_JSON OUT --seed S` which writes a model folder.
+
+Python: `make_engine(args) -> (Engine, tokenizer)` as in the reference
+(cli.py:14-45), or `engine_for(model_folder, **options)` and `Engine.generate`.
+"""
+from __future__ import annotations
+
+import argparse
+from dataclasses import asdict
+import json
+from pathlib import Path
+import platform
+import sys
+
+
+def _engine_options(p):
+    p.add_argument("model", help="local folder with config.json and safetensors weights; nothing is downloaded")
+    p.add_argument("--device", choices=["auto", "cuda"], default="auto", help="only a GPU can run this engine")
+    p.add_argument("--dtype", choices=["auto", "float32", "bfloat16"], default="auto",
+                   help="auto is bfloat16; float32 runs every kernel in true 32-bit")
+    p.add_argument("--max-context", type=int, default=2048, help="prompt + generated tokens per request")
+    p.add_argument("--kv-blocks", type=int, default=256, help="physical cache pages")
+    p.add_argument("--block-size", type=int, default=16, help="tokens per page")
+    p.add_argument("--max-active", type=int, default=4, help="requests admitted at once")
+    p.add_argument("--prefill-chunk", type=int, default=256, help="largest prompt portion in one step")
+    p.add_argument("--target-step-ms", type=float, default=50, help="step time the adaptive portion aims at")
+    p.add_argument("--attention", choices=["hip"], default="hip", help="one backend: the HIP paged kernels")
+    p.add_argument("--no-prefix-cache", action="store_true", help="do not reuse pages of equal prompt prefixes")
+    p.add_argument("--unfused", action="store_true", help="ablation: keep q/k/v and gate/up as separate matrices")
+    p.add_argument("--log", default="runs/engine.jsonl", help="JSONL event log")
+    p.add_argument("--max-step-tokens", type=int, default=0, help="token budget of one step (0: max-active + prefill-chunk)")
+    p.add_argument("--adaptive-chunk", action="store_true", help="size prompt portions by measured step time")
+    p.add_argument("--no-graphs", action="store_true", help="never replay decode steps from HIP graphs")
+
+
+def build_parser():
+    parser = argparse.ArgumentParser(prog="flow-inference",
+                                     description="Qwen2.5 dense inference engine for AMD MI355X")
+    sub = parser.add_subparsers(dest="command", required=True)
+    sub.add_parser("doctor", help="read-only report of the runtime and the accelerator")
+    inspect = sub.add_parser("inspect", help="validate config.json and explain the cache allocation; no weights are read")
+    inspect.add_argument("model")
+    inspect.add_argument("--kv-blocks", type=int, default=256)
+    inspect.add_argument("--block-size", type=int, default=16)
+    replay = sub.add_parser("replay", help="print the scheduler events of a JSONL log (no inference)")
+    replay.add_argument("log")
+    gen = sub.add_parser("generate", help="generate tokens for one prompt")
+    _engine_options(gen)
+    gen.add_argument("--prompt", help="text; needs the model folder's tokenizer with a chat template")
+    gen.add_argument("--prompt-ids", help="comma-separated token ids")
+    gen.add_argument("--prompt-file", help="file with token ids separated by commas or white space")
+    gen.add_argument("--max-tokens", type=int, default=128)
+    gen.add_argument("--temperature", type=float, default=0.0)
+    gen.add_argument("--seed", type=int, default=0)
+    gen.add_argument("--ignore-eos", action="store_true")
+    rnd = sub.add_parser("random-weights", help="write a model folder with seeded random weights")
+    rnd.add_argument("config", help="a config.json (or a folder that holds one)")
+    rnd.add_argument("out", help="folder to write config.json and model.safetensors into")
+    rnd.add_argument("--seed", type=int, default=0)
+    rnd.add_argument("--std", type=float, default=0.02)
+    rnd.add_argument("--store-dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    return parser
+
+
+def resolve_device_dtype(args):
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("no GPU is visible: this engine has no CPU path")
+    dtype = "bfloat16" if args.dtype == "auto" else args.dtype
+    return "cuda:0", dtype
+
+
+def make_engine(args):
+    """(Engine, tokenizer or None) from parsed `generate` options."""
+    from .config import EngineConfig
+    from .engine import Engine, Trace
+    from .weights import load_model
+    import torch
+
+    device, dtype = resolve_device_dtype(args)
+    trace = Trace(args.log)
+    argv = list(sys.argv)
+    for i, argument in enumerate(argv):            # prompts never reach the log
+        if argument in ("--prompt", "--prompt-ids") and i + 1 < len(argv):
+            argv[i + 1] = "[REDACTED]"
+        elif argument.startswith(("--prompt=", "--prompt-ids=")):
+            argv[i] = argument.split("=")[0] + "=[REDACTED]"
+    trace.emit("launch", argv=argv, python=sys.version, torch=torch.__version__, device=device, dtype=dtype)
+    print(f"Loading local weights: {args.model} ({device}, {dtype})", file=sys.stderr, flush=True)
+    folder = Path(args.model).resolve(strict=True)
+    model = load_model(folder, dtype=dtype, device=device, packed=not args.unfused)
+    config = model.config
+    engine_config = EngineConfig(
+        block_size=args.block_size, kv_blocks=args.kv_blocks, max_context=args.max_context,
+        max_active=args.max_active, prefill_chunk=args.prefill_chunk,
+        min_prefill_chunk=min(16, args.prefill_chunk), target_step_ms=args.target_step_ms,
+        prefix_cache=not args.no_prefix_cache, dtype=dtype, max_step_tokens=args.max_step_tokens,
+        adaptive_chunk=args.adaptive_chunk, use_graphs=not args.no_graphs)
+    tokenizer = None
+    if getattr(args, "prompt", None):
+        from transformers import AutoTokenizer          # tokenizer files only; no model code of the library runs
+        tokenizer = AutoTokenizer.from_pretrained(str(folder), local_files_only=True, trust_remote_code=False)
+        if not tokenizer.chat_template:
+            raise ValueError("a tokenizer chat_template is required; no template will be guessed")
+    engine = Engine(model, engine_config, trace)
+    trace.emit("loaded", engine=asdict(engine_config), model=config.describe(), kv_bytes=engine.cache.allocated_bytes)
+    return engine, tokenizer
+
+
+def engine_for(model_folder, **options):
+    """An Engine for MODEL_FOLDER; OPTIONS are `generate`'s long option names with underscores."""
+    argv = ["generate", str(model_folder), "--prompt-ids", "0"]
+    args = build_parser().parse_args(argv)
+    for key, value in options.items():
+        if not hasattr(args, key):
+            raise TypeError(f"unknown engine option {key!r}")
+        setattr(args, key, value)
+    if "log" not in options:
+        args.log = None
+    return make_engine(args)[0]
+
+
+def _prompt_ids(args, tokenizer):
+    given = [v for v in (args.prompt, args.prompt_ids, args.prompt_file) if v]
+    if len(given) != 1:
+        raise SystemExit("give exactly one of --prompt, --prompt-ids, --prompt-file")
+    if args.prompt:
+        return list(tokenizer.apply_chat_template([{"role": "user", "content": args.prompt}], tokenize=True,
+                                                  add_generation_prompt=True))
+    text = args.prompt_ids if args.prompt_ids else Path(args.prompt_file).read_text()
+    return [int(v) for v in text.replace(",", " ").split()]
+
+
+def main(argv=None):
+    parser = build_parser()
+    args = parser.parse_args(argv)
+    if args.command == "doctor":
+        import torch
+        report = {"python": sys.version, "platform": platform.platform(), "torch": torch.__version__,
+                  "hip": getattr(torch.version, "hip", None), "gpu": torch.cuda.is_available()}
+        if torch.cuda.is_available():
+            props = torch.cuda.get_device_properties(0)
+            report.update(device=props.name, arch=getattr(props, "gcnArchName", None),
+                          memory_bytes=props.total_memory, compute_units=props.multi_processor_count)
+        from .kernels import build
+        report["kernel_library"] = str(build.find_library() or "not built yet")
+        print(json.dumps(report, indent=2))
+    elif args.command == "inspect":
+        from .config import build_model, read_model_config
+        if min(args.kv_blocks, args.block_size) < 1:
+            parser.error("positive block count and size are required")
+        c = read_model_config(args.model)
+        layout = build_model(c).cache_layout()
+        tokens = args.kv_blocks * args.block_size
+        print(json.dumps({"architecture": c.describe(),
+                          "kv_formula": "2 * layers * KV_heads * head_dim * bytes_per_element * blocks * block_size",
+                          "kv_bf16_bytes": layout.bytes_per_token(2) * tokens,
+                          "kv_fp32_bytes": layout.bytes_per_token(4) * tokens,
+                          "cache_groups": [{"layers": len(g.slots), "kv_heads": g.spec.kv_heads,
+                                            "head_dim": g.spec.head_dim, "window": g.spec.window}
+                                           for g in layout.groups],
+                          "excludes": ["weights", "activations and scratch buffers", "runtime/allocator"]}, indent=2))
+    elif args.command == "replay":
+        from .engine.trace import read_events
+        for event in read_events(args.log):
+            print(json.dumps(event, ensure_ascii=False))
+    elif args.command == "random-weights":
+        from .config import config_from_dict
+        from .weights import write_model_folder
+        src = Path(args.config)
+        src = src / "config.json" if src.is_dir() else src
+        config = config_from_dict(json.loads(src.read_text()))
+        out = write_model_folder(args.out, config, args.seed, args.std, args.store_dtype)
+        print(str(out))
+    else:
+        engine, tokenizer = make_engine(args)
+        try:
+            ids = _prompt_ids(args, tokenizer)
+            r = engine.submit(ids, args.max_tokens, temperature=args.temperature, seed=args.seed,
+                              ignore_eos=args.ignore_eos)
+            engine.start()
+            while True:
+                event = r.events.get()
+                if event["type"] == "done":
+                    if event["error"]:
+                        raise RuntimeError(event["error"])
+                    break
+            if tokenizer is not None:
+                print(tokenizer.decode(r.output, skip_special_tokens=True))
+            else:
+                print(" ".join(str(t) for t in r.output))
+            print(json.dumps(event), file=sys.stderr)
+        finally:
+            engine.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

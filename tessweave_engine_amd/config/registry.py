@@ -79,10 +79,13 @@ def read_model_config(folder):
     return with_generation_eos(config, folder)
 
 
-def build_model(config):
-    """The architecture's model for CONFIG, assembled from parts, weights not yet bound."""
+def build_model(config, **options):
+    """The architecture's model for CONFIG, assembled from parts, weights not yet bound.
+
+    OPTIONS go to the architecture's builder (e.g. packed=False keeps q/k/v apart).
+    """
     _load_builtin()
     arch = _ARCHITECTURES.get(getattr(config, "architecture", None))
     if arch is None:
         raise ConfigError(f"no registered architecture named {getattr(config, 'architecture', None)!r}")
-    return arch.builder(config)
+    return arch.builder(config, **options)

@@ -109,6 +109,9 @@ class Stepper:
     def close(self):
         self._drop_graphs()
 
+    def synchronize(self):
+        self.stream.synchronize()
+
     # ---- the step ----------------------------------------------------------------------
     def step(self, entries):
         """Run ENTRIES as one batch; float32 logits [sum(len(e.want)), vocab] in the order of entries and want.

@@ -138,13 +138,13 @@ def read_tensors(folder, specs, compute_dtype, device):
     return tensors
 
 
-def load_model(folder, dtype="bfloat16", device="cuda"):
+def load_model(folder, dtype="bfloat16", device="cuda", **build_options):
     """Model of FOLDER (config.json picks the class) with its weights on DEVICE."""
     from ..config import read_model_config, build_model
 
     folder = Path(folder).resolve(strict=True)
     config = read_model_config(folder)
-    model = build_model(config)
+    model = build_model(config, **build_options)
     compute_dtype = resolve_dtype(dtype)
     tensors = read_tensors(folder, model.tensor_specs(), compute_dtype, device)
     model.bind(tensors, compute_dtype, torch.device(device))
