@@ -121,6 +121,38 @@ class Stepper:
         entries = list(entries)
         if not entries:
             return torch.empty(0, self.model.vocab_size, dtype=torch.float32, device=self.device)
+        ctx, ordered, graphable = self.prepare(entries)
+        caller = torch.cuda.current_stream(self.device)
+        self.stream.wait_stream(caller)
+        with torch.cuda.stream(self.stream):
+            self.upload(ctx)
+            if graphable:
+                logits = self._run_graphable(ctx, ctx.n_seqs)
+            else:
+                logits = self.model.forward(ctx)
+        caller.wait_stream(self.stream)
+        self.finish(ordered)
+        return logits
+
+    def finish(self, ordered):
+        """Record in the cache that the step's tokens are now held."""
+        for e in ordered:
+            self.cache.advance(e.seq, e.seq.computed + len(e.tokens))
+        self.steps += 1
+
+    def upload(self, ctx):
+        """Copy the step's packed metadata to the device (on the current stream)."""
+        k = ctx.staging_index
+        self._meta_dev.copy_(self._staging[k], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record(torch.cuda.current_stream(self.device))
+        self._staging_events[k] = event
+
+    def prepare(self, entries):
+        """Check ENTRIES, take their pages, and build the step's context (host side; nothing runs yet).
+
+        Returns (context, entries in batch order, whether the step can be replayed from a graph).
+        """
         vocab, seen = self.model.vocab_size, set()
         for e in entries:
             if not e.tokens:
@@ -214,22 +246,8 @@ class Stepper:
         graphable = (self.use_graphs and n_decode == n_seqs and n_logits == n_seqs
                      and rows == list(range(n_seqs)))
         ctx.capturing = graphable       # fixed launch shapes in warm-up, capture and replay alike
-        caller = torch.cuda.current_stream(self.device)
-        self.stream.wait_stream(caller)
-        with torch.cuda.stream(self.stream):
-            self._meta_dev.copy_(self._staging[k], non_blocking=True)
-            event = torch.cuda.Event()
-            event.record(self.stream)
-            self._staging_events[k] = event
-            if graphable:
-                logits = self._run_graphable(ctx, n_seqs)
-            else:
-                logits = self.model.forward(ctx)
-        caller.wait_stream(self.stream)
-        for e in ordered:
-            self.cache.advance(e.seq, e.seq.computed + len(e.tokens))
-        self.steps += 1
-        return logits
+        ctx.staging_index = k
+        return ctx, ordered, graphable
 
     def _first_positions(self, group, computed):
         """Per sequence, the first position whose page a windowed group must still hold."""

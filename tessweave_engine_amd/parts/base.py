@@ -155,6 +155,7 @@ class StepContext:
         self.cache = None            # cache.CacheManager
         self.workspace = None        # Workspace
         self.shared = {}             # per-step values shared by layers (rotary tables, ...)
+        self.staging_index = 0       # which host staging buffer holds this step's metadata
 
     def scratch(self, tag, shape, dtype=None):
         """Per-token scratch [n, ...]: the buffer is sized once for the largest step."""

@@ -1,0 +1,395 @@
+"""The engine on the GPU: generation through the entry point, long decoding, sampling, prefix reuse,
+each part alone, schedules that name a layer twice or share a cache, and a toy mixer with its own state."""
+import json
+import math
+
+import pytest
+import torch
+
+import plain_model as plain
+from tiny_configs import TINY, make_folder
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def tiny(request, tmp_path_factory, device):
+    name = request.param
+    folder = tmp_path_factory.mktemp(f"eng{name}")
+    cfg, page = make_folder(folder, name)
+    config, weights = plain.read_folder(folder)
+    return dict(name=name, folder=folder, page=page, cfg=cfg, config=config, weights=weights)
+
+
+def prompts_for(tiny, lengths, seed=5):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, tiny["cfg"]["vocab_size"], (n,), generator=g).tolist() for n in lengths]
+
+
+def engine(tiny, dtype="float32", **kw):
+    from tessweave_engine_amd.cli import engine_for
+    options = dict(dtype=dtype, block_size=tiny["page"], kv_blocks=128, max_context=256, prefill_chunk=13,
+                   max_active=4, no_prefix_cache=True)
+    options.update(kw)
+    return engine_for(tiny["folder"], **options)
+
+
+def test_greedy_generation_through_the_entry_point(tiny):
+    """The workloads of the two tiny configurations: ragged prompts, portions of 13 beside decode tokens."""
+    lengths, count = ([5, 17, 33], 16) if tiny["name"] == "A" else ([1, 9, 40, 64, 100], 24)
+    prompts = prompts_for(tiny, lengths)
+    want = [plain.greedy(tiny["config"], tiny["weights"], p, count) for p in prompts]
+    e = engine(tiny)
+    got = e.generate(prompts, max_tokens=count, ignore_eos=True)
+    stats = e.stats()
+    e.close()
+    assert got == want
+    assert stats["graph_replays"] > 0 and stats["free_blocks"] == stats["physical_blocks"]
+    # the same through the unpacked projections (the --unfused ablation) and without graphs
+    e = engine(tiny, unfused=True, no_graphs=True)
+    assert e.generate(prompts[:2], max_tokens=6, ignore_eos=True) == [w[:6] for w in want[:2]]
+    e.close()
+
+
+def test_bfloat16_generation_agrees_where_the_choice_is_clear(tiny):
+    prompts = prompts_for(tiny, [7, 30], seed=9)
+    e = engine(tiny, dtype="bfloat16")
+    got = e.generate(prompts, max_tokens=8, ignore_eos=True)
+    e.close()
+    for p, out in zip(prompts, got):
+        tokens = list(p)
+        for t in out:
+            logits = plain.forward(tiny["config"], tiny["weights"], tokens)[-1]
+            top = logits.topk(2).values
+            if float(top[0] - top[1]) > 0.04 * float(logits.abs().max()):
+                assert t == int(logits.argmax())
+            tokens.append(t)
+
+
+def test_long_decoding_and_the_first_tokens(tiny):
+    """One token after the other for hundreds of steps (pages fill and new ones are taken), from position 0."""
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.weights import load_model
+    n = 300
+    tokens = prompts_for(tiny, [n], seed=21)[0]
+    want = plain.forward(tiny["config"], tiny["weights"], tokens)
+    for dtype in ("float32", "bfloat16"):
+        model = load_model(tiny["folder"], dtype=dtype, device="cuda:0")
+        cache = CacheManager(model.cache_layout(), tiny["page"], math.ceil(n / tiny["page"]), 2, dtype=dtype,
+                             device=model.device, prefix_cache=False, max_request_tokens=n + tiny["page"])
+        stepper = Stepper(model, cache, max_step_tokens=16)
+        seq = cache.open("long")
+        rows = [stepper.step([StepEntry(seq, [t], [0])]).cpu().clone() for t in tokens]
+        got = torch.cat(rows)
+        assert stepper.graph_replays >= n - 2
+        if dtype == "float32":
+            torch.testing.assert_close(got, want, atol=5e-6, rtol=2e-5)
+            torch.testing.assert_close(got[:3], want[:3], atol=5e-6, rtol=2e-5)      # positions 0, 1, 2
+        else:
+            assert float((got - want).abs().max()) <= 0.02 * float(want.abs().max())
+        cache.close(seq)
+        cache.check()
+        stepper.close()
+
+
+def test_sampling_seed_is_independent_of_other_requests(tiny):
+    """tests/test_engine.py:251-260 of the reference, with the device sampler."""
+    p = prompts_for(tiny, [5, 4], seed=2)
+    e = engine(tiny)
+    a = e.submit(p[0], 7, temperature=.8, seed=9, ignore_eos=True)
+    e.drain()
+    e.submit(p[1], 9, temperature=.5, seed=8, ignore_eos=True)
+    b = e.submit(p[0], 7, temperature=.8, seed=9, ignore_eos=True)
+    c = e.submit(p[0], 7, temperature=.8, seed=10, ignore_eos=True)
+    e.drain()
+    assert a.output == b.output and len(a.output) == 7
+    assert c.output != a.output                      # another seed, another stream (7 draws at T=0.8)
+    cold = e.submit(p[0], 7, temperature=1e-4, seed=3, ignore_eos=True)
+    e.drain()
+    assert cold.output == plain.greedy(tiny["config"], tiny["weights"], p[0], 7)
+    e.close()
+
+
+def test_prefix_pages_are_reused_on_the_gpu(tiny):
+    page = tiny["page"]
+    shared = prompts_for(tiny, [32], seed=4)[0]
+    p1, p2 = shared + [3, 4, 5], shared + [9, 1]
+    e = engine(tiny, no_prefix_cache=False)
+    first = e.submit(p1, 6, ignore_eos=True)
+    e.drain()
+    again = e.submit(p1, 6, ignore_eos=True)
+    other = e.submit(p2, 6, ignore_eos=True)
+    e.drain()
+    assert again.cached == 32 and other.cached == 32          # 32 tokens = full pages at both page sizes
+    assert again.output == first.output == plain.greedy(tiny["config"], tiny["weights"], p1, 6)
+    assert other.output == plain.greedy(tiny["config"], tiny["weights"], p2, 6)
+    e.close()
+    e.cache.check()
+    assert len(e.cache.pools[0].free) == e.cache.pools[0].capacity
+
+
+# ---- each part alone --------------------------------------------------------------------------------
+class PartHarness:
+    """A cache, a step context and the GPU stream for running single parts on given sequences."""
+
+    def __init__(self, model, page, dtype):
+        from tessweave_engine_amd.cache import CacheManager
+        from tessweave_engine_amd.engine import Stepper
+        self.cache = CacheManager(model.cache_layout(), page, 64, 4, dtype=dtype, device=model.device,
+                                  prefix_cache=False, max_request_tokens=256)
+        self.stepper = Stepper(model, self.cache, max_step_tokens=64, use_graphs=False)
+
+    def context(self, entries):
+        ctx, ordered, _ = self.stepper.prepare(entries)
+        self.stepper.upload(ctx)
+        return ctx, ordered
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_each_part_alone(tiny, dtype):
+    from tessweave_engine_amd.engine import StepEntry
+    from tessweave_engine_amd.parts import LayerRun
+    from tessweave_engine_amd.weights import load_model
+    model = load_model(tiny["folder"], dtype=dtype, device="cuda:0")
+    torch_dtype = model.dtype
+    s, w = plain.sizes(tiny["config"]), tiny["weights"]
+    h = PartHarness(model, tiny["page"], dtype)
+    a, b = h.cache.open("a"), h.cache.open("b")
+    toks = prompts_for(tiny, [11, 6], seed=8)
+    tight = dict(atol=2e-5, rtol=2e-5) if dtype == "float32" else dict(atol=3e-2, rtol=3e-2)
+    with torch.cuda.stream(h.stepper.stream):
+        ctx, ordered = h.context([StepEntry(a, toks[0], []), StepEntry(b, toks[1], [])])
+        n = ctx.n_tokens
+        # embedding
+        x = model.embedding.forward(ctx)
+        ids = torch.tensor(toks[0] + toks[1])
+        torch.testing.assert_close(x.cpu(), w["model.embed_tokens.weight"][ids], atol=0, rtol=0)
+        # norm
+        block = model.blocks[0]
+        x0 = torch.randn(n, s["hidden"], generator=torch.Generator().manual_seed(1))
+        xd = x0.to("cuda")
+        hn = block.mixer_norm.forward(ctx, xd)
+        want_h = plain.rms_norm(x0, w["model.layers.0.input_layernorm.weight"], s["eps"])
+        torch.testing.assert_close(hn.float().cpu(), want_h, **tight)
+        # position encoding
+        cos, sin = block.mixer.position.tables(ctx)
+        pos = torch.cat([torch.arange(11), torch.arange(6)]).float()
+        inv = s["theta"] ** (-torch.arange(0, s["head_dim"], 2, dtype=torch.float32) / s["head_dim"])
+        torch.testing.assert_close(cos.cpu(), (pos[:, None] * inv).cos(), atol=2e-6, rtol=0)
+        torch.testing.assert_close(sin.cpu(), (pos[:, None] * inv).sin(), atol=2e-6, rtol=0)
+        # mixer: adds attention of the normalised input into the residual stream
+        h_in = want_h.to(torch_dtype)
+        xr = xd.clone()
+        block.mixer.forward(ctx, LayerRun(0, 0), h_in.to("cuda"), xr)
+        want_x = x0.clone()
+        want_x[:11] += plain.attention_block(h_in.float()[:11], torch.arange(11), w, "model.layers.0.self_attn.", s)
+        want_x[11:] += plain.attention_block(h_in.float()[11:], torch.arange(6), w, "model.layers.0.self_attn.", s)
+        torch.testing.assert_close(xr.cpu(), want_x, **tight)
+        # feed-forward
+        xf = xd.clone()
+        block.ffn.forward(ctx, h_in.to("cuda"), xf)
+        p = "model.layers.0.mlp."
+        want_f = x0 + plain.swiglu(h_in.float(), w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+        torch.testing.assert_close(xf.cpu(), want_f, **tight)
+        # whole block
+        xb = xd.clone()
+        block.forward(ctx, LayerRun(0, 0), xb)
+        want_b = torch.cat([plain.decoder_layer(x0[:11], torch.arange(11), w, 0, s),
+                            plain.decoder_layer(x0[11:], torch.arange(6), w, 0, s)])
+        torch.testing.assert_close(xb.cpu(), want_b, **(tight if dtype == "float32" else dict(atol=6e-2, rtol=6e-2)))
+        # head on chosen rows
+        rows = torch.tensor([0, n - 1], dtype=torch.int32, device="cuda")
+        hf = model.final_norm.forward(ctx, xd, rows=rows, tag="norm.final")
+        logits = model.head.forward(ctx, hf)
+        head_w = w["model.embed_tokens.weight"] if s["tied"] else w["lm_head.weight"]
+        want_l = plain.rms_norm(x0[[0, n - 1]], w["model.norm.weight"], s["eps"]) @ head_w.T
+        torch.testing.assert_close(logits.cpu(), want_l, **(dict(atol=1e-4, rtol=1e-4) if dtype == "float32" else dict(atol=.15, rtol=.05)))
+    torch.cuda.synchronize()
+
+
+# ---- schedules: a layer named twice, a layer that reads another layer's cache --------------------------
+def test_schedule_names_a_layer_twice_and_shares_a_cache(tiny):
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.config import build_model, config_from_dict
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.parts import LayerRun
+    from tessweave_engine_amd.weights import read_tensors
+    cfg = config_from_dict(tiny["cfg"])
+    model = build_model(cfg)
+    last = len(model.blocks) - 1
+    # block 0 runs twice (each run with a cache slot of its own); the last run reuses block `last`
+    # but READS the keys and values that the second run of block 0 wrote
+    model.schedule = [LayerRun(0, 0), LayerRun(0, 1), LayerRun(last, 1, writes_cache=False)]
+    model._layout = None
+    model.bind(read_tensors(tiny["folder"], model.tensor_specs(), torch.float32, "cuda:0"), torch.float32, "cuda:0")
+    assert len(model.cache_layout().needs) == 2
+    s, w = plain.sizes(tiny["config"]), tiny["weights"]
+    tokens = prompts_for(tiny, [23], seed=6)[0]
+
+    def plain_run(tokens):
+        x = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+        pos = torch.arange(len(tokens))
+        x = plain.decoder_layer(x, pos, w, 0, s)
+        # second run of block 0: keep its rotated keys and its values for the sharing layer
+        p0 = "model.layers.0."
+        hn = plain.rms_norm(x, w[p0 + "input_layernorm.weight"], s["eps"])
+        t = len(tokens)
+        k = (hn @ w[p0 + "self_attn.k_proj.weight"].T + w[p0 + "self_attn.k_proj.bias"]).reshape(t, s["kv_heads"], s["head_dim"])
+        v = (hn @ w[p0 + "self_attn.v_proj.weight"].T + w[p0 + "self_attn.v_proj.bias"]).reshape(t, s["kv_heads"], s["head_dim"])
+        k = plain.rope(k, pos, s["theta"])
+        x = plain.decoder_layer(x, pos, w, 0, s)
+        # sharing layer: its own q, the other layer's k and v
+        pl = f"model.layers.{last}."
+        hn = plain.rms_norm(x, w[pl + "input_layernorm.weight"], s["eps"])
+        q = (hn @ w[pl + "self_attn.q_proj.weight"].T + w[pl + "self_attn.q_proj.bias"]).reshape(t, s["heads"], s["head_dim"])
+        q = plain.rope(q, pos, s["theta"])
+        att = plain.attention(q, k, v, pos).reshape(t, -1) @ w[pl + "self_attn.o_proj.weight"].T
+        x = x + att
+        hn = plain.rms_norm(x, w[pl + "post_attention_layernorm.weight"], s["eps"])
+        x = x + plain.swiglu(hn, w[pl + "mlp.gate_proj.weight"], w[pl + "mlp.up_proj.weight"], w[pl + "mlp.down_proj.weight"])
+        x = plain.rms_norm(x, w["model.norm.weight"], s["eps"])
+        head = w["model.embed_tokens.weight"] if s["tied"] else w["lm_head.weight"]
+        return x @ head.T
+
+    want = plain_run(tokens)
+    cache = CacheManager(model.cache_layout(), tiny["page"], 16, 2, dtype="float32", device=model.device,
+                         prefix_cache=False, max_request_tokens=64)
+    stepper = Stepper(model, cache, max_step_tokens=32)
+    seq = cache.open("s")
+    outs = [stepper.step([StepEntry(seq, tokens[:9], list(range(9)))]).cpu().clone(),
+            stepper.step([StepEntry(seq, tokens[9:20], list(range(11)))]).cpu().clone()]
+    outs += [stepper.step([StepEntry(seq, [t], [0])]).cpu().clone() for t in tokens[20:]]
+    torch.testing.assert_close(torch.cat(outs), want, atol=5e-6, rtol=2e-5)
+    stepper.close()
+
+
+# ---- a toy mixer with state of its own, defined here, registered and stepped without touching the package ----
+def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, device):
+    from dataclasses import dataclass
+    from safetensors.torch import save_file
+    from tessweave_engine_amd.cache import CacheManager, CacheNeed, FixedState
+    from tessweave_engine_amd.config import register_architecture, unregister_architecture
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.parts import (DecoderModel, Mixer, OutputHead, PreNormBlock, RMSNorm, SwiGLU,
+                                            TokenEmbedding, LayerRun, GroupedQueryAttention, RotaryEmbedding)
+    from tessweave_engine_amd.weights import MATRIX, TensorSpec, load_model, random_tensors
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str
+        vocab_size: int
+        hidden_size: int
+        intermediate_size: int
+        decay: float
+        max_position_embeddings: int = 256
+        eos_token_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls("ToyDecayForCausalLM", d["vocab_size"], d["hidden_size"], d["intermediate_size"], d["decay"])
+
+        def to_dict(self):
+            return dict(architectures=[self.architecture], model_type="toy_decay", vocab_size=self.vocab_size,
+                        hidden_size=self.hidden_size, intermediate_size=self.intermediate_size, decay=self.decay)
+
+    class DecayMixer(Mixer):
+        """state_t = decay * state_{t-1} + h_t;  output_t = state_t @ W.T.  The state is the request's own."""
+        graph_safe = False                      # written with torch operations
+
+        def __init__(self, name, hidden, decay):
+            self.name, self.hidden, self.decay = name, hidden, decay
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.hidden, self.hidden), MATRIX)]
+
+        def bind(self, tensors, dtype, device):
+            self.weight = tensors.pop(self.name + ".weight").float()
+
+        def cache_need(self):
+            return CacheNeed(state=FixedState((self.hidden,), "float32"))
+
+        def forward(self, ctx, run, h, x):
+            state = ctx.cache.state[run.cache_slot]
+            for s in range(ctx.n_seqs):
+                slot = ctx.h_state_slots[s]
+                for row in range(ctx.h_q_start[s], ctx.h_q_start[s + 1]):
+                    state[slot] = self.decay * state[slot] + h[row].float()
+                    x[row] += state[slot] @ self.weight.T
+
+    def build_toy(c):
+        emb = TokenEmbedding("emb", c.vocab_size, c.hidden_size)
+        rotary = RotaryEmbedding(16, 10000.0)
+        blocks = [PreNormBlock(RMSNorm("l0.n1", c.hidden_size, 1e-5), DecayMixer("l0.mix", c.hidden_size, c.decay),
+                               RMSNorm("l0.n2", c.hidden_size, 1e-5), SwiGLU("l0.ff.", c.hidden_size, c.intermediate_size)),
+                  PreNormBlock(RMSNorm("l1.n1", c.hidden_size, 1e-5),
+                               GroupedQueryAttention("l1.att.", c.hidden_size, 2, 1, 16, rotary, qkv_bias=False),
+                               RMSNorm("l1.n2", c.hidden_size, 1e-5), SwiGLU("l1.ff.", c.hidden_size, c.intermediate_size))]
+        return DecoderModel(c, emb, blocks, RMSNorm("final", c.hidden_size, 1e-5),
+                            OutputHead("head", c.vocab_size, c.hidden_size, tied_to=emb),
+                            schedule=[LayerRun(0, 0), LayerRun(1, 1), LayerRun(0, 2)])    # the toy layer runs twice
+
+    register_architecture("ToyDecayForCausalLM", "toy_decay", ToyConfig, build_toy)
+    try:
+        cfg = ToyConfig("ToyDecayForCausalLM", 61, 32, 48, 0.75)
+        (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+        tensors = random_tensors(build_toy(cfg).tensor_specs(), 3, std=0.2)
+        save_file(tensors, str(tmp_path / "model.safetensors"))
+        model = load_model(tmp_path, dtype="float32", device="cuda:0")          # config.json picks the toy class
+        assert type(model.blocks[0].mixer).__name__ == "DecayMixer" and not model.graph_safe_model
+        layout = model.cache_layout()
+        assert layout.state_slots == (0, 2) and len(layout.groups) == 1 and not layout.shares_prefixes
+
+        w = {k: v.float() for k, v in tensors.items()}
+
+        def plain_toy(tokens):
+            x = w["emb.weight"][torch.tensor(tokens)]
+            pos = torch.arange(len(tokens))
+
+            def toy_layer(x):
+                hn = plain.rms_norm(x, w["l0.n1.weight"], 1e-5)
+                state, rows = torch.zeros(32), []
+                for t in range(len(tokens)):
+                    state = 0.75 * state + hn[t]
+                    rows.append(state @ w["l0.mix.weight"].T)
+                x = x + torch.stack(rows)
+                hn = plain.rms_norm(x, w["l0.n2.weight"], 1e-5)
+                return x + plain.swiglu(hn, w["l0.ff.gate_proj.weight"], w["l0.ff.up_proj.weight"], w["l0.ff.down_proj.weight"])
+            x = toy_layer(x)
+            hn = plain.rms_norm(x, w["l1.n1.weight"], 1e-5)
+            t = len(tokens)
+            q = plain.rope((hn @ w["l1.att.q_proj.weight"].T).reshape(t, 2, 16), pos, 10000.0)
+            k = plain.rope((hn @ w["l1.att.k_proj.weight"].T).reshape(t, 1, 16), pos, 10000.0)
+            v = (hn @ w["l1.att.v_proj.weight"].T).reshape(t, 1, 16)
+            x = x + plain.attention(q, k, v, pos).reshape(t, 32) @ w["l1.att.o_proj.weight"].T
+            hn = plain.rms_norm(x, w["l1.n2.weight"], 1e-5)
+            x = x + plain.swiglu(hn, w["l1.ff.gate_proj.weight"], w["l1.ff.up_proj.weight"], w["l1.ff.down_proj.weight"])
+            x = toy_layer(x)
+            return plain.rms_norm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T
+
+        g = torch.Generator().manual_seed(1)
+        seqs = {name: torch.randint(0, 61, (n,), generator=g).tolist() for name, n in (("a", 19), ("b", 12), ("c", 9))}
+        cache = CacheManager(layout, 8, 8, 2, dtype="float32", device=model.device, max_request_tokens=32)
+        stepper = Stepper(model, cache, max_step_tokens=32)
+        a, b = cache.open("a"), cache.open("b")
+        got = {"a": [], "b": [], "c": []}
+
+        def run(*items):
+            entries = [StepEntry(seq, seqs[name][lo:hi], list(range(hi - lo))) for name, seq, lo, hi in items]
+            out, row = stepper.step(entries).cpu(), 0
+            for name, _, lo, hi in items:
+                got[name].append(out[row:row + hi - lo].clone())
+                row += hi - lo
+        run(("a", a, 0, 7))
+        run(("a", a, 7, 8), ("b", b, 0, 5))                 # a decodes beside b's prompt portion
+        run(("b", b, 5, 12), ("a", a, 8, 10))
+        cache.close(b)                                       # b's state slot and pages go to c
+        c = cache.open("c")
+        assert c.state_slot == b.state_slot
+        run(("a", a, 10, 19), ("c", c, 0, 9))
+        for name in seqs:
+            torch.testing.assert_close(torch.cat(got[name]), plain_toy(seqs[name]), atol=2e-5, rtol=2e-5)
+        assert stepper.graph_replays == 0
+        stepper.close()
+    finally:
+        unregister_architecture("ToyDecayForCausalLM")

@@ -1,0 +1,301 @@
+"""The scheduler's decisions, with a fake step function and sampler (no GPU)."""
+import queue
+
+import pytest
+import torch
+
+from tessweave_engine_amd.cache import CacheManager, CapacityError
+from tessweave_engine_amd.config import EngineConfig, build_model, config_from_dict
+from tessweave_engine_amd.engine import Engine
+
+VOCAB = 128
+CFG = dict(model_type="qwen2", vocab_size=VOCAB, hidden_size=64, intermediate_size=64, num_hidden_layers=2,
+           num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=128)
+
+
+def next_token(history):
+    """A deterministic toy language model: the next token is a function of the whole history."""
+    return (sum((i + 1) * t for i, t in enumerate(history)) * 7 + len(history)) % VOCAB
+
+
+class FakeStepper:
+    """Keeps each request's tokens as the real cache would, returns one-hot logits, logs every batch."""
+
+    def __init__(self, cache):
+        self.cache, self.history, self.batches, self.fail = cache, {}, [], None
+
+    def step(self, entries):
+        if self.fail:
+            raise self.fail
+        rows = []
+        self.batches.append([(e.seq.id, e.seq.computed, len(e.tokens), list(e.want)) for e in entries])
+        for e in entries:
+            self.cache.ensure(e.seq, e.seq.computed + len(e.tokens))
+            h = self.history.setdefault(e.seq.id, [None] * 0)
+            assert len(h) <= e.seq.computed                          # prefix-shared tokens were never run here
+            h.extend([None] * (e.seq.computed - len(h)))
+            h.extend(e.tokens)
+            for w in e.want:
+                rows.append((e, e.seq.computed + w + 1))
+        logits = torch.zeros(len(rows), VOCAB)
+        for i, (e, upto) in enumerate(rows):
+            logits[i, next_token(self.full[e.seq.id][:upto])] = 1.0
+        for e in entries:
+            self.cache.advance(e.seq, e.seq.computed + len(e.tokens))
+        return logits
+
+    full = {}
+
+
+class FakeSampler:
+    def sample(self, logits, temperatures, seeds, counters):
+        self.last = (list(temperatures), list(seeds), list(counters))
+        return logits.argmax(-1).tolist()
+
+
+def make(**kw):
+    defaults = dict(block_size=4, kv_blocks=32, max_context=64, prefill_chunk=4, min_prefill_chunk=1, dtype="float32")
+    defaults.update(kw)
+    config = EngineConfig(**defaults)
+    model = build_model(config_from_dict(CFG))
+    cache = CacheManager(model.cache_layout(), config.block_size, config.kv_blocks, config.max_active,
+                         prefix_cache=config.prefix_cache, max_request_tokens=config.max_context)
+    stepper = FakeStepper(cache)
+    stepper.full = {}
+    engine = Engine(model, config, stepper=stepper, cache=cache, sampler=FakeSampler())
+    submit = engine.submit
+
+    def tracked(tokens, *a, **k):
+        r = submit(tokens, *a, **k)
+        stepper.full[r.id] = r.tokens                                  # the request's growing token list
+        return r
+    engine.submit = tracked
+    return engine, stepper
+
+
+def expected(prompt, n):
+    tokens, out = list(prompt), []
+    for _ in range(n):
+        out.append(next_token(tokens))
+        tokens.append(out[-1])
+    return out
+
+
+def drain(engine):
+    for _ in range(500):
+        if not engine.step():
+            return
+    raise AssertionError("engine did not terminate")
+
+
+def test_submit_validation():
+    e, _ = make()
+    for prompt, count in (([], 1), ([VOCAB], 1), ([1], 64), ([1], 0), ([1.0], 1), ([-1], 1)):
+        with pytest.raises(ValueError):
+            e.submit(prompt, count)
+    for t in (-0.1, 2.5, float("nan"), float("inf")):
+        with pytest.raises(ValueError):
+            e.submit([1], 1, temperature=t)
+    small, _ = make(kv_blocks=2)
+    with pytest.raises(ValueError):
+        small.submit([1] * 8, 4)                                       # could never fit: refused, not queued
+    e.close()
+
+
+def test_chunked_prompts_decode_and_outputs():
+    e, s = make()
+    prompts = [[4, 5, 6, 7, 8], [2, 3, 4, 5, 6, 7, 8, 9, 10]]
+    rs = [e.submit(p, 7) for p in prompts]
+    drain(e)
+    for r, p in zip(rs, prompts):
+        assert r.output == expected(p, 7) and r.status == "length"
+        assert r.events.qsize() == 8
+    # every step: decode tokens first, then prompt portions, within the token budget
+    for batch in s.batches:
+        counts = [c for _, _, c, _ in batch]
+        kinds = [c == 1 and bool(w) for _, _, c, w in batch]
+        assert sum(counts) <= e.config.step_token_budget
+    e.close()
+    e.cache.check()
+    assert len(e.cache.pools[0].free) == 32
+
+
+def test_round_robin_and_first_token_from_the_completing_portion():
+    e, s = make(max_step_tokens=4, max_active=2)          # room for one portion of 4 per step
+    a = e.submit(list(range(1, 11)), 2)                   # 10 tokens: portions 4, 4, 2
+    b = e.submit(list(range(20, 29)), 2)                  # 9 tokens: portions 4, 4, 1
+    e.step(); e.step(); e.step(); e.step()
+    order = [[(rid, start, n) for rid, start, n, _ in batch] for batch in s.batches]
+    assert order[0] == [(a.id, 0, 4)] and order[1] == [(b.id, 0, 4)]          # round-robin over the two prompts
+    assert order[2] == [(a.id, 4, 4)] and order[3] == [(b.id, 4, 4)]
+    assert not a.output and not b.output
+    e.step()          # a's last portion (2 tokens) completes its prompt; the budget's rest completes b's
+    assert s.batches[4] == [(a.id, 8, 2, [1]), (b.id, 8, 1, [0])]
+    assert a.output == expected(a.prompt, 1) and b.output == expected(b.prompt, 1)
+    e.step()          # both decode: one token each, logits wanted for both
+    assert s.batches[5] == [(a.id, 10, 1, [0]), (b.id, 9, 1, [0])]
+    assert a.status == "length" and b.status == "length" and b.output == expected(b.prompt, 2)
+    assert not e.step()
+    # decode comes first in a mixed step
+    e, s = make(max_step_tokens=5, max_active=2)
+    a = e.submit([1, 2], 3)
+    e.step()
+    b = e.submit(list(range(30, 40)), 1)
+    e.step()
+    assert s.batches[1] == [(a.id, 2, 1, [0]), (b.id, 0, 4, [])]
+    e.close()
+
+
+def test_budget_lets_several_prompts_advance_but_no_crumbs():
+    e, s = make(max_step_tokens=16, prefill_chunk=8, min_prefill_chunk=4, max_active=3)
+    a, b, c = e.submit([1] * 20, 1), e.submit([2] * 20, 1), e.submit([3] * 20, 1)
+    e.step()
+    assert [(rid, n) for rid, _, n, _ in s.batches[0]] == [(a.id, 8), (b.id, 8)]      # 16 tokens; nothing left for c
+    e, s = make(max_step_tokens=11, prefill_chunk=8, min_prefill_chunk=4, max_active=3)
+    a, b = e.submit([1] * 20, 1), e.submit([2] * 20, 1)
+    e.step()
+    assert [(rid, n) for rid, _, n, _ in s.batches[0]] == [(a.id, 8)]                 # 3 left: below the minimum portion
+    e.close()
+
+
+def test_eos_is_emitted_then_stops_and_ignore_eos():
+    prompt = [3, 4, 5, 6, 7]
+    want = expected(prompt, 12)
+    end = next(i for i in range(2, 12) if want[i] not in want[:i])
+    cfg = dict(CFG, eos_token_id=want[end])
+    model = build_model(config_from_dict(cfg))
+    config = EngineConfig(block_size=4, kv_blocks=32, max_context=64, prefill_chunk=4, min_prefill_chunk=1, dtype="float32")
+    cache = CacheManager(model.cache_layout(), 4, 32, 4, max_request_tokens=64)
+    s = FakeStepper(cache)
+    s.full = {}
+    e = Engine(model, config, stepper=s, cache=cache, sampler=FakeSampler())
+    r = e.submit(prompt, 12)
+    s.full[r.id] = r.tokens
+    r2 = e.submit(prompt, 12, ignore_eos=True)
+    s.full[r2.id] = r2.tokens
+    drain(e)
+    assert r.status == "stop" and r.output == want[:end + 1]            # EOS is part of the output
+    assert r2.status == "length" and r2.output == want
+    done = [ev for ev in iter(lambda: r.events.get_nowait() if not r.events.empty() else None, None)][-1]
+    assert done["finish_reason"] == "stop" and done["usage"] == {"prompt_tokens": 5, "completion_tokens": end + 1,
+                                                                 "total_tokens": 6 + end}
+    e.close()
+
+
+def test_admission_reserves_the_worst_case_and_waits_in_order():
+    # reference vector (tests/test_engine.py:160-170): 4 pages of 4; two requests of 6 + 6 tokens need 3 each
+    e, s = make(kv_blocks=4)
+    a = e.submit([1, 2, 3, 4, 5, 6], 6)
+    b = e.submit([8, 9, 10, 11, 12, 13], 6)
+    e.step()
+    assert a.status == "active" and b.status == "waiting"
+    drain(e)
+    assert len(a.output) == 6 and len(b.output) == 6 and b.output == expected(b.prompt, 6)
+    # no skipping ahead: a small request behind a large one waits too
+    e, s = make(kv_blocks=4, max_active=3)
+    first = e.submit([1] * 6, 6)
+    large = e.submit([2] * 10, 6)        # 4 pages: cannot be admitted while `first` runs
+    small = e.submit([3], 1)             # 1 page would fit, but it is behind `large`
+    e.step()
+    assert (first.status, large.status, small.status) == ("active", "waiting", "waiting")
+    drain(e)
+    assert [r.status for r in (first, large, small)] == ["length"] * 3
+    e.cache.check()
+    e.close()
+
+
+def test_pages_never_run_out_mid_generation():
+    e, s = make(kv_blocks=6, max_active=4)
+    rs = [e.submit([i + 1] * 5, 7) for i in range(4)]          # 3 pages each: two at a time
+    while e.step():
+        e.cache.check()
+        assert len(e.active) <= 2
+    assert all(r.status == "length" and len(r.output) == 7 for r in rs)
+    e.close()
+
+
+def test_prefix_reuse_vectors():
+    # tests/test_engine.py:113-126 of the reference: cached == 8, one prompt token runs, same output
+    e, s = make()
+    p = [2, 3, 4, 5, 6, 7, 8, 9, 10]
+    first = e.submit(p, 5)
+    drain(e)
+    count = e.counters["prefill_tokens"]
+    second = e.submit(p, 5)
+    drain(e)
+    assert first.output == second.output and second.cached == 8
+    assert e.counters["prefill_tokens"] - count == 1
+    # :128-137: a divergent tail shares only the full block before it
+    third = e.submit([2, 3, 4, 5, 60, 70], 4)
+    drain(e)
+    assert third.cached == 4 and third.output == expected(third.prompt, 4)
+    # :139-147: another namespace shares nothing
+    fourth = e.submit(p, 2, namespace="tenant-b")
+    drain(e)
+    assert fourth.cached == 0
+    e.close()
+    e.cache.check()
+    assert len(e.cache.pools[0].free) == e.cache.pools[0].capacity
+
+
+def test_cancel_queue_limit_and_slow_consumer():
+    e, s = make(max_active=1)
+    a = e.submit([1, 2, 3, 4, 5, 6, 7], 8)
+    b = e.submit([1, 2], 8)
+    e.step()
+    e.cancel(b.id)
+    e.cancel(a.id)
+    assert not e.step() and (a.status, b.status) == ("cancelled", "cancelled")
+    assert len(e.cache.pools[0].free) == e.cache.pools[0].capacity
+    e.close()
+    e, s = make(max_queue=1)
+    r = e.submit([1, 2], 4)
+    with pytest.raises(CapacityError):
+        e.submit([1, 2], 4)
+    r.events = queue.Queue(maxsize=1)
+    drain(e)
+    assert r.status == "error" and r.events.get()["finish_reason"] == "error"
+    e.close()
+
+
+def test_a_failing_step_ends_every_request_and_frees_everything():
+    e, s = make()
+    r = e.submit([1, 2], 3)
+    s.fail = RuntimeError("test kernel failure")
+    e.start()
+    e.thread.join(timeout=3)
+    assert "test kernel failure" in e.fatal
+    assert r.events.get()["finish_reason"] == "error"
+    assert len(e.cache.pools[0].free) == e.cache.pools[0].capacity
+    with pytest.raises(RuntimeError):
+        e.submit([1], 1)
+    e.close()
+
+
+def test_sampling_arguments_are_per_request():
+    e, s = make()
+    a = e.submit([1, 2, 3], 3, temperature=0.8, seed=9)
+    b = e.submit([4, 5, 6, 7], 3)
+    drain(e)
+    temps, seeds, counters = e.sampler.last
+    assert a.temperature == 0.8 and a.seed == 9 and b.temperature == 0.0
+    assert len(a.output) == 3 and len(b.output) == 3
+    e.close()
+
+
+def test_generate_convenience_and_worker_thread():
+    e, s = make()
+    orig = e.submit
+    prompts = [[1, 2, 3], [9, 8, 7, 6, 5, 4]]
+    outs = e.generate(prompts, max_tokens=4)
+    assert outs == [expected(p, 4) for p in prompts]
+    r = orig([5, 5, 5], 3)
+    e.start()
+    got = []
+    while True:
+        ev = r.events.get(timeout=5)
+        if ev["type"] == "done":
+            break
+        got.append(ev["token_id"])
+    assert got == expected([5, 5, 5], 3) and e.stats()["finished"] == 3
+    e.close()
