@@ -141,6 +141,10 @@ def main():
     achieved = (weight_bytes + kv_bytes) / (ms_per_step / 1000) / 1e9
 
     t = args.prefill_tokens
+    if t <= 0:                      # decode only (profiling runs)
+        print(json.dumps({"value": round(value, 1), "ms_per_step": round(ms_per_step, 4), "batch": args.batch,
+                          "roofline_frac": round(achieved / HBM_PEAK_GBS, 4)}))
+        return 0
     prefill_ms = prefill_run(model, torch, t, args.dtype, args.seed)
     linear_flops = 2.0 * t * c.num_hidden_layers * layer_weights + 2.0 * c.vocab_size * c.hidden_size
     attn_flops = c.num_hidden_layers * 4.0 * c.num_attention_heads * c.head_dim * (t * (t + 1) / 2)

@@ -134,22 +134,22 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 // `partial[split][M][N]` and `splitk_reduce_kernel` finishes, always in the
 // same order, so results do not depend on timing.
 // =====================================================================================
-template <typename T, typename OutT, int MT>
+template <typename T, typename OutT, int MT, int TW, int U>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const T* __restrict__ A, long lda,
                                                           const T* __restrict__ W, long ldw,
                                                           const float* __restrict__ bias,
                                                           const float* residual, long ldr, OutT* C,
                                                           long ldc, float* __restrict__ partial, int M,
-                                                          int N, int K, int n_tiles, int splits) {
+                                                          int N, int K, int n_groups, int splits) {
+  // A wave owns TW tiles of 16 output columns (16*TW rows of W) and one K range.
   typedef typename Elem<T>::Frag Frag;
   constexpr int EPF = Elem<T>::kPerFrag;
-  constexpr int U = 4;                       // MFMA steps per loop iteration
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int unit = blockIdx.x * 4 + wave;
-  if (unit >= n_tiles * splits) return;
-  const int tile = unit % n_tiles, split = unit / n_tiles;
+  if (unit >= n_groups * splits) return;
+  const int group = unit % n_groups, split = unit / n_groups;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = tile * 16;
+  const int n0 = group * 16 * TW;
 
   const int chunks = K / EPF;                              // 16-byte chunks per row
   const int steps = (chunks + 3) / 4;                      // MFMA steps over all of K
@@ -157,41 +157,214 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const T* __restrict__ 
   const int step_begin = split * steps_per_split;
   const int step_end = min(steps, step_begin + steps_per_split);
 
-  f32x4 acc[MT];
+  f32x4 acc[TW][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < TW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const bool w_row_ok = n0 + r < N;
-  const T* w_row = W + (size_t)(w_row_ok ? n0 + r : 0) * ldw;
+  // Rows past the end are clamped to the last valid row: what they produce is
+  // never stored, and the main loop needs no per-load predicate.
+  const T* w_row[TW];
+#pragma unroll
+  for (int t = 0; t < TW; ++t) w_row[t] = W + (size_t)min(n0 + t * 16 + r, N - 1) * ldw + g * EPF;
   const T* a_row[MT];
-  bool a_ok[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    a_ok[mt] = mt * 16 + r < M;
-    a_row[mt] = A + (size_t)(a_ok[mt] ? mt * 16 + r : 0) * lda;
-  }
+  for (int mt = 0; mt < MT; ++mt) a_row[mt] = A + (size_t)min(mt * 16 + r, M - 1) * lda + g * EPF;
 
-  for (int s0 = step_begin; s0 < step_end; s0 += U) {
-    Frag wf[U];
+  // Two register stages of U MFMA steps each: the loads of one stage are in
+  // flight while the other is multiplied.
+  Frag wf[2][U][TW], xf[2][U][MT];
+  auto load = [&](const int buf, int s0) {          // all U steps lie inside [step_begin, full_end)
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int chunk = (s0 + u) * 4 + g;
-      const bool ok = w_row_ok && (s0 + u) < step_end && chunk < chunks;
-      wf[u] = ok ? tw_load_frag(w_row + (size_t)chunk * EPF) : Elem<T>::zero();
+      const size_t off = (size_t)(s0 + u) * 4 * EPF;
+#pragma unroll
+      for (int t = 0; t < TW; ++t) wf[buf][u][t] = tw_load_frag(w_row[t] + off);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xf[buf][u][mt] = tw_load_frag(a_row[mt] + off);
     }
+  };
+  auto multiply = [&](const int buf) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int chunk = (s0 + u) * 4 + g;
-      const bool in_k = (s0 + u) < step_end && chunk < chunks;
+    for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const Frag af = (a_ok[mt] && in_k) ? tw_load_frag(a_row[mt] + (size_t)chunk * EPF) : Elem<T>::zero();
-        tw_mma16(acc[mt], wf[u], af);
+      for (int t = 0; t < TW; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) tw_mma16(acc[t][mt], wf[buf][u][t], xf[buf][u][mt]);
+  };
+  // steps whose four chunks all exist, in whole stages
+  const int whole_steps = min(step_end, chunks / 4);
+  const int n_stages = whole_steps > step_begin ? (whole_steps - step_begin) / U : 0;
+  const int full_end = step_begin + n_stages * U;
+  if (n_stages > 0) {
+    load(0, step_begin);
+    int s0 = step_begin;
+    for (int i = 0; i + 2 <= n_stages; i += 2, s0 += 2 * U) {
+      load(1, s0 + U);
+      multiply(0);
+      if (i + 2 < n_stages) load(0, s0 + 2 * U);
+      multiply(1);
+    }
+    if (n_stages & 1) multiply(0);
+  }
+  // tail: single steps with per-chunk predicates
+  for (int s = full_end; s < step_end; ++s) {
+    const int chunk = s * 4 + g;
+    const bool ok = chunk < chunks;
+    const size_t off = (size_t)s * 4 * EPF;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const Frag af = ok ? tw_load_frag(a_row[mt] + off) : Elem<T>::zero();
+#pragma unroll
+      for (int t = 0; t < TW; ++t) {
+        const Frag wfrag = ok ? tw_load_frag(w_row[t] + off) : Elem<T>::zero();
+        tw_mma16(acc[t][mt], wfrag, af);
       }
     }
   }
 
-  // acc[mt][j] = sum_k W[n0 + 4g + j][k] * A[16 mt + r][k]
+  // acc[t][mt][j] = sum_k W[n0 + 16 t + 4g + j][k] * A[16 mt + r][k]
+#pragma unroll
+  for (int t = 0; t < TW; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int row = mt * 16 + r;
+      if (row >= M) continue;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = n0 + t * 16 + 4 * g + j;
+        if (col >= N) continue;
+        if (splits > 1) {
+          partial[((size_t)split * M + row) * N + col] = acc[t][mt][j];
+        } else {
+          float v = acc[t][mt][j] + (bias ? bias[col] : 0.f);
+          if (residual) v += residual[(size_t)row * ldr + col];
+          C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
+        }
+      }
+    }
+}
+
+// =====================================================================================
+// Skinny kernel, workgroup-cooperative form. The 4 waves of a workgroup own 4
+// neighbouring tiles of 16 output columns and the SAME K range. Per stage of U
+// MFMA steps the workgroup copies the activations' K slice [16*MT rows][U*64 B]
+// to LDS once (instead of every wave reading it from L2); each wave streams its
+// own 16 weight rows from global memory into registers. Two stages in flight.
+// =====================================================================================
+#define TW_XROW(U) ((U) * 64 + 16)          /* LDS bytes per activation row of a stage, padded */
+
+template <typename T, typename OutT, int MT, int U>
+__global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restrict__ A, long lda,
+                                                              const T* __restrict__ W, long ldw,
+                                                              const float* __restrict__ bias,
+                                                              const float* residual, long ldr, OutT* C,
+                                                              long ldc, float* __restrict__ partial, int M,
+                                                              int N, int K, int n_groups, int splits) {
+  typedef typename Elem<T>::Frag Frag;
+  constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr int XROW = TW_XROW(U);
+  constexpr int XSTAGE = MT * 16 * XROW;
+  constexpr int XLOADS = MT * U / 4;                   // activation fragments per thread per stage
+  static_assert(U % 4 == 0, "a stage is copied by 256 threads in whole rounds");
+  __shared__ __attribute__((aligned(16))) char lds[2 * XSTAGE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int group = blockIdx.x % n_groups, split = blockIdx.x / n_groups;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = group * 64 + wave * 16;
+
+  const int chunks = K / EPF;
+  const int steps = (chunks + 3) / 4;
+  const int steps_per_split = (steps + splits - 1) / splits;
+  const int step_begin = split * steps_per_split;
+  const int step_end = min(steps, step_begin + steps_per_split);
+  const int n_stages = step_end > step_begin ? (step_end - step_begin + U - 1) / U : 0;
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const T* w_row = W + (size_t)min(n0 + r, N - 1) * ldw;
+  // this thread's share of the activation slice: fragment f = i*256 + tid -> (row f / (4U), chunk f % (4U))
+  const T* x_src[XLOADS];
+  int x_dst[XLOADS], x_chunk[XLOADS];
+#pragma unroll
+  for (int i = 0; i < XLOADS; ++i) {
+    const int f = i * 256 + tid, row = f / (4 * U), c = f % (4 * U);
+    x_src[i] = A + (size_t)min(row, M - 1) * lda;
+    x_chunk[i] = c;
+    x_dst[i] = row * XROW + c * 16;
+  }
+
+  Frag wf[2][U], xg[XLOADS];
+  auto load_w = [&](const int buf, int s0, bool whole) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int chunk = (s0 + u) * 4 + g;
+      if (whole || ((s0 + u) < step_end && chunk < chunks))
+        wf[buf][u] = tw_load_frag(w_row + (size_t)chunk * EPF);
+      else
+        wf[buf][u] = Elem<T>::zero();
+    }
+  };
+  auto load_x = [&](int s0, bool whole) {
+#pragma unroll
+    for (int i = 0; i < XLOADS; ++i) {
+      const int chunk = s0 * 4 + x_chunk[i];
+      if (whole || (chunk < step_end * 4 && chunk < chunks))
+        xg[i] = tw_load_frag(x_src[i] + (size_t)chunk * EPF);
+      else
+        xg[i] = Elem<T>::zero();
+    }
+  };
+  auto store_x = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < XLOADS; ++i) *reinterpret_cast<Frag*>(lds + buf * XSTAGE + x_dst[i]) = xg[i];
+  };
+  auto multiply = [&](const int buf) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const Frag xf = *reinterpret_cast<const Frag*>(lds + buf * XSTAGE + (mt * 16 + r) * XROW + (u * 4 + g) * 16);
+        tw_mma16(acc[mt], wf[buf][u], xf);
+      }
+  };
+  auto whole_stage = [&](int s0) { return s0 + U <= step_end && (s0 + U) * 4 <= chunks; };
+
+  if (n_stages > 0) {
+    {
+      const bool whole = whole_stage(step_begin);
+      load_w(0, step_begin, whole);
+      load_x(step_begin, whole);
+      store_x(0);
+    }
+    __syncthreads();
+    for (int i = 0; i < n_stages; i += 2) {
+      const int s0 = step_begin + i * U;
+      const bool more1 = i + 1 < n_stages, more2 = i + 2 < n_stages;
+      if (more1) {
+        const bool whole = whole_stage(s0 + U);
+        load_w(1, s0 + U, whole);
+        load_x(s0 + U, whole);
+      }
+      multiply(0);
+      if (more1) store_x(1);
+      __syncthreads();
+      if (!more1) break;
+      if (more2) {
+        const bool whole = whole_stage(s0 + 2 * U);
+        load_w(0, s0 + 2 * U, whole);
+        load_x(s0 + 2 * U, whole);
+      }
+      multiply(1);
+      if (more2) store_x(0);
+      __syncthreads();
+    }
+  }
+
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int row = mt * 16 + r;
@@ -270,14 +443,27 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
   return TW_LAUNCH_RESULT();
 }
 
+// Output tiles per wave of the skinny kernel (they share the activation fragments).
+static int skinny_tiles_per_wave(int N) { return N >= 16384 ? 2 : 1; }
+
 // How many K ranges the skinny kernel uses for an [N, K] weight: enough waves
-// to fill 256 CUs several times over, each range at least 32 MFMA steps long.
+// to fill 256 CUs several times over, each range at least 16 MFMA steps long.
 // The choice depends on N and K only, never on the rows of a batch.
 static int skinny_splits(int N, int K, int epf) {
-  const int n_tiles = tw_div_up(N, 16);
+  const int groups = tw_div_up(N, 16 * skinny_tiles_per_wave(N));
   const int steps = tw_div_up(K / epf, 4);
-  int splits = tw_div_up(2048, n_tiles);
-  const int max_by_k = steps / 32 > 0 ? steps / 32 : 1;
+  int splits = tw_div_up(2048, groups);
+  const int max_by_k = steps / 16 > 0 ? steps / 16 : 1;
+  if (splits > max_by_k) splits = max_by_k;
+  if (splits > 16) splits = 16;
+  return splits < 1 ? 1 : splits;
+}
+
+static int skinny_lds_splits(int N, int K, int epf) {
+  const int groups = tw_div_up(N, 64);
+  const int steps = tw_div_up(K / epf, 4);
+  int splits = tw_div_up(512, groups);
+  const int max_by_k = steps / 16 > 0 ? steps / 16 : 1;
   if (splits > max_by_k) splits = max_by_k;
   if (splits > 16) splits = 16;
   return splits < 1 ? 1 : splits;
@@ -287,26 +473,56 @@ extern "C" long tw_linear_workspace_bytes(int dtype, int max_rows, int N, int K)
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
   if (K % epf) return 0;
   const int rows = max_rows < 64 ? max_rows : 64;
-  const int splits = skinny_splits(N, K, epf);
+  int splits = skinny_splits(N, K, epf);
+  const int coop = skinny_lds_splits(N, K, epf);
+  if (coop > splits) splits = coop;
   return splits > 1 ? (long)splits * rows * N * 4 : 0;
+}
+
+template <typename T, typename OutT, int MT, int TW>
+static int launch_skinny_tw(const T* A, long lda, const T* W, long ldw, const float* bias,
+                            const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                            long partial_bytes, int M, int N, int K, hipStream_t stream) {
+  constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr int U = (MT * TW <= 2) ? 8 : 4;
+  const int groups = tw_div_up(N, 16 * TW);
+  int splits = skinny_splits(N, K, EPF);
+  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) splits = 1;
+  const int units = groups * splits;
+  gemm_skinny_kernel<T, OutT, MT, TW, U><<<tw_div_up(units, 4), 256, 0, stream>>>(
+      A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
+  int err = TW_LAUNCH_RESULT();
+  if (err || splits == 1) return err;
+  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
+                                                                             ldr, C, ldc, M, N);
+  return TW_LAUNCH_RESULT();
+}
+
+template <typename T, typename OutT, int MT>
+static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const float* bias,
+                             const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                             long partial_bytes, int M, int N, int K, hipStream_t stream) {
+  constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr int U = MT == 1 ? 8 : 4;
+  const int groups = tw_div_up(N, 64);
+  int splits = skinny_lds_splits(N, K, EPF);
+  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) splits = 1;
+  gemm_skinny_lds_kernel<T, OutT, MT, U><<<groups * splits, 256, 0, stream>>>(
+      A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
+  int err = TW_LAUNCH_RESULT();
+  if (err || splits == 1) return err;
+  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
+                                                                             ldr, C, ldc, M, N);
+  return TW_LAUNCH_RESULT();
 }
 
 template <typename T, typename OutT, int MT>
 static int launch_skinny(const T* A, long lda, const T* W, long ldw, const float* bias,
                          const float* residual, long ldr, OutT* C, long ldc, float* partial,
                          long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  constexpr int EPF = Elem<T>::kPerFrag;
-  const int n_tiles = tw_div_up(N, 16);
-  int splits = skinny_splits(N, K, EPF);
-  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) splits = 1;
-  const int units = n_tiles * splits;
-  gemm_skinny_kernel<T, OutT, MT><<<tw_div_up(units, 4), 256, 0, stream>>>(
-      A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, n_tiles, splits);
-  int err = TW_LAUNCH_RESULT();
-  if (err || splits == 1) return err;
-  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
-                                                                             ldr, C, ldc, M, N);
-  return TW_LAUNCH_RESULT();
+  if (skinny_tiles_per_wave(N) == 2)
+    return launch_skinny_tw<T, OutT, MT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  return launch_skinny_tw<T, OutT, MT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
 }
 
 template <typename T, typename OutT>
@@ -316,14 +532,22 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
   constexpr int EPF = Elem<T>::kPerFrag;
   const bool aligned = K % EPF == 0 && lda % EPF == 0 && ldw % EPF == 0 &&
                        ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
-  // force: 0 = choose, 1 = generic, 2 = skinny, 3 = tiled 128x128, 4 = tiled 128x256
+  // force: 0 = choose, 1 = generic, 2 = skinny (per-wave), 3 = tiled 128x128, 4 = tiled 128x256,
+  //        5 = skinny (workgroup-cooperative)
   if (force == 1 || !aligned) {
     TW_REQUIRE(force <= 1);
     gemm_generic_kernel<T, OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(A, lda, W, ldw, bias, residual,
                                                                                ldr, C, ldc, M, N, K);
     return TW_LAUNCH_RESULT();
   }
-  if (force == 2 || (force == 0 && M <= 64)) {
+  if (force == 5 || (force == 0 && M <= 64)) {
+    TW_REQUIRE(M <= 64);
+    if (M <= 16) return launch_skinny_lds<T, OutT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    if (M <= 32) return launch_skinny_lds<T, OutT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    if (M <= 48) return launch_skinny_lds<T, OutT, 3>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny_lds<T, OutT, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  }
+  if (force == 2) {
     TW_REQUIRE(M <= 64);
     if (M <= 16) return launch_skinny<T, OutT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
     if (M <= 32) return launch_skinny<T, OutT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);

@@ -135,7 +135,7 @@ def linear_workspace_bytes(dtype, max_rows, n, k):
     return int(library().tw_linear_workspace_bytes(dtype_id(dtype), int(max_rows), int(n), int(k)))
 
 
-GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE = 0, 1, 2, 3, 4
+GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY_COOP = 0, 1, 2, 3, 4, 5
 
 
 def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_AUTO):

@@ -129,11 +129,11 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
     bias = rand((n,), torch.float32, device, 0.5, seed=3)
     res = rand((m, n), torch.float32, device, 1.0, seed=4)
     want = x.double().cpu() @ w.double().cpu().T
-    ws_bytes = max(ops.linear_workspace_bytes(dtype, m, n, k), 16)
+    ws_bytes = max(ops.linear_workspace_bytes(dtype, m, n, k), 16 * 64 * n * 4)
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=device)
     forces = [ops.GEMM_AUTO, ops.GEMM_GENERIC, ops.GEMM_TILED, ops.GEMM_TILED_WIDE]
     if m <= 64:
-        forces.append(ops.GEMM_SKINNY)
+        forces += [ops.GEMM_SKINNY, ops.GEMM_SKINNY_COOP]
     scale = math.sqrt(k) * 0.05
     t = dict(atol=2e-5 * scale, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2 * scale, rtol=2e-2)
     for force in forces:
