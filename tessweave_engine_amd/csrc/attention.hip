@@ -56,6 +56,7 @@ struct AttnArgs {
   int q_heads, kv_heads, head_dim, page_size, window;
   float scale;
   int splits;
+  int page_shift;         // log2(page_size) if it is a power of two, else -1
 };
 
 // Per-wave online-softmax state for one 16-row tile. Lane (r, g) belongs to row r.
@@ -251,25 +252,262 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
   }
 }
 
-// Merge the splits of one (sequence, head): grid = (q_heads, n_seqs), one thread per d.
+// =====================================================================================
+// Decode, bfloat16, pages of 8 keys or a multiple: blocks of 32 keys.
+// Row i = 4a + j of the block's first (second) score tile stands for key 8a + j
+// (8a + 4 + j), so lane group g ends up with the probabilities of the 8
+// CONSECUTIVE keys 8g .. 8g+7: they are the B operand of one 16x16x32 MFMA per
+// 16 output dims, whose A operand is a single 16-byte load of values[d][8g..8g+7].
+// The keys and values of the next block are loaded while this one is computed.
+// =====================================================================================
+template <int DTMAX>
+struct KVBlock {
+  static constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
+  bf16x8 k[2][NSMAX];
+  bf16x8 v[DTMAX];
+};
+
+template <int DTMAX>
+__global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
+  constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
+  __shared__ float lds_o[3][16][DTMAX * 16];
+  __shared__ float lds_ml[3][16][2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int G = a.q_heads / a.kv_heads;
+  const int row_tiles = (G + 15) / 16;
+  const int kvh = blockIdx.y / row_tiles, rt = blockIdx.y % row_tiles;
+  const int seq = a.seq0 + blockIdx.z;
+  const int split = blockIdx.x;
+  const int kv_len = a.kv_len[seq];
+  const int token = a.q_start[seq];
+  const int t = kv_len - 1;
+  const int* table = a.block_table + (size_t)seq * a.table_stride;
+  const int D = a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
+  const bf16_t* keys = (const bf16_t*)a.keys;
+  const bf16_t* values = (const bf16_t*)a.values;
+
+  const int hig = rt * 16 + r;
+  const bool row_ok = hig < G;
+  const int head = kvh * G + hig;
+  bf16x8 qf[NSMAX];
+  {
+    const bf16_t* q_row = (const bf16_t*)a.q + (size_t)token * a.ldq + (size_t)head * D;
+#pragma unroll
+    for (int st = 0; st < NSMAX; ++st) {
+      const int chunk = st * 4 + g;
+      qf[st] = (row_ok && chunk < chunks) ? tw_load_frag(q_row + chunk * 8) : Elem<bf16_t>::zero();
+    }
+  }
+  f32x4 acc[DTMAX];
+#pragma unroll
+  for (int dt = 0; dt < DTMAX; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  const int lo = a.window > 0 ? max(0, t - a.window + 1) : 0;
+  const int blk_lo = lo / 32, blk_hi = (kv_len + 31) / 32;
+  const int per_split = (blk_hi - blk_lo + a.splits - 1) / a.splits;
+  const int begin = blk_lo + split * per_split;
+  const int end = min(blk_hi, begin + per_split);
+
+  // Page ids of a 32-key block are the same for every lane: they are read with
+  // scalar loads (blk is made wave-uniform), off the vector-memory queue.
+  const int pshift = a.page_shift, pmask = P - 1;
+  const int ppb = P >= 32 ? 1 : (32 >> pshift);                    // pages per block: 1, 2 or 4
+  const unsigned head_stride = (unsigned)P * D;                      // elements of one (page, kv head)
+  auto issue = [&](int blk_v, KVBlock<DTMAX>& L) {
+    const int blk = __builtin_amdgcn_readfirstlane(blk_v);
+    const int p0 = blk * 32;
+    const int first = p0 >> pshift;
+    int pg[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pg[i] = (i < ppb && p0 + (i << pshift) < kv_len) ? table[first + i] : -1;
+    auto page_of = [&](int ko) {                                     // ko: key offset inside the block
+      const int i = P >= 32 ? 0 : (ko >> pshift);
+      return i == 0 ? pg[0] : (i == 1 ? pg[1] : (i == 2 ? pg[2] : pg[3]));
+    };
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+      const int ko = 8 * (r >> 2) + 4 * tile + (r & 3);              // the key this lane's row stands for
+      const int p = p0 + ko;
+      int page = page_of(ko);
+      if (p >= kv_len || p < lo) page = -1;
+      const size_t base = ((size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh) * head_stride;
+      const bf16_t* k_row = keys + base + (unsigned)(p & pmask) * D + g * 8;
+#pragma unroll
+      for (int st = 0; st < NSMAX; ++st)
+        L.k[tile][st] = (page >= 0 && st * 4 + g < chunks) ? tw_load_frag(k_row + st * 32) : Elem<bf16_t>::zero();
+    }
+    const int kv0 = 8 * g;                                            // this lane's 8 consecutive keys
+    int vpage = page_of(kv0);
+    if (p0 + kv0 >= kv_len || p0 + kv0 + 7 < lo) vpage = -1;
+    const size_t vbase = ((size_t)(vpage < 0 ? 0 : vpage) * a.kv_heads + kvh) * head_stride;
+    const bf16_t* v_base = values + vbase + ((p0 + kv0) & pmask) + (unsigned)r * P;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+        L.v[dt] = vpage >= 0 ? tw_load_frag(v_base + (unsigned)(dt * 16) * P) : Elem<bf16_t>::zero();
+  };
+
+  auto compute = [&](int blk, KVBlock<DTMAX>& L) {
+    const int p0 = blk * 32;
+    f32x4 s[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int st = 0; st < NSMAX; ++st)
+        if (st * 4 < chunks) tw_mma16(s[tile], L.k[tile][st], qf[st]);
+    // this lane: row r (a head), keys p0 + 8g + e, e = 4*tile + j
+    float pr[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int p = p0 + 8 * g + e;
+      const bool ok = row_ok && p < kv_len && p >= lo;                  // decode: every cached key is at or before t
+      pr[e] = ok ? s[e >> 2][e & 3] * a.scale : -INFINITY;
+      mx = fmaxf(mx, pr[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __expf(m - m_use);
+    float sum = 0.f;
+    bf16x8 pb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = __expf(pr[e] - m_use);
+      sum += pe;
+      pb[e] = (bf16_t)pe;
+    }
+    sum += __shfl_xor(sum, 16, TW_WAVE);
+    sum += __shfl_xor(sum, 32, TW_WAVE);
+    l = l * alpha + sum;
+    m = m_new;
+    const bool edge = p0 + 32 > kv_len || p0 < lo;                      // only edge blocks hold keys to blank out
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts) {
+        bf16x8 vq = L.v[dt];
+        if (edge) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int p = p0 + 8 * g + e;
+            if (p >= kv_len || p < lo) vq[e] = (bf16_t)0.f;
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[dt][j] *= alpha;
+        tw_mma16(acc[dt], vq, pb);
+      }
+  };
+
+  {
+    // One block in registers per wave; several waves per SIMD hide each other's memory latency.
+    KVBlock<DTMAX> A;
+    for (int blk = begin + wave; blk < end; blk += 4) {
+      issue(blk, A);
+      compute(blk, A);
+    }
+  }
+
+  // ---- merge the 4 waves (fixed order: wave 0 absorbs 1, 2, 3) -------------------
+  if (wave > 0) {
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) lds_o[wave - 1][r][dt * 16 + 4 * g + j] = acc[dt][j];
+    if (g == 0) {
+      lds_ml[wave - 1][r][0] = m;
+      lds_ml[wave - 1][r][1] = l;
+    }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  float m_all = m;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) m_all = fmaxf(m_all, lds_ml[w][r][0]);
+  const float m_use = m_all == -INFINITY ? 0.f : m_all;
+  const float own = __expf(m - m_use);
+  l *= own;
+#pragma unroll
+  for (int dt = 0; dt < DTMAX; ++dt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[dt][j] *= own;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    const float f = __expf(lds_ml[w][r][0] - m_use);
+    l += lds_ml[w][r][1] * f;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[dt][j] += lds_o[w][r][dt * 16 + 4 * g + j] * f;
+  }
+  if (!row_ok) return;
+  if (a.splits == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* dst = (bf16_t*)a.out + (size_t)token * a.ldo + (size_t)head * D;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = (bf16_t)(acc[dt][j] * inv);
+  } else {
+    const size_t slot = ((size_t)blockIdx.z * a.q_heads + head) * a.splits + split;
+    float* dst = a.part_o + slot * D;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = acc[dt][j];
+    if (g == 0) {
+      a.part_ml[slot * 2] = m_all;
+      a.part_ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
+// Merge the splits of one (sequence, head): grid = (q_heads, n_seqs). Thread (d, c)
+// sums the splits c, c + C, ... of output dim d; the C partial sums are then
+// added in a fixed order, so the result does not depend on timing.
+#define TW_REDUCE_THREADS 256
 template <typename T>
-__global__ void attn_decode_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                          const int* __restrict__ q_start, int seq0, T* out, long ldo,
-                                          int q_heads, int head_dim, int splits) {
-  const int head = blockIdx.x, local = blockIdx.y;
+__global__ __launch_bounds__(TW_REDUCE_THREADS) void attn_decode_reduce_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ q_start,
+    int seq0, T* out, long ldo, int q_heads, int head_dim, int splits) {
+  __shared__ float s_w[64];                    // weight of each split: exp(m_s - m)
+  __shared__ float s_acc[TW_REDUCE_THREADS];
+  __shared__ float s_l;
+  const int head = blockIdx.x, local = blockIdx.y, tid = threadIdx.x;
   const size_t slot0 = ((size_t)local * q_heads + head) * splits;
-  float m = -INFINITY;
-  for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
-  const float m_use = m == -INFINITY ? 0.f : m;
-  float l = 0.f;
-  for (int s = 0; s < splits; ++s) l += part_ml[(slot0 + s) * 2 + 1] * expf(part_ml[(slot0 + s) * 2] - m_use);
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  const int token = q_start[seq0 + local];
-  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float o = 0.f;
-    for (int s = 0; s < splits; ++s)
-      o += part_o[(slot0 + s) * head_dim + d] * expf(part_ml[(slot0 + s) * 2] - m_use);
-    out[(size_t)token * ldo + (size_t)head * head_dim + d] = tw_from_float<T>(o * inv);
+  if (tid < 64) {
+    const float mine = tid < splits ? part_ml[(slot0 + tid) * 2] : -INFINITY;
+    const float m = tw_wave_max(mine);
+    const float m_use = m == -INFINITY ? 0.f : m;
+    const float w = tid < splits ? expf(mine - m_use) : 0.f;
+    s_w[tid] = w;
+    const float lw = tid < splits ? part_ml[(slot0 + tid) * 2 + 1] * w : 0.f;
+    // fixed-order sum over the splits
+    float l = 0.f;
+    for (int i = 0; i < 64; ++i) l += __shfl(lw, i, TW_WAVE);
+    if (tid == 0) s_l = l;
+  }
+  __syncthreads();
+  const int cols = TW_REDUCE_THREADS / head_dim > 0 ? TW_REDUCE_THREADS / head_dim : 1;   // head_dim <= 256
+  const int d = tid % head_dim, c = tid / head_dim;
+  float o = 0.f;
+  if (c < cols)
+    for (int sp = c; sp < splits; sp += cols) o += part_o[(slot0 + sp) * head_dim + d] * s_w[sp];
+  s_acc[tid] = o;
+  __syncthreads();
+  if (tid < head_dim) {
+    float total = 0.f;
+    for (int i = 0; i < cols; ++i) total += s_acc[i * head_dim + tid];
+    const float l = s_l;
+    const int token = q_start[seq0 + local];
+    out[(size_t)token * ldo + (size_t)head * head_dim + tid] = tw_from_float<T>(l > 0.f ? total / l : 0.f);
   }
 }
 
@@ -345,11 +583,21 @@ extern "C" long tw_attn_decode_workspace_floats(int n_seqs, int q_heads, int hea
   return splits > 1 ? (long)n_seqs * q_heads * splits * (head_dim + 2) : 0;
 }
 
+template <typename T> struct IsBf16 { static constexpr bool value = false; };
+template <> struct IsBf16<bf16_t> { static constexpr bool value = true; };
+
 template <typename T>
-static int decode_launch(AttnArgs a, int n_seqs, hipStream_t stream) {
+static int decode_launch(AttnArgs a, int n_seqs, int generic, hipStream_t stream) {
   const int G = a.q_heads / a.kv_heads;
   dim3 grid(a.splits, a.kv_heads * ((G + 15) / 16), n_seqs);
-  if (a.head_dim <= 64)
+  if (IsBf16<T>::value && a.page_shift >= 3 && !generic) {
+    if (a.head_dim <= 64)
+      attn_decode_bf16_kernel<4><<<grid, 256, 0, stream>>>(a);
+    else if (a.head_dim <= 128)
+      attn_decode_bf16_kernel<8><<<grid, 256, 0, stream>>>(a);
+    else
+      attn_decode_bf16_kernel<16><<<grid, 256, 0, stream>>>(a);
+  } else if (a.head_dim <= 64)
     attn_decode_kernel<T, 4><<<grid, 256, 0, stream>>>(a);
   else if (a.head_dim <= 128)
     attn_decode_kernel<T, 8><<<grid, 256, 0, stream>>>(a);
@@ -357,26 +605,29 @@ static int decode_launch(AttnArgs a, int n_seqs, hipStream_t stream) {
     attn_decode_kernel<T, 16><<<grid, 256, 0, stream>>>(a);
   int err = TW_LAUNCH_RESULT();
   if (err || a.splits == 1) return err;
-  const int threads = a.head_dim <= 64 ? 64 : (a.head_dim <= 128 ? 128 : 256);
-  attn_decode_reduce_kernel<T><<<dim3(a.q_heads, n_seqs), threads, 0, stream>>>(
+  attn_decode_reduce_kernel<T><<<dim3(a.q_heads, n_seqs), TW_REDUCE_THREADS, 0, stream>>>(
       a.part_o, a.part_ml, a.q_start, a.seq0, (T*)a.out, a.ldo, a.q_heads, a.head_dim, a.splits);
   return TW_LAUNCH_RESULT();
 }
 
 // Sequences seq0 .. seq0 + n_seqs - 1 must each have exactly one token in this step.
 // `workspace` holds tw_attn_decode_workspace_floats floats when splits > 1.
+// generic != 0 forces the kernel that takes every type and page size.
 extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* keys, const void* values,
                               const int* block_table, int table_stride, const int* q_start,
                               const int* kv_len, int seq0, int n_seqs, void* out, long ldo,
                               float* workspace, long workspace_floats, int q_heads, int kv_heads,
                               int head_dim, int page_size, int window, float scale, int splits,
-                              hipStream_t stream) {
+                              int generic, hipStream_t stream) {
   AttnArgs a;
   a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
   a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = splits;
   a.part_o = nullptr; a.part_ml = nullptr;
+  a.page_shift = -1;
+  for (int sh = 0; sh < 20; ++sh)
+    if ((1 << sh) == page_size) a.page_shift = sh;
   int err = check_common(a);
   if (err) return err;
   TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && splits >= 1 && splits <= 64 && n_seqs <= 65535);
@@ -387,8 +638,8 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
     a.part_o = workspace;
     a.part_ml = workspace + (size_t)n_seqs * q_heads * splits * head_dim;
   }
-  if (dtype == TW_DTYPE_F32) return decode_launch<float>(a, n_seqs, stream);
-  if (dtype == TW_DTYPE_BF16) return decode_launch<bf16_t>(a, n_seqs, stream);
+  if (dtype == TW_DTYPE_F32) return decode_launch<float>(a, n_seqs, generic, stream);
+  if (dtype == TW_DTYPE_BF16) return decode_launch<bf16_t>(a, n_seqs, generic, stream);
   return TW_ERR_BAD_ARGUMENT;
 }
 
@@ -418,6 +669,9 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = 1;
   a.part_o = nullptr; a.part_ml = nullptr;
+  a.page_shift = -1;
+  for (int sh = 0; sh < 20; ++sh)
+    if ((1 << sh) == page_size) a.page_shift = sh;
   int err = check_common(a);
   if (err) return err;
   TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && max_q_len >= 1 && n_seqs <= 65535);

@@ -194,8 +194,12 @@ def _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads
 
 
 def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out, q_heads, kv_heads,
-                head_dim, scale, window=0, splits=1, workspace=None):
-    """Attention of sequences seq0..seq0+n_seqs-1, each with ONE query token, over their pages."""
+                head_dim, scale, window=0, splits=1, workspace=None, generic=False):
+    """Attention of sequences seq0..seq0+n_seqs-1, each with ONE query token, over their pages.
+
+    generic=True forces the kernel that takes every type and page size (bfloat16 with
+    pages of a multiple of 8 keys otherwise runs a faster kernel of its own).
+    """
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
     ws_ptr, ws_floats = None, 0
@@ -206,7 +210,8 @@ def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out
                                    _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
                                    _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
                                    seq0, n_seqs, _dev(out), ldo, ws_ptr, ws_floats, q_heads, kv_heads, head_dim,
-                                   keys.shape[2], int(window or 0), float(scale), int(splits), _stream()),
+                                   keys.shape[2], int(window or 0), float(scale), int(splits), 1 if generic else 0,
+                                   _stream()),
           "attn_decode")
     return out
 

@@ -216,11 +216,11 @@ def test_attn_decode_matrix(ops, device, dtype, head_dim, heads, kv_heads):
     qd = q.reshape(len(lengths), heads * head_dim).to(device)
     q_start = torch.arange(len(lengths) + 1, dtype=torch.int32, device=device)
     kv_len = torch.tensor(lengths, dtype=torch.int32, device=device)
-    for splits in (1, 2, 5):
+    for splits, generic in ((1, False), (2, False), (5, False), (1, True), (3, True)):
         out = torch.full((len(lengths), heads * head_dim), float("nan"), dtype=dtype, device=device)
         ws = torch.empty(max(1, ops.attn_decode_workspace_floats(len(lengths), heads, head_dim, splits)), device=device)
         ops.attn_decode(qd, keys, values, table, q_start, kv_len, 0, len(lengths), out, heads, kv_heads,
-                        head_dim, head_dim ** -0.5, splits=splits, workspace=ws)
+                        head_dim, head_dim ** -0.5, splits=splits, workspace=ws, generic=generic)
         torch.testing.assert_close(out.float().cpu().reshape(len(lengths), heads, head_dim), want, **ATTN_TOL[dtype])
 
 
