@@ -31,24 +31,30 @@ extern "C" int tw_embed_gather(int dtype, const int* ids, const void* table, flo
 // ---- RMS norm -------------------------------------------------------------------------
 // y = x * rsqrt(mean(x^2) + eps) * w, statistics and products in float32, one
 // rounding to the output type. `rows` (optional) picks the input row of each
-// output row. If `add` is given the input row is x + sum_s add[s] and that sum
-// is written back to x first (split-K partial sums of the layer before).
+// output row. If `add` is given the input row is (sum_s add[s]) + x (split-K
+// partial sums of the layer before, added up in the order the separate
+// reduction kernel uses); without `rows` that sum is also written back to x.
 template <typename T>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ w, T* __restrict__ out,
                                const int* __restrict__ rows, int hidden, float eps,
-                               const float* __restrict__ add, int add_splits, size_t add_stride) {
+                               const float* __restrict__ add, int add_splits, size_t add_stride,
+                               float* __restrict__ row_scratch) {
   __shared__ float lds[16];
   const int o = blockIdx.x;
   const int r = rows ? rows[o] : o;
   float* src = x + (size_t)r * hidden;
   float ss = 0.f;
   if (add) {
+    // with gathered rows the sums go to a scratch row (two outputs may name one input row)
+    float* dst = rows ? row_scratch + (size_t)o * hidden : src;
     for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
-      float v = src[h];
+      float v = 0.f;
       for (int s = 0; s < add_splits; ++s) v += add[s * add_stride + (size_t)r * hidden + h];
-      src[h] = v;
+      v += src[h];
+      dst[h] = v;
       ss += v * v;
     }
+    src = dst;
   } else {
     for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
       const float v = src[h];
@@ -62,21 +68,77 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ 
     dst[h] = tw_from_float<T>(src[h] * scale * w[h]);
 }
 
+// The same for hidden % 4 == 0 with at most 4 * blockDim.x elements per row: every
+// thread owns ONE group of 4 consecutive elements, kept in registers between the
+// two passes; the partial sums are read with independent 16-byte loads. (The sum
+// of squares is associated differently from the kernel above: results of the two
+// kernels agree to rounding, not to the bit.)
+template <typename T>
+__global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restrict__ w, T* __restrict__ out,
+                                    const int* __restrict__ rows, int hidden, float eps,
+                                    const float* __restrict__ add, int add_splits, size_t add_stride) {
+  __shared__ float lds[16];
+  const int o = blockIdx.x;
+  const int r = rows ? rows[o] : o;
+  const int h = threadIdx.x * 4;
+  const bool mine = h < hidden;
+  float* src = x + (size_t)r * hidden;
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  if (mine) {
+    if (add) {
+      const float* p = add + (size_t)r * hidden + h;
+      int s = 0;
+      for (; s + 4 <= add_splits; s += 4) {
+        const f32x4 a0 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 0) * add_stride);
+        const f32x4 a1 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 1) * add_stride);
+        const f32x4 a2 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 2) * add_stride);
+        const f32x4 a3 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 3) * add_stride);
+        v = (((v + a0) + a1) + a2) + a3;
+      }
+      for (; s < add_splits; ++s) v = v + *reinterpret_cast<const f32x4*>(p + (size_t)s * add_stride);
+      v = v + *reinterpret_cast<const f32x4*>(src + h);
+      if (!rows) *reinterpret_cast<f32x4*>(src + h) = v;
+    } else {
+      v = *reinterpret_cast<const f32x4*>(src + h);
+    }
+  }
+  float ss = mine ? ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3] : 0.f;
+  ss = tw_block_sum(ss, lds);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+  if (mine) {
+    const f32x4 wv = *reinterpret_cast<const f32x4*>(w + h);
+    T* dst = out + (size_t)o * hidden + h;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) dst[e] = tw_from_float<T>(v[e] * scale * wv[e]);
+  }
+}
+
 extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, const int* rows,
                           int n_out, int hidden, float eps, const float* add, int add_splits,
-                          long add_stride, hipStream_t stream) {
+                          long add_stride, float* row_scratch, hipStream_t stream) {
   TW_REQUIRE(n_out >= 0 && hidden > 0 && eps > 0.f);
-  TW_REQUIRE(add == nullptr || (rows == nullptr && add_splits > 0));
+  TW_REQUIRE(add == nullptr || (add_splits > 0 && (rows == nullptr || row_scratch != nullptr)));
   if (n_out == 0) return 0;
+  if (out_dtype != TW_DTYPE_F32 && out_dtype != TW_DTYPE_BF16) return TW_ERR_BAD_ARGUMENT;
+  // few rows (decode): one group of 4 elements per thread, everything in registers
+  if (n_out <= 64 && hidden % 4 == 0 && hidden <= 4096 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+      (add == nullptr || ((uintptr_t)add % 16 == 0 && add_stride % 4 == 0))) {
+    const int threads = (hidden / 4 + 63) / 64 * 64;
+    if (out_dtype == TW_DTYPE_F32)
+      rmsnorm_vec4_kernel<float><<<n_out, threads, 0, stream>>>(x, w, (float*)out, rows, hidden, eps, add,
+                                                                add_splits, (size_t)add_stride);
+    else
+      rmsnorm_vec4_kernel<bf16_t><<<n_out, threads, 0, stream>>>(x, w, (bf16_t*)out, rows, hidden, eps, add,
+                                                                 add_splits, (size_t)add_stride);
+    return TW_LAUNCH_RESULT();
+  }
   const int threads = hidden >= 2048 ? 512 : 256;
   if (out_dtype == TW_DTYPE_F32)
     rmsnorm_kernel<float><<<n_out, threads, 0, stream>>>(x, w, (float*)out, rows, hidden, eps, add,
-                                                         add_splits, (size_t)add_stride);
-  else if (out_dtype == TW_DTYPE_BF16)
-    rmsnorm_kernel<bf16_t><<<n_out, threads, 0, stream>>>(x, w, (bf16_t*)out, rows, hidden, eps, add,
-                                                          add_splits, (size_t)add_stride);
+                                                         add_splits, (size_t)add_stride, row_scratch);
   else
-    return TW_ERR_BAD_ARGUMENT;
+    rmsnorm_kernel<bf16_t><<<n_out, threads, 0, stream>>>(x, w, (bf16_t*)out, rows, hidden, eps, add,
+                                                          add_splits, (size_t)add_stride, row_scratch);
   return TW_LAUNCH_RESULT();
 }
 
@@ -107,14 +169,29 @@ extern "C" int tw_rope_table(const int* positions, const float* inv_freq, float*
 //   keys  [page][kv_head][offset][d]      and raw v to
 //   values[page][kv_head][d][offset]      (transposed inside the page),
 // slot = page * page_size + offset; a negative slot writes nothing.
+// If `partial` is given, the row's values are first formed as
+// round_T(sum_s partial[s][n][col] + bias[col]) (the split-K sums of the q/k/v
+// projection) and q, k, v are all written to qkv before anything else happens.
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* __restrict__ cos_t,
                                      const float* __restrict__ sin_t, const int* __restrict__ slots,
                                      T* __restrict__ keys, T* __restrict__ values, int q_heads,
-                                     int kv_heads, int head_dim, int rot, int page_size, int write_cache) {
+                                     int kv_heads, int head_dim, int rot, int page_size, int write_cache,
+                                     const float* __restrict__ partial, int splits, size_t split_stride,
+                                     const float* __restrict__ bias) {
   const int n = blockIdx.x;
   const int half = rot / 2;
   T* row = qkv + (size_t)n * ld;
+  if (partial) {
+    const int width = (q_heads + 2 * kv_heads) * head_dim;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      float v = 0.f;
+      for (int s = 0; s < splits; ++s) v += partial[s * split_stride + (size_t)n * width + c];
+      if (bias) v += bias[c];
+      row[c] = tw_from_float<T>(v);
+    }
+    __syncthreads();
+  }
   const float* c = cos_t + (size_t)n * half;
   const float* s = sin_t + (size_t)n * half;
   const int slot = write_cache ? slots[n] : -1;
@@ -155,23 +232,85 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* 
   }
 }
 
+// The same work from split-K partial sums, one workgroup per (token, head): the
+// head's values are round_T(sum_s partial[s][n][col] + bias[col]); q heads are
+// rotated into qkv, k heads are rotated into the pages, v heads go to the pages.
+template <typename T>
+__global__ void qkv_finish_kernel(T* __restrict__ qkv, long ld, const float* __restrict__ cos_t,
+                                  const float* __restrict__ sin_t, const int* __restrict__ slots,
+                                  T* __restrict__ keys, T* __restrict__ values, int q_heads, int kv_heads,
+                                  int head_dim, int rot, int page_size, int write_cache,
+                                  const float* __restrict__ partial, int splits, size_t split_stride,
+                                  const float* __restrict__ bias) {
+  const int head = blockIdx.x, n = blockIdx.y;
+  const int width = (q_heads + 2 * kv_heads) * head_dim;
+  const int half = rot / 2;
+  const int col0 = head * head_dim;
+  const float* src = partial + (size_t)n * width + col0;
+  auto value = [&](int d) {
+    float v = 0.f;
+    for (int s = 0; s < splits; ++s) v += src[s * split_stride + d];
+    if (bias) v += bias[col0 + d];
+    return tw_to_float(tw_from_float<T>(v));          // what the projection would have stored
+  };
+  const int slot = write_cache ? slots[n] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  T* row = qkv + (size_t)n * ld + col0;
+  if (head < q_heads + kv_heads) {
+    const bool is_q = head < q_heads;
+    if (!is_q && slot < 0) return;
+    T* dst = is_q ? row : keys + (((size_t)page * kv_heads + (head - q_heads)) * page_size + off) * head_dim;
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+      const float lo = value(j), hi = value(j + half);
+      const float cj = cos_t[(size_t)n * half + j], sj = sin_t[(size_t)n * half + j];
+      dst[j] = tw_from_float<T>(lo * cj - hi * sj);
+      dst[j + half] = tw_from_float<T>(hi * cj + lo * sj);
+    }
+    for (int d = rot + threadIdx.x; d < head_dim; d += blockDim.x) dst[d] = tw_from_float<T>(value(d));
+  } else {
+    if (slot < 0) return;
+    const int kh = head - q_heads - kv_heads;
+    T* dst = values + ((size_t)page * kv_heads + kh) * head_dim * page_size + off;
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) dst[(size_t)d * page_size] = tw_from_float<T>(value(d));
+  }
+}
+
 extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_t, const float* sin_t,
                                 const int* slots, void* keys, void* values, int n, int q_heads,
                                 int kv_heads, int head_dim, int rot, int page_size, int write_cache,
-                                hipStream_t stream) {
+                                const float* partial, int splits, const float* bias, hipStream_t stream) {
+  TW_REQUIRE(partial == nullptr || splits >= 1);
+  const size_t split_stride = (size_t)n * (q_heads + 2 * kv_heads) * head_dim;
   TW_REQUIRE(n >= 0 && q_heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0);
   TW_REQUIRE(rot >= 0 && rot <= head_dim && rot % 2 == 0);
   TW_REQUIRE(ld >= (long)(q_heads + 2 * kv_heads) * head_dim);
   TW_REQUIRE(!write_cache || (slots && keys && values));
   if (n == 0) return 0;
+  if (partial && n <= 65535) {
+    dim3 grid(q_heads + 2 * kv_heads, n);
+    const int threads = head_dim / 2 <= 64 ? 64 : 128;
+    if (dtype == TW_DTYPE_F32)
+      qkv_finish_kernel<float><<<grid, threads, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
+                                                            (float*)values, q_heads, kv_heads, head_dim, rot,
+                                                            page_size, write_cache, partial, splits, split_stride, bias);
+    else if (dtype == TW_DTYPE_BF16)
+      qkv_finish_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots, (bf16_t*)keys,
+                                                             (bf16_t*)values, q_heads, kv_heads, head_dim, rot,
+                                                             page_size, write_cache, partial, splits, split_stride, bias);
+    else
+      return TW_ERR_BAD_ARGUMENT;
+    return TW_LAUNCH_RESULT();
+  }
   if (dtype == TW_DTYPE_F32)
     rope_kv_write_kernel<float><<<n, 256, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
                                                        (float*)values, q_heads, kv_heads, head_dim, rot,
-                                                       page_size, write_cache);
+                                                       page_size, write_cache, partial, splits, split_stride, bias);
   else if (dtype == TW_DTYPE_BF16)
     rope_kv_write_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots,
                                                         (bf16_t*)keys, (bf16_t*)values, q_heads, kv_heads,
-                                                        head_dim, rot, page_size, write_cache);
+                                                        head_dim, rot, page_size, write_cache, partial, splits,
+                                                        split_stride, bias);
   else
     return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();

@@ -255,7 +255,22 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const T* __restrict__ 
 // =====================================================================================
 #define TW_XROW(U) ((U) * 64 + 16)          /* LDS bytes per activation row of a stage, padded */
 
-template <typename T, typename OutT, int MT, int U>
+// silu(g) * u on a fragment pair, float32 arithmetic, one rounding to T
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::Frag tw_silu_mul_frag(typename Elem<T>::Frag gf, typename Elem<T>::Frag uf) {
+  typename Elem<T>::Frag out;
+#pragma unroll
+  for (int e = 0; e < Elem<T>::kPerFrag; ++e) {
+    const float gv = tw_to_float(gf[e]), uv = tw_to_float(uf[e]);
+    out[e] = tw_from_float<T>(gv / (1.0f + expf(-gv)) * uv);
+  }
+  return out;
+}
+
+// SILU: the activations are [M][2K] = [gate | up]; the kernel multiplies silu(gate) * up by W
+// (the rounded product is what a separate SiLU-multiply kernel would have written).
+// PARTIAL: always write float32 partial sums partial[split][M][N] (splits >= 1), no epilogue.
+template <typename T, typename OutT, int MT, int U, bool SILU, bool PARTIAL>
 __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restrict__ A, long lda,
                                                               const T* __restrict__ W, long ldw,
                                                               const float* __restrict__ bias,
@@ -298,7 +313,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
     x_dst[i] = row * XROW + c * 16;
   }
 
-  Frag wf[2][U], xg[XLOADS];
+  Frag wf[2][U], xg[XLOADS], xu[SILU ? XLOADS : 1];
   auto load_w = [&](const int buf, int s0, bool whole) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -313,15 +328,19 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
       const int chunk = s0 * 4 + x_chunk[i];
-      if (whole || (chunk < step_end * 4 && chunk < chunks))
+      if (whole || (chunk < step_end * 4 && chunk < chunks)) {
         xg[i] = tw_load_frag(x_src[i] + (size_t)chunk * EPF);
-      else
+        if (SILU) xu[i] = tw_load_frag(x_src[i] + (size_t)K + (size_t)chunk * EPF);
+      } else {
         xg[i] = Elem<T>::zero();
+        if (SILU) xu[i] = Elem<T>::zero();
+      }
     }
   };
   auto store_x = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < XLOADS; ++i) *reinterpret_cast<Frag*>(lds + buf * XSTAGE + x_dst[i]) = xg[i];
+    for (int i = 0; i < XLOADS; ++i)
+      *reinterpret_cast<Frag*>(lds + buf * XSTAGE + x_dst[i]) = SILU ? tw_silu_mul_frag<T>(xg[i], xu[i]) : xg[i];
   };
   auto multiply = [&](const int buf) {
 #pragma unroll
@@ -373,7 +392,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
     for (int j = 0; j < 4; ++j) {
       const int col = n0 + 4 * g + j;
       if (col >= N) continue;
-      if (splits > 1) {
+      if (PARTIAL || splits > 1) {
         partial[((size_t)split * M + row) * N + col] = acc[mt][j];
       } else {
         float v = acc[mt][j] + (bias ? bias[col] : 0.f);
@@ -498,7 +517,7 @@ static int launch_skinny_tw(const T* A, long lda, const T* W, long ldw, const fl
   return TW_LAUNCH_RESULT();
 }
 
-template <typename T, typename OutT, int MT>
+template <typename T, typename OutT, int MT, bool SILU, bool PARTIAL>
 static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const float* bias,
                              const float* residual, long ldr, OutT* C, long ldc, float* partial,
                              long partial_bytes, int M, int N, int K, hipStream_t stream) {
@@ -506,14 +525,28 @@ static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const f
   constexpr int U = MT == 1 ? 8 : 4;
   const int groups = tw_div_up(N, 64);
   int splits = skinny_lds_splits(N, K, EPF);
-  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) splits = 1;
-  gemm_skinny_lds_kernel<T, OutT, MT, U><<<groups * splits, 256, 0, stream>>>(
+  if (PARTIAL) {
+    TW_REQUIRE(partial != nullptr && partial_bytes >= (long)splits * M * N * 4);
+  } else if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) {
+    splits = 1;
+  }
+  gemm_skinny_lds_kernel<T, OutT, MT, U, SILU, PARTIAL><<<groups * splits, 256, 0, stream>>>(
       A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
   int err = TW_LAUNCH_RESULT();
-  if (err || splits == 1) return err;
+  if (err || splits == 1 || PARTIAL) return err;
   splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
                                                                              ldr, C, ldc, M, N);
   return TW_LAUNCH_RESULT();
+}
+
+template <typename T, typename OutT, bool SILU, bool PARTIAL>
+static int launch_skinny_lds_m(const T* A, long lda, const T* W, long ldw, const float* bias,
+                               const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                               long partial_bytes, int M, int N, int K, hipStream_t stream) {
+  if (M <= 16) return launch_skinny_lds<T, OutT, 1, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 32) return launch_skinny_lds<T, OutT, 2, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 48) return launch_skinny_lds<T, OutT, 3, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  return launch_skinny_lds<T, OutT, 4, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
 }
 
 template <typename T, typename OutT, int MT>
@@ -542,10 +575,7 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
   }
   if (force == 5 || (force == 0 && M <= 64)) {
     TW_REQUIRE(M <= 64);
-    if (M <= 16) return launch_skinny_lds<T, OutT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-    if (M <= 32) return launch_skinny_lds<T, OutT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-    if (M <= 48) return launch_skinny_lds<T, OutT, 3>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-    return launch_skinny_lds<T, OutT, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny_lds_m<T, OutT, false, false>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
   if (force == 2) {
     TW_REQUIRE(M <= 64);
@@ -578,6 +608,34 @@ extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const 
                                             (float*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
     return linear_dispatch<bf16_t, bf16_t>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, residual, ldr,
                                            (bf16_t*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
+  }
+  return TW_ERR_BAD_ARGUMENT;
+}
+
+// ---- decode-path forms: few rows, 16-byte aligned K ------------------------------------
+// Number of K ranges tw_linear_partials uses for an [N, K] weight (0: shape not supported).
+extern "C" int tw_linear_partial_splits(int dtype, int N, int K) {
+  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
+  if (K % epf) return 0;
+  return skinny_lds_splits(N, K, epf);
+}
+
+// partial[split][M][N] (float32) = A[:, K range of split] W[:, same]^T for every split; the caller's
+// next kernel adds the splits up (with bias, residual, norm or rotation as it needs).
+// silu != 0: A is [M][2K] = [gate | up] and silu(gate) * up stands in for the activations.
+extern "C" int tw_linear_partials(int dtype, int silu, const void* A, long lda, const void* W, long ldw,
+                                  float* partial, long partial_bytes, int M, int N, int K,
+                                  hipStream_t stream) {
+  TW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && ldw >= K && lda >= (silu ? 2L * K : (long)K));
+  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
+  TW_REQUIRE(K % epf == 0 && lda % epf == 0 && ldw % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
+  if (dtype == TW_DTYPE_F32) {
+    if (silu) return launch_skinny_lds_m<float, float, true, true>((const float*)A, lda, (const float*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny_lds_m<float, float, false, true>((const float*)A, lda, (const float*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+  }
+  if (dtype == TW_DTYPE_BF16) {
+    if (silu) return launch_skinny_lds_m<bf16_t, float, true, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny_lds_m<bf16_t, float, false, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
   }
   return TW_ERR_BAD_ARGUMENT;
 }

@@ -18,11 +18,13 @@ _SIGNATURES = {
     "tw_graph_launch": (I, [P, P]),
     "tw_graph_destroy": (I, [P]),
     "tw_embed_gather": (I, [I, P, P, P, I, I, I, P]),
-    "tw_rmsnorm": (I, [I, P, P, P, P, I, I, F, P, I, L, P]),
+    "tw_rmsnorm": (I, [I, P, P, P, P, I, I, F, P, I, L, P, P]),
     "tw_rope_table": (I, [P, P, P, P, I, I, P]),
-    "tw_rope_kv_write": (I, [I, P, L, P, P, P, P, P, I, I, I, I, I, I, I, P]),
+    "tw_rope_kv_write": (I, [I, P, L, P, P, P, P, P, I, I, I, I, I, I, I, P, I, P, P]),
     "tw_silu_mul": (I, [I, P, P, I, I, P]),
     "tw_linear_workspace_bytes": (L, [I, I, I, I]),
+    "tw_linear_partial_splits": (I, [I, I, I]),
+    "tw_linear_partials": (I, [I, I, P, L, P, L, P, L, I, I, I, P]),
     "tw_linear": (I, [I, I, P, L, P, L, P, P, L, P, L, P, L, I, I, I, I, P]),
     "tw_attn_decode_splits": (I, [I, I, I, I]),
     "tw_attn_decode_workspace_floats": (L, [I, I, I, I]),

@@ -56,11 +56,12 @@ def embed_gather(ids, table, out):
     return out
 
 
-def rmsnorm(x, weight, eps, out, rows=None, add=None):
+def rmsnorm(x, weight, eps, out, rows=None, add=None, row_scratch=None):
     """out = x * rsqrt(mean(x^2) + eps) * weight per row; x float32, weight float32.
 
     rows: int32 indices choosing the input row of each output row.
-    add: float32 [splits, n, hidden] partial sums first added into x (x is updated).
+    add: float32 [splits, n, hidden] partial sums first added to x. Without `rows`
+    x itself is updated; with `rows` the sums go to row_scratch [n_out, hidden].
     """
     _need(x.dim() == 2 and x.is_contiguous(), "rmsnorm input must be contiguous [n, hidden]")
     n, hidden = x.shape
@@ -68,15 +69,19 @@ def rmsnorm(x, weight, eps, out, rows=None, add=None):
     _need(out.is_contiguous() and tuple(out.shape) == (n_out, hidden), "rmsnorm output has the wrong shape")
     _need(weight.numel() == hidden, "rmsnorm weight has the wrong size")
     add_ptr, splits, stride = None, 0, 0
+    scratch_ptr = None
     if add is not None:
-        _need(rows is None, "rmsnorm cannot gather rows and add partial sums at once")
         _need(add.dim() == 3 and add.is_contiguous() and tuple(add.shape[1:]) == (n, hidden),
               "rmsnorm partial sums must be [splits, n, hidden]")
         add_ptr, splits, stride = _dev(add, torch.float32, "add"), add.shape[0], n * hidden
+        if rows is not None:
+            _need(row_scratch is not None and row_scratch.is_contiguous()
+                  and tuple(row_scratch.shape) == (n_out, hidden), "rmsnorm with rows and partial sums needs row_scratch [n_out, hidden]")
+            scratch_ptr = _dev(row_scratch, torch.float32, "row_scratch")
     check(library().tw_rmsnorm(dtype_id(out.dtype), _dev(x, torch.float32, "x"),
                                _dev(weight, torch.float32, "weight"), _dev(out),
                                _dev(rows, torch.int32, "rows") if rows is not None else None,
-                               n_out, hidden, float(eps), add_ptr, splits, stride, _stream()), "rmsnorm")
+                               n_out, hidden, float(eps), add_ptr, splits, stride, scratch_ptr, _stream()), "rmsnorm")
     return out
 
 
@@ -92,11 +97,13 @@ def rope_table(positions, inv_freq, cos, sin):
 
 
 def rope_kv_write(qkv, cos, sin, slots, keys, values, q_heads, kv_heads, head_dim, page_size,
-                  write_cache=True):
+                  write_cache=True, partial=None, bias=None):
     """Rotate q (in place) and k of qkv[n] = [q | k | v]; write rotated k and v to the pages.
 
     keys [pages, kv_heads, page_size, head_dim]; values hold the same number of
     elements and are written as [pages, kv_heads, head_dim, page_size].
+    partial: float32 [splits, n, width] split-K sums of the projection; qkv is then
+    first filled with round(sum of the splits + bias).
     """
     n, width, ld = _rows(qkv, "qkv")
     _need(width == (q_heads + 2 * kv_heads) * head_dim, "qkv width does not match the head counts")
@@ -112,13 +119,21 @@ def rope_kv_write(qkv, cos, sin, slots, keys, values, q_heads, kv_heads, head_di
         _need(tuple(keys.shape[1:]) == (kv_heads, page_size, head_dim), "keys must be [pages, kv_heads, page_size, head_dim]")
         _need(values.numel() == keys.numel(), "keys and values differ in size")
         _need(slots.numel() == n, "one cache slot per token is needed")
+    if partial is not None:
+        _need(partial.dim() == 3 and partial.is_contiguous() and tuple(partial.shape[1:]) == (n, width),
+              "projection partial sums must be [splits, n, width]")
+        _need(bias is None or bias.numel() == width, "bias has the wrong size")
     dummy = qkv
     check(library().tw_rope_kv_write(
         dtype_id(qkv.dtype), _dev(qkv), ld,
         _dev(cos, torch.float32, "cos") if rot else _dev(dummy), _dev(sin, torch.float32, "sin") if rot else _dev(dummy),
         _dev(slots, torch.int32, "slots") if write_cache else None,
         _dev(keys) if write_cache else None, _dev(values) if write_cache else None,
-        n, q_heads, kv_heads, head_dim, rot, page_size, 1 if write_cache else 0, _stream()), "rope_kv_write")
+        n, q_heads, kv_heads, head_dim, rot, page_size, 1 if write_cache else 0,
+        _dev(partial, torch.float32, "partial") if partial is not None else None,
+        partial.shape[0] if partial is not None else 0,
+        _dev(bias, torch.float32, "bias") if (partial is not None and bias is not None) else None,
+        _stream()), "rope_kv_write")
 
 
 def silu_mul(gate_up, out):
@@ -133,6 +148,30 @@ def silu_mul(gate_up, out):
 
 def linear_workspace_bytes(dtype, max_rows, n, k):
     return int(library().tw_linear_workspace_bytes(dtype_id(dtype), int(max_rows), int(n), int(k)))
+
+
+def linear_partial_splits(dtype, n, k):
+    """K ranges `linear_partials` uses for an [n, k] weight; 0 if the shape is not supported."""
+    return int(library().tw_linear_partial_splits(dtype_id(dtype), int(n), int(k)))
+
+
+def linear_partials(x, weight, partial, silu_gate=False):
+    """partial[s] = x[:, K range s] @ weight[:, K range s].T in float32, for at most 64 rows.
+
+    The caller's next kernel adds the splits up. silu_gate: x is [m, 2k] = [gate | up] and
+    silu(gate) * up (rounded to x's type) stands in for the activations.
+    """
+    m, kx, lda = _rows(x, "x")
+    n, k, ldw = _rows(weight, "weight")
+    _need(kx == (2 * k if silu_gate else k), "linear_partials shapes do not agree")
+    _need(x.dtype == weight.dtype and 1 <= m <= 64, "linear_partials takes 1..64 rows of the weight's type")
+    splits = linear_partial_splits(weight.dtype, n, k)
+    _need(splits > 0, "linear_partials needs K to be a multiple of 16 bytes")
+    _need(partial.is_contiguous() and tuple(partial.shape) == (splits, m, n), f"partial must be [{splits}, {m}, {n}]")
+    check(library().tw_linear_partials(dtype_id(x.dtype), 1 if silu_gate else 0, _dev(x), lda, _dev(weight), ldw,
+                                       _dev(partial, torch.float32, "partial"), partial.numel() * 4, m, n, k,
+                                       _stream()), "linear_partials")
+    return partial
 
 
 GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY_COOP = 0, 1, 2, 3, 4, 5

@@ -1,5 +1,5 @@
 from .base import (Block, FeedForward, GroupStep, LayerRun, Mixer, Norm, Part, PositionEncoding,
-                   StepContext, Workspace)
+                   StepContext, Workspace, fold_pending)
 from .linear import Linear
 from .norms import RMSNorm
 from .positions import NoPositionEncoding, RotaryEmbedding
@@ -10,6 +10,6 @@ from .embedding import OutputHead, TokenEmbedding
 from .model import DecoderModel, walk
 
 __all__ = ["Block", "FeedForward", "GroupStep", "LayerRun", "Mixer", "Norm", "Part", "PositionEncoding",
-           "StepContext", "Workspace", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEmbedding",
+           "StepContext", "Workspace", "fold_pending", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEmbedding",
            "GroupedQueryAttention", "SwiGLU", "PreNormBlock", "OutputHead", "TokenEmbedding",
            "DecoderModel", "walk"]

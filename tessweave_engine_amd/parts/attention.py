@@ -52,12 +52,19 @@ class GroupedQueryAttention(Mixer):
         n = ctx.n_tokens
         width = (self.q_heads + 2 * self.kv_heads) * self.head_dim
         qkv = ctx.scratch("attn.qkv", (n, width))
-        self.qkv.forward(ctx, h, qkv)
         cos, sin = self.position.tables(ctx)
         keys, values, g = ctx.cache.keys_values(run.cache_slot)
         group = ctx.groups[g]
-        ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
-                          self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache)
+        if self.qkv.deferrable(n):
+            # few rows: the projection leaves split-K sums; bias, rotation and cache write finish them
+            partial = self.qkv.forward_partials(ctx, h, "qkv")
+            ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
+                              self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache,
+                              partial=partial, bias=self.qkv.biases[0] if self.qkv.biases else None)
+        else:
+            self.qkv.forward(ctx, h, qkv)
+            ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
+                              self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache)
         out = ctx.scratch("attn.out", (n, self.q_heads * self.head_dim))
         window = self.window or 0
         if ctx.n_decode:
@@ -77,4 +84,7 @@ class GroupedQueryAttention(Mixer):
             ops.attn_prefill(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode,
                              ctx.n_seqs - ctx.n_decode, ctx.max_q_len, out, self.q_heads, self.kv_heads,
                              self.head_dim, self.scale, window=window)
+        if not self.o.biases and self.o.deferrable(n):
+            return self.o.forward_partials(ctx, out, "o")          # the next norm adds them into x
         self.o.forward(ctx, out, x, residual=x)
+        return None

@@ -50,7 +50,11 @@ class Part:
 
 class Norm(Part):
     def forward(self, ctx, x, rows=None, add=None):
-        """x float32 [n, hidden] -> normalised rows in the compute type."""
+        """x float32 [n, hidden] -> normalised rows in the compute type.
+
+        add: pending partial sums (float32 [splits, n, hidden]) of the part before, to be
+        added into x first (see `Mixer.forward`). rows: int32 indices of the rows wanted.
+        """
         raise NotImplementedError
 
 
@@ -69,21 +73,36 @@ class Mixer(Part):
         return None
 
     def forward(self, ctx, run, h, x):
-        """Add the mixer's output for normalised input H into the residual stream X (float32, in place)."""
+        """Add the mixer's output for normalised input H into the residual stream X (float32, in place).
+
+        Returns None, or PENDING partial sums (float32 [splits, n, hidden]) that are not yet in X:
+        whoever runs next (the following norm) adds them up and into X. This saves a kernel per
+        projection when a step has few rows.
+        """
         raise NotImplementedError
 
 
 class FeedForward(Part):
     def forward(self, ctx, h, x):
-        """Add the feed-forward's output for normalised input H into X (float32, in place)."""
+        """Add the feed-forward's output for normalised input H into X (float32, in place);
+        returns None or pending partial sums as `Mixer.forward` does."""
         raise NotImplementedError
 
 
 class Block(Part):
     mixer: Mixer
 
-    def forward(self, ctx, run, x):
+    def forward(self, ctx, run, x, pending=None):
+        """Run the block on X in place. PENDING: partial sums the block before left to be added
+        into X; returns what this block leaves pending (or None)."""
         raise NotImplementedError
+
+
+def fold_pending(x, pending):
+    """Add pending partial sums into X with plain tensor operations (for parts written in torch)."""
+    if pending is not None:
+        x += pending.sum(0)
+    return None
 
 
 class Workspace:

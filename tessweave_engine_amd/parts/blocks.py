@@ -21,8 +21,8 @@ class PreNormBlock(Block):
         for p in self.parts():
             p.bind(tensors, dtype, device)
 
-    def forward(self, ctx, run, x):
-        h = self.mixer_norm.forward(ctx, x)
-        self.mixer.forward(ctx, run, h, x)
-        h = self.ffn_norm.forward(ctx, x)
-        self.ffn.forward(ctx, h, x)
+    def forward(self, ctx, run, x, pending=None):
+        h = self.mixer_norm.forward(ctx, x, add=pending)
+        pending = self.mixer.forward(ctx, run, h, x)
+        h = self.ffn_norm.forward(ctx, x, add=pending)
+        return self.ffn.forward(ctx, h, x)

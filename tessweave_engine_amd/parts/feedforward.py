@@ -27,6 +27,11 @@ class SwiGLU(FeedForward):
         n = h.shape[0]
         gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
         self.gate_up.forward(ctx, h, gu)
+        if self.down.deferrable(n):
+            # few rows: silu(gate) * up is formed while the down projection stages its input,
+            # and its split-K sums are left to the next norm
+            return self.down.forward_partials(ctx, gu, "down", silu_gate=True)
         act = ctx.scratch("ffn.act", (n, self.intermediate))
         ops.silu_mul(gu, act)
         self.down.forward(ctx, act, x, residual=x)
+        return None

@@ -71,3 +71,21 @@ class Linear(Part):
             ops.linear(x, w, target, bias=self.biases[i] if self.biases else None, residual=res, workspace=ws)
             col += rows
         return out
+
+    # ---- few rows: leave the split-K sums to the next kernel --------------------------------
+    def deferrable(self, n_rows):
+        """Can `forward_partials` run for N_ROWS rows? (one packed matrix, no bias of its own to add)"""
+        if len(self.weights) != 1 or not 1 <= n_rows <= 64:
+            return False
+        w = self.weights[0]
+        if "splits" not in self._ws_floats:
+            self._ws_floats["splits"] = ops.linear_partial_splits(w.dtype, w.shape[0], w.shape[1])
+        return self._ws_floats["splits"] > 0
+
+    def forward_partials(self, ctx, x, tag, silu_gate=False):
+        """float32 [splits, n, out] partial sums of x @ W.T (bias NOT added); see ops.linear_partials."""
+        w = self.weights[0]
+        splits = self._ws_floats["splits"]
+        buf = ctx.workspace.get("linear.partial." + tag, (splits, 64, w.shape[0]), torch.float32)
+        partial = buf.view(-1)[:splits * x.shape[0] * w.shape[0]].view(splits, x.shape[0], w.shape[0])
+        return ops.linear_partials(x, w, partial, silu_gate=silu_gate)

@@ -27,4 +27,8 @@ class RMSNorm(Norm):
     def forward(self, ctx, x, rows=None, add=None, tag="norm.out"):
         n_out = rows.numel() if rows is not None else x.shape[0]
         out = ctx.scratch(tag, (n_out, self.size))
-        return ops.rmsnorm(x, self.weight, self.eps, out, rows=rows, add=add)
+        scratch = None
+        if add is not None and rows is not None:
+            import torch
+            scratch = ctx.scratch(tag + ".rows", (n_out, self.size), torch.float32)
+        return ops.rmsnorm(x, self.weight, self.eps, out, rows=rows, add=add, row_scratch=scratch)

@@ -149,7 +149,7 @@ class PartHarness:
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_each_part_alone(tiny, dtype):
     from tessweave_engine_amd.engine import StepEntry
-    from tessweave_engine_amd.parts import LayerRun
+    from tessweave_engine_amd.parts import LayerRun, fold_pending
     from tessweave_engine_amd.weights import load_model
     model = load_model(tiny["folder"], dtype=dtype, device="cuda:0")
     torch_dtype = model.dtype
@@ -181,20 +181,20 @@ def test_each_part_alone(tiny, dtype):
         # mixer: adds attention of the normalised input into the residual stream
         h_in = want_h.to(torch_dtype)
         xr = xd.clone()
-        block.mixer.forward(ctx, LayerRun(0, 0), h_in.to("cuda"), xr)
+        fold_pending(xr, block.mixer.forward(ctx, LayerRun(0, 0), h_in.to("cuda"), xr))
         want_x = x0.clone()
         want_x[:11] += plain.attention_block(h_in.float()[:11], torch.arange(11), w, "model.layers.0.self_attn.", s)
         want_x[11:] += plain.attention_block(h_in.float()[11:], torch.arange(6), w, "model.layers.0.self_attn.", s)
         torch.testing.assert_close(xr.cpu(), want_x, **tight)
         # feed-forward
         xf = xd.clone()
-        block.ffn.forward(ctx, h_in.to("cuda"), xf)
+        fold_pending(xf, block.ffn.forward(ctx, h_in.to("cuda"), xf))
         p = "model.layers.0.mlp."
         want_f = x0 + plain.swiglu(h_in.float(), w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
         torch.testing.assert_close(xf.cpu(), want_f, **tight)
         # whole block
         xb = xd.clone()
-        block.forward(ctx, LayerRun(0, 0), xb)
+        fold_pending(xb, block.forward(ctx, LayerRun(0, 0), xb))
         want_b = torch.cat([plain.decoder_layer(x0[:11], torch.arange(11), w, 0, s),
                             plain.decoder_layer(x0[11:], torch.arange(6), w, 0, s)])
         torch.testing.assert_close(xb.cpu(), want_b, **(tight if dtype == "float32" else dict(atol=6e-2, rtol=6e-2)))

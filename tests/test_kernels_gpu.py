@@ -59,6 +59,14 @@ def test_rmsnorm(ops, device, dtype, hidden, eps):
     torch.testing.assert_close(x2.cpu(), total.float(), atol=1e-5, rtol=1e-6)
     want3 = plain.rms_norm(total, w.cpu().double(), eps).float()
     torch.testing.assert_close(out3.float().cpu(), want3, **tol(dtype, (3e-6, 3e-6), (1e-2, 1e-2)))
+    # gathered rows AND partial sums (a row may be named twice): x itself stays as it was
+    rows2 = torch.tensor([6, 0, 6], dtype=torch.int32, device=device)
+    x3 = x.clone()
+    out4 = torch.empty(3, hidden, dtype=dtype, device=device)
+    scratch = torch.empty(3, hidden, dtype=torch.float32, device=device)
+    ops.rmsnorm(x3, w, eps, out4, rows=rows2, add=add, row_scratch=scratch)
+    torch.testing.assert_close(x3, x, atol=0, rtol=0)
+    torch.testing.assert_close(out4, out3[rows2.long()], atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -103,6 +111,20 @@ def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, p
     assert torch.isnan(kflat[~written]).all()
     vflat = vc.permute(0, 3, 1, 2).reshape(pages * page, -1)
     assert torch.isnan(vflat[~written]).all()
+    # the same from split-K partial sums plus bias: identical bits
+    bias = rand((width,), torch.float32, device, 0.3, seed=9)
+    parts = rand((3, n, width), torch.float32, device, 1.0, seed=10)
+    summed = ((parts[0] + parts[1] + parts[2]) + bias).to(dtype)
+    keys2, values2 = torch.zeros_like(keys), torch.zeros_like(values)
+    ops.rope_kv_write(summed.clone(), cos, sin, slots, keys2, values2, q_heads, kv_heads, head_dim, page)
+    qkv3 = torch.full((n, width), float("nan"), dtype=dtype, device=device)
+    keys3, values3 = torch.zeros_like(keys), torch.zeros_like(values)
+    ops.rope_kv_write(qkv3, cos, sin, slots, keys3, values3, q_heads, kv_heads, head_dim, page, partial=parts, bias=bias)
+    torch.testing.assert_close(keys3, keys2, atol=0, rtol=0)
+    torch.testing.assert_close(values3, values2, atol=0, rtol=0)
+    ref = summed.clone()
+    ops.rope_kv_write(ref, cos, sin, slots, torch.zeros_like(keys), torch.zeros_like(values), q_heads, kv_heads, head_dim, page)
+    torch.testing.assert_close(qkv3[:, :q_heads * head_dim], ref[:, :q_heads * head_dim], atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -151,6 +173,27 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
         ops.linear(x, w, out2, bias=bias, force=force)
         torch.testing.assert_close(out2.double().cpu(), want + bias.double().cpu(),
                                    atol=t["atol"] if dtype == torch.float32 else 2e-5 * scale + 1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 389, 2048), (17, 130, 4096), (64, 96, 9472)])
+def test_linear_partials_and_fused_silu(ops, device, dtype, m, n, k):
+    x = rand((m, k), dtype, device, 1.0, seed=1)
+    w = rand((n, k), dtype, device, 0.05, seed=2)
+    splits = ops.linear_partial_splits(dtype, n, k)
+    part = torch.full((splits, m, n), float("nan"), device=device)
+    ops.linear_partials(x, w, part)
+    want = x.double().cpu() @ w.double().cpu().T
+    scale = math.sqrt(k) * 0.05
+    torch.testing.assert_close(part.double().sum(0).cpu(), want, atol=3e-5 * scale, rtol=1e-5)
+    # [gate | up] input: silu(gate) * up, rounded to the input type, is what gets multiplied
+    gu = rand((m, 2 * k), dtype, device, 1.0, seed=3)
+    act = torch.empty(m, k, dtype=dtype, device=device)
+    ops.silu_mul(gu, act)
+    ops.linear_partials(act, w, part)
+    plain_sum = part.sum(0).clone()
+    ops.linear_partials(gu, w, part, silu_gate=True)
+    torch.testing.assert_close(part.sum(0), plain_sum, atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
