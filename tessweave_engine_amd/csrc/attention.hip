@@ -557,6 +557,310 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 }
 
 // =====================================================================================
+// Prefill, bfloat16, pages of 8 keys or a power of two above: a workgroup of 4
+// waves owns 128 consecutive (token, head) rows of one kv head, 32 per wave. The
+// keys and values of each 32-key block are copied ONCE per workgroup into LDS
+// (keys outside the sequence as zeros) while the block before is computed; every
+// K or V fragment a wave reads from LDS serves both of its 16-row tiles.
+// Key/row layout inside a block as in the decode kernel above.
+// =====================================================================================
+#define TW_PF_VROW 80                       /* LDS bytes per value row (32 keys = 64 B, padded) */
+
+template <bool V> struct BoolTag { static constexpr bool value = V; };
+
+template <int DTMAX>
+__global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
+  constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
+  constexpr int KROW = DTMAX * 32 + 16;                 // LDS bytes per key row, padded
+  constexpr int KSTAGE = 32 * KROW, VSTAGE = DTMAX * 16 * TW_PF_VROW;
+  constexpr int KPIECES = (32 * DTMAX * 2 + 255) / 256;  // 16-byte pieces per thread per block
+  constexpr int VPIECES = (DTMAX * 16 * 4 + 255) / 256;
+  constexpr int CH = DTMAX * 2;                          // 16-byte chunks per key row of this size class
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* lds_k = lds;
+  char* lds_v = lds + 2 * KSTAGE;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int G = a.q_heads / a.kv_heads;
+  const int kvh = blockIdx.y;
+  const int seq = a.seq0 + blockIdx.z;
+  const int kv_len = a.kv_len[seq];
+  const int token0 = a.q_start[seq];
+  const int q_len = a.q_start[seq + 1] - token0;
+  const int rows = q_len * G;
+  // the tiles that see the most keys start first
+  const int n_tiles = (rows + 127) / 128;
+  if ((int)blockIdx.x >= n_tiles) return;
+  const int wg_row0 = (n_tiles - 1 - blockIdx.x) * 128;
+  const int* table = a.block_table + (size_t)seq * a.table_stride;
+  const int D = a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
+  const int pshift = a.page_shift, pmask = P - 1;
+  const int ppb = P >= 32 ? 1 : (32 >> pshift);
+  const unsigned head_stride = (unsigned)P * D;
+  const bf16_t* keys = (const bf16_t*)a.keys;
+  const bf16_t* values = (const bf16_t*)a.values;
+  const int first_pos = kv_len - q_len;
+  const bool whole_chunks = (chunks & 3) == 0;           // head_dim a multiple of 32: no partial MFMA step
+  const float c2 = a.scale * 1.44269504088896340736f;    // scores are kept in the log2 domain
+
+  // ---- this wave's two row tiles -----------------------------------------------
+  bf16x8 qf[2][NSMAX];
+  int t_row[2], tok[2], head[2];
+  bool row_ok[2];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int row = wg_row0 + wave * 32 + rt * 16 + r;
+    row_ok[rt] = row < rows;
+    tok[rt] = row / G;
+    head[rt] = kvh * G + row % G;
+    t_row[rt] = row_ok[rt] ? first_pos + tok[rt] : -1;
+    const bf16_t* q_row = (const bf16_t*)a.q + (size_t)(token0 + tok[rt]) * a.ldq + (size_t)head[rt] * D;
+#pragma unroll
+    for (int st = 0; st < NSMAX; ++st) {
+      const int chunk = st * 4 + g;
+      qf[rt][st] = (row_ok[rt] && chunk < chunks) ? tw_load_frag(q_row + chunk * 8) : Elem<bf16_t>::zero();
+    }
+  }
+  f32x4 acc[2][DTMAX];
+  float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt) acc[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- the workgroup's key range ------------------------------------------------
+  const int t_min = first_pos + wg_row0 / G;
+  const int t_max = first_pos + min(rows - 1, wg_row0 + 127) / G;
+  const int lo = a.window > 0 ? max(0, t_min - a.window + 1) : 0;       // keys below are never loaded
+  const int blk_begin = lo / 32, blk_end = t_max / 32 + 1;
+  const int wave_t_max = first_pos + min(rows - 1, wg_row0 + wave * 32 + 31) / G;
+  const int wave_t_min = first_pos + min(rows - 1, wg_row0 + wave * 32) / G;
+  const bool wave_live = wg_row0 + wave * 32 < rows;
+  const bool wave_full = wg_row0 + wave * 32 + 32 <= rows;
+  const int wave_lo_max = a.window > 0 ? wave_t_max - a.window + 1 : 0;  // largest lower bound among the wave's rows
+
+  // This thread's share of a block, fixed for the whole loop: K piece i is 16 bytes
+  // (chunk k_chunk) of key k_key; V piece i is keys 8*v_oct .. +7 of output dim v_d.
+  bf16x8 kreg[KPIECES], vreg[VPIECES];
+  int k_key[KPIECES], k_goff[KPIECES], k_loff[KPIECES], k_slot[KPIECES];
+  int v_oct[VPIECES], v_goff[VPIECES], v_loff[VPIECES], v_slot[VPIECES];
+  bool k_use[KPIECES], v_use[VPIECES];
+#pragma unroll
+  for (int i = 0; i < KPIECES; ++i) {
+    const int q = tid + i * 256, key = q / CH, chunk = q % CH;
+    k_use[i] = key < 32 && chunk < chunks;
+    k_key[i] = key;
+    k_slot[i] = P >= 32 ? 0 : (key >> pshift);             // which of the block's pages
+    k_goff[i] = (P >= 32 ? key : (key & pmask)) * D + chunk * 8;
+    k_loff[i] = key * KROW + chunk * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < VPIECES; ++i) {
+    const int q = tid + i * 256, d = q >> 2, oct = q & 3;
+    v_use[i] = d < D;
+    v_oct[i] = oct;
+    v_slot[i] = P >= 32 ? 0 : ((8 * oct) >> pshift);
+    v_goff[i] = d * P + (P >= 32 ? 8 * oct : ((8 * oct) & pmask));
+    v_loff[i] = d * TW_PF_VROW + oct * 16;
+  }
+  auto fetch = [&](int blk_v) {                              // global -> registers
+    const int blk = __builtin_amdgcn_readfirstlane(blk_v);
+    const int p0 = blk * 32;
+    const int first = p0 >> pshift;
+    int pg[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pg[i] = (i < ppb && p0 + (i << pshift) < kv_len) ? table[first + i] : -1;
+    const int in_page = P >= 32 ? (p0 & pmask) : 0;          // where the block starts inside its page
+    if (p0 >= lo && p0 + 32 <= kv_len && pg[0] >= 0 && (ppb < 2 || pg[1] >= 0) && (ppb < 4 || (pg[2] >= 0 && pg[3] >= 0))) {
+      // every key of the block is inside the sequence: no predicates, page bases in scalar registers
+      size_t kb[4], vb[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const size_t base = ((size_t)(i < ppb ? pg[i] : pg[0]) * a.kv_heads + kvh) * head_stride;
+        kb[i] = base + (size_t)in_page * D;
+        vb[i] = base + in_page;
+      }
+#pragma unroll
+      for (int i = 0; i < KPIECES; ++i) {
+        const int sl = k_slot[i];
+        const size_t base = sl == 0 ? kb[0] : (sl == 1 ? kb[1] : (sl == 2 ? kb[2] : kb[3]));
+        if (k_use[i]) kreg[i] = tw_load_frag(keys + base + k_goff[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < VPIECES; ++i) {
+        const int sl = v_slot[i];
+        const size_t base = sl == 0 ? vb[0] : (sl == 1 ? vb[1] : (sl == 2 ? vb[2] : vb[3]));
+        if (v_use[i]) vreg[i] = tw_load_frag(values + base + v_goff[i]);
+      }
+      return;
+    }
+    // a block at the edge of the sequence: keys outside it are loaded as zeros
+    auto page_of = [&](int ko) {
+      const int i = P >= 32 ? 0 : (ko >> pshift);
+      return i == 0 ? pg[0] : (i == 1 ? pg[1] : (i == 2 ? pg[2] : pg[3]));
+    };
+#pragma unroll
+    for (int i = 0; i < KPIECES; ++i) {
+      const int p = p0 + k_key[i];
+      int page = k_use[i] ? page_of(k_key[i]) : -1;
+      if (p >= kv_len || p < lo) page = -1;
+      const size_t base = ((size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh) * head_stride;
+      kreg[i] = page >= 0 ? tw_load_frag(keys + base + (unsigned)(p & pmask) * D + (k_loff[i] - k_key[i] * KROW) / 2)
+                          : Elem<bf16_t>::zero();
+    }
+#pragma unroll
+    for (int i = 0; i < VPIECES; ++i) {
+      const int p = p0 + 8 * v_oct[i];
+      int page = v_use[i] ? page_of(8 * v_oct[i]) : -1;
+      if (p >= kv_len || p + 7 < lo) page = -1;
+      const size_t base = ((size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh) * head_stride;
+      const int d = (v_loff[i] - v_oct[i] * 16) / TW_PF_VROW;
+      bf16x8 v = page >= 0 ? tw_load_frag(values + base + (unsigned)d * P + (p & pmask)) : Elem<bf16_t>::zero();
+      if (page >= 0 && (p + 8 > kv_len || p < lo)) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (p + e >= kv_len || p + e < lo) v[e] = (bf16_t)0.f;
+      }
+      vreg[i] = v;
+    }
+  };
+  auto stash = [&](int buf) {                                // registers -> LDS
+#pragma unroll
+    for (int i = 0; i < KPIECES; ++i)
+      if (k_use[i]) *reinterpret_cast<bf16x8*>(lds_k + buf * KSTAGE + k_loff[i]) = kreg[i];
+#pragma unroll
+    for (int i = 0; i < VPIECES; ++i)
+      if (v_use[i]) *reinterpret_cast<bf16x8*>(lds_v + buf * VSTAGE + v_loff[i]) = vreg[i];
+  };
+
+  // LDS addresses of this lane's fragments in stage 0
+  const char* k_frag[2];
+#pragma unroll
+  for (int tile = 0; tile < 2; ++tile)
+    k_frag[tile] = lds_k + (8 * (r >> 2) + 4 * tile + (r & 3)) * KROW + g * 16;
+  const char* v_frag = lds_v + r * TW_PF_VROW + g * 16;
+
+  // EDGE false: every key of the block is visible to every row of the wave (no masks).
+  auto compute = [&](int blk, int buf, auto edge_tag) {
+    constexpr bool EDGE = decltype(edge_tag)::value;
+    const int p0 = blk * 32;
+    f32x4 s[2][2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+      for (int tile = 0; tile < 2; ++tile) s[rt][tile] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+      const char* base = k_frag[tile] + buf * KSTAGE;
+#pragma unroll
+      for (int st = 0; st < NSMAX; ++st)
+        if (st * 4 < chunks) {
+          bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + st * 64);
+          if (!whole_chunks && st * 4 + g >= chunks) kf = Elem<bf16_t>::zero();
+          tw_mma16(s[0][tile], kf, qf[0][st]);
+          tw_mma16(s[1][tile], kf, qf[1][st]);
+        }
+    }
+    bf16x8 pb[2];
+    float alpha[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+      float x[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        x[e] = s[rt][e >> 2][e & 3] * c2;
+        if (EDGE) {
+          const int p = p0 + 8 * g + e;
+          const int lo_row = a.window > 0 ? t_row[rt] - a.window + 1 : 0;
+          if (!(p <= t_row[rt] && p >= lo_row && p < kv_len)) x[e] = -INFINITY;
+        }
+        mx = fmaxf(mx, x[e]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
+      const float m_new = fmaxf(m[rt], mx);
+      const float m_use = (EDGE && m_new == -INFINITY) ? 0.f : m_new;
+      alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - m_use);
+      float sum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pe = __builtin_amdgcn_exp2f(x[e] - m_use);
+        sum += pe;
+        pb[rt][e] = (bf16_t)pe;
+      }
+      sum += __shfl_xor(sum, 16, TW_WAVE);
+      sum += __shfl_xor(sum, 32, TW_WAVE);
+      l[rt] = l[rt] * alpha[rt] + sum;
+      m[rt] = m_new;
+    }
+    // rescale the running output only if some row's maximum moved
+    const bool moved = __any(alpha[0] != 1.f || alpha[1] != 1.f);
+    const char* vbase = v_frag + buf * VSTAGE;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+          if (moved) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[rt][dt][j] *= alpha[rt];
+          }
+          tw_mma16(acc[rt][dt], vf, pb[rt]);
+        }
+      }
+  };
+
+  fetch(blk_begin);
+  stash(0);
+  __syncthreads();
+  for (int blk = blk_begin; blk < blk_end; ++blk) {
+    const int buf = (blk - blk_begin) & 1;
+    if (blk + 1 < blk_end) fetch(blk + 1);
+    if (wave_live && blk * 32 <= wave_t_max) {
+      const int p0 = blk * 32;
+      if (wave_full && p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len)
+        compute(blk, buf, BoolTag<false>());
+      else
+        compute(blk, buf, BoolTag<true>());
+    }
+    if (blk + 1 < blk_end) stash(buf ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    if (!row_ok[rt]) continue;
+    const float inv = l[rt] > 0.f ? 1.f / l[rt] : 0.f;
+    bf16_t* dst = (bf16_t*)a.out + (size_t)(token0 + tok[rt]) * a.ldo + (size_t)head[rt] * D;
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (dt < dts)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = (bf16_t)(acc[rt][dt][j] * inv);
+  }
+}
+
+template <int DTMAX>
+static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
+  const int G = a.q_heads / a.kv_heads;
+  const long rows = (long)max_q_len * G;
+  dim3 grid(tw_div_up(rows, 128), a.kv_heads, n_seqs);
+  const size_t lds_bytes = 2 * 32 * (DTMAX * 32 + 16) + 2 * DTMAX * 16 * TW_PF_VROW;
+  auto kernel = attn_prefill_bf16_kernel<DTMAX>;
+  static bool attribute_set = false;
+  if (!attribute_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    attribute_set = true;
+  }
+  kernel<<<grid, 256, lds_bytes, stream>>>(a);
+  return TW_LAUNCH_RESULT();
+}
+
+// =====================================================================================
 // Host side
 // =====================================================================================
 static int check_common(const AttnArgs& a) {
@@ -644,7 +948,12 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
 }
 
 template <typename T>
-static int prefill_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
+static int prefill_launch(AttnArgs a, int n_seqs, int max_q_len, int generic, hipStream_t stream) {
+  if (IsBf16<T>::value && a.page_shift >= 3 && !generic) {
+    if (a.head_dim <= 64) return prefill_bf16_launch<4>(a, n_seqs, max_q_len, stream);
+    if (a.head_dim <= 128) return prefill_bf16_launch<8>(a, n_seqs, max_q_len, stream);
+    return prefill_bf16_launch<16>(a, n_seqs, max_q_len, stream);
+  }
   const int G = a.q_heads / a.kv_heads;
   const long rows = (long)max_q_len * G;
   dim3 grid(tw_div_up(rows, 64), a.kv_heads, n_seqs);
@@ -662,7 +971,7 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
                                const int* block_table, int table_stride, const int* q_start,
                                const int* kv_len, int seq0, int n_seqs, int max_q_len, void* out,
                                long ldo, int q_heads, int kv_heads, int head_dim, int page_size,
-                               int window, float scale, hipStream_t stream) {
+                               int window, float scale, int generic, hipStream_t stream) {
   AttnArgs a;
   a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
   a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
@@ -676,7 +985,7 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
   if (err) return err;
   TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && max_q_len >= 1 && n_seqs <= 65535);
   if (n_seqs == 0) return 0;
-  if (dtype == TW_DTYPE_F32) return prefill_launch<float>(a, n_seqs, max_q_len, stream);
-  if (dtype == TW_DTYPE_BF16) return prefill_launch<bf16_t>(a, n_seqs, max_q_len, stream);
+  if (dtype == TW_DTYPE_F32) return prefill_launch<float>(a, n_seqs, max_q_len, generic, stream);
+  if (dtype == TW_DTYPE_BF16) return prefill_launch<bf16_t>(a, n_seqs, max_q_len, generic, stream);
   return TW_ERR_BAD_ARGUMENT;
 }

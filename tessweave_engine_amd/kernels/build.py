@@ -22,8 +22,12 @@ CSRC = Path(__file__).resolve().parent.parent / "csrc"
 ARCH = "gfx950"
 # Packed float32 instructions are switched off: some of their forms have given
 # wrong results on this hardware generation.
+# MFMA results are kept in ordinary vector registers: with the default heuristic the
+# compiler parks accumulators in AGPRs and moves them to VGPRs and back around every
+# float32 operation on them (the online-softmax rescale), hundreds of moves per block.
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value",
+         "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 
 def sources():

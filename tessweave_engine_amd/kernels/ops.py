@@ -256,7 +256,7 @@ def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out
 
 
 def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_q_len, out, q_heads,
-                 kv_heads, head_dim, scale, window=0):
+                 kv_heads, head_dim, scale, window=0, generic=False):
     """Attention of sequences seq0..seq0+n_seqs-1 with up to max_q_len query tokens each."""
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
@@ -264,7 +264,8 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
                                     _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
                                     _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
                                     seq0, n_seqs, int(max_q_len), _dev(out), ldo, q_heads, kv_heads, head_dim,
-                                    keys.shape[2], int(window or 0), float(scale), _stream()), "attn_prefill")
+                                    keys.shape[2], int(window or 0), float(scale), 1 if generic else 0,
+                                    _stream()), "attn_prefill")
     return out
 
 

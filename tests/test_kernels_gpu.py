@@ -315,11 +315,12 @@ def test_attn_prefill_portions(ops, device, dtype, heads, kv_heads, head_dim, pa
     # q lives inside a wider qkv buffer
     buf = torch.zeros(total_q, (heads + 2 * kv_heads) * head_dim, dtype=dtype, device=device)
     buf[:, :heads * head_dim] = q.reshape(total_q, -1).to(device)
-    out = torch.full((total_q, heads * head_dim), float("nan"), dtype=dtype, device=device)
-    ops.attn_prefill(buf, keys, values, table, torch.tensor(q_start, dtype=torch.int32, device=device),
-                     torch.tensor(lengths, dtype=torch.int32, device=device), 0, len(cases), max(c[1] for c in cases),
-                     out, heads, kv_heads, head_dim, head_dim ** -0.5, window=window)
-    torch.testing.assert_close(out.float().cpu().reshape(total_q, heads, head_dim), want, **ATTN_TOL[dtype])
+    for generic in (False, True):
+        out = torch.full((total_q, heads * head_dim), float("nan"), dtype=dtype, device=device)
+        ops.attn_prefill(buf, keys, values, table, torch.tensor(q_start, dtype=torch.int32, device=device),
+                         torch.tensor(lengths, dtype=torch.int32, device=device), 0, len(cases), max(c[1] for c in cases),
+                         out, heads, kv_heads, head_dim, head_dim ** -0.5, window=window, generic=generic)
+        torch.testing.assert_close(out.float().cpu().reshape(total_q, heads, head_dim), want, **ATTN_TOL[dtype])
     # the decode kernel on the one-token sequence must agree with the prefill kernel
     s = len(cases) - 1
     out1 = torch.full_like(out, float("nan"))
