@@ -40,6 +40,7 @@ def parse():
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--points", default="1,64", help="further decode batch sizes to measure")
     p.add_argument("--no-graphs", action="store_true")
+    p.add_argument("--prefill-only", action="store_true", help="measure only the prefill (profiling runs)")
     p.add_argument("--seed", type=int, default=0)
     return p.parse_args()
 
@@ -130,6 +131,11 @@ def main():
     c = config
     use_graphs = not args.no_graphs
 
+    if args.prefill_only:
+        ms = prefill_run(model, torch, args.prefill_tokens, args.dtype, args.seed)
+        print(json.dumps({"prefill_ms": round(ms, 3), "tokens": args.prefill_tokens,
+                          "tokens_per_s": round(args.prefill_tokens / (ms / 1000), 1)}))
+        return 0
     value, ms_per_step, replays = decode_run(model, torch, args.batch, args.context, args.steps, args.warmup,
                                              args.dtype, use_graphs, args.seed)
     element = 2 if args.dtype == "bfloat16" else 4

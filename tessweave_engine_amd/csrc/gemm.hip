@@ -8,6 +8,18 @@
 //   gemm_generic - any K (rows not 16-byte aligned): one output per thread
 #include "tw_common.h"
 
+// silu(g) * u on a fragment pair, float32 arithmetic, one rounding to T
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::Frag tw_silu_mul_frag(typename Elem<T>::Frag gf, typename Elem<T>::Frag uf) {
+  typename Elem<T>::Frag out;
+#pragma unroll
+  for (int e = 0; e < Elem<T>::kPerFrag; ++e) {
+    const float gv = tw_to_float(gf[e]), uv = tw_to_float(uf[e]);
+    out[e] = tw_from_float<T>(gv / (1.0f + expf(-gv)) * uv);
+  }
+  return out;
+}
+
 // =====================================================================================
 // Tiled kernel. Workgroup = 4 waves in a 2x2 grid, wave tile (32*WM) x (32*WN).
 // One stage holds 128 bytes of K per row (64 bf16 / 32 f32), rows padded to 144
@@ -17,7 +29,8 @@
 // =====================================================================================
 #define TW_LDS_ROW 144
 
-template <typename T, typename OutT, int WM, int WN>
+// SILU: A is [M][2K] = [gate | up] and silu(gate) * up (rounded to T) stands in for the activations.
+template <typename T, typename OutT, int WM, int WN, bool SILU>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A, long lda,
                                                          const T* __restrict__ W, long ldw,
                                                          const float* __restrict__ bias,
@@ -61,7 +74,13 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
     for (int i = 0; i < A_LOADS; ++i) {
       const int c = tid + i * 256, row = c >> 3, kc = c & 7;
       const int gm = m0 + row, gk = kt * BK + kc * EPF;
-      a_reg[i] = (gm < M && gk < K) ? tw_load_frag(A + (size_t)gm * lda + gk) : Elem<T>::zero();
+      if (SILU) {
+        a_reg[i] = (gm < M && gk < K) ? tw_silu_mul_frag<T>(tw_load_frag(A + (size_t)gm * lda + gk),
+                                                            tw_load_frag(A + (size_t)gm * lda + K + gk))
+                                      : Elem<T>::zero();
+      } else {
+        a_reg[i] = (gm < M && gk < K) ? tw_load_frag(A + (size_t)gm * lda + gk) : Elem<T>::zero();
+      }
     }
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
@@ -255,18 +274,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const T* __restrict__ 
 // =====================================================================================
 #define TW_XROW(U) ((U) * 64 + 16)          /* LDS bytes per activation row of a stage, padded */
 
-// silu(g) * u on a fragment pair, float32 arithmetic, one rounding to T
-template <typename T>
-__device__ __forceinline__ typename Elem<T>::Frag tw_silu_mul_frag(typename Elem<T>::Frag gf, typename Elem<T>::Frag uf) {
-  typename Elem<T>::Frag out;
-#pragma unroll
-  for (int e = 0; e < Elem<T>::kPerFrag; ++e) {
-    const float gv = tw_to_float(gf[e]), uv = tw_to_float(uf[e]);
-    out[e] = tw_from_float<T>(gv / (1.0f + expf(-gv)) * uv);
-  }
-  return out;
-}
-
 // SILU: the activations are [M][2K] = [gate | up]; the kernel multiplies silu(gate) * up by W
 // (the rounded product is what a separate SiLU-multiply kernel would have written).
 // PARTIAL: always write float32 partial sums partial[split][M][N] (splits >= 1), no epilogue.
@@ -439,7 +446,7 @@ __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* 
 // =====================================================================================
 // Host side
 // =====================================================================================
-template <typename T, typename OutT, int WM, int WN>
+template <typename T, typename OutT, int WM, int WN, bool SILU = false>
 static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
                         const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
                         hipStream_t stream) {
@@ -449,7 +456,7 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
   TW_REQUIRE(n_blocks < (1L << 30));
   const int grid = (int)((n_blocks + 7) / 8 * 8);
   const size_t lds_bytes = 2 * (size_t)(BM + BN) * TW_LDS_ROW;
-  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN>;
+  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, SILU>;
   static bool attribute_set = false;   // per instantiation
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -584,7 +591,7 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
     if (M <= 48) return launch_skinny<T, OutT, 3>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
     return launch_skinny<T, OutT, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
-  if (force == 4 || (force == 0 && M > 1024 && N >= 4096))
+  if (force == 4)
     return launch_tiled<T, OutT, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
   return launch_tiled<T, OutT, 2, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
 }
@@ -636,6 +643,29 @@ extern "C" int tw_linear_partials(int dtype, int silu, const void* A, long lda, 
   if (dtype == TW_DTYPE_BF16) {
     if (silu) return launch_skinny_lds_m<bf16_t, float, true, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
     return launch_skinny_lds_m<bf16_t, float, false, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+  }
+  return TW_ERR_BAD_ARGUMENT;
+}
+
+// C = (silu(gate) * up) W^T (+ residual) for any number of rows with A = [gate | up] ([M][2K]) and
+// 16-byte aligned K: the tiled kernel forms the product while it loads its A tiles.
+extern "C" int tw_linear_silu(int dtype, int out_f32, const void* A, long lda, const void* W, long ldw,
+                              const float* residual, long ldr, void* C, long ldc, int M, int N, int K,
+                              hipStream_t stream) {
+  TW_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= 2L * K && ldw >= K && ldc >= N);
+  TW_REQUIRE(residual == nullptr || (ldr >= N && out_f32));
+  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
+  TW_REQUIRE(K % epf == 0 && lda % epf == 0 && ldw % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
+  if (M == 0) return 0;
+  if (dtype == TW_DTYPE_F32)
+    return launch_tiled<float, float, 2, 2, true>((const float*)A, lda, (const float*)W, ldw, nullptr, residual, ldr,
+                                                  (float*)C, ldc, M, N, K, stream);
+  if (dtype == TW_DTYPE_BF16) {
+    if (out_f32)
+      return launch_tiled<bf16_t, float, 2, 2, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
+                                                     ldr, (float*)C, ldc, M, N, K, stream);
+    return launch_tiled<bf16_t, bf16_t, 2, 2, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
+                                                    ldr, (bf16_t*)C, ldc, M, N, K, stream);
   }
   return TW_ERR_BAD_ARGUMENT;
 }

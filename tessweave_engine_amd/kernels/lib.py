@@ -25,6 +25,7 @@ _SIGNATURES = {
     "tw_linear_workspace_bytes": (L, [I, I, I, I]),
     "tw_linear_partial_splits": (I, [I, I, I]),
     "tw_linear_partials": (I, [I, I, P, L, P, L, P, L, I, I, I, P]),
+    "tw_linear_silu": (I, [I, I, P, L, P, L, P, L, P, L, I, I, I, P]),
     "tw_linear": (I, [I, I, P, L, P, L, P, P, L, P, L, P, L, I, I, I, I, P]),
     "tw_attn_decode_splits": (I, [I, I, I, I]),
     "tw_attn_decode_workspace_floats": (L, [I, I, I, I]),

@@ -174,6 +174,26 @@ def linear_partials(x, weight, partial, silu_gate=False):
     return partial
 
 
+def linear_silu(gate_up, weight, out, residual=None):
+    """out = (silu(gate) * up) @ weight.T (+ residual) with gate_up = [gate | up] ([m, 2k]); K 16-byte aligned."""
+    m, k2, lda = _rows(gate_up, "gate_up")
+    n, k, ldw = _rows(weight, "weight")
+    mo, no, ldc = _rows(out, "out")
+    _need(k2 == 2 * k and (mo, no) == (m, n) and gate_up.dtype == weight.dtype, "linear_silu shapes or types do not agree")
+    _need(k % (8 if weight.dtype == torch.bfloat16 else 4) == 0, "linear_silu needs K to be a multiple of 16 bytes")
+    out_f32 = out.dtype == torch.float32
+    _need(out_f32 or out.dtype == weight.dtype, "out must be float32 or the input type")
+    ldr = 0
+    if residual is not None:
+        _need(out_f32, "a residual needs a float32 output")
+        mr, nr, ldr = _rows(residual, "residual")
+        _need((mr, nr) == (m, n), "residual shape differs from the output")
+    check(library().tw_linear_silu(dtype_id(weight.dtype), 1 if out_f32 else 0, _dev(gate_up), lda, _dev(weight), ldw,
+                                   _dev(residual, torch.float32, "residual") if residual is not None else None, ldr,
+                                   _dev(out), ldc, m, n, k, _stream()), "linear_silu")
+    return out
+
+
 GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY_COOP = 0, 1, 2, 3, 4, 5
 
 

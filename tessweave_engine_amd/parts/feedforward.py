@@ -31,6 +31,8 @@ class SwiGLU(FeedForward):
             # few rows: silu(gate) * up is formed while the down projection stages its input,
             # and its split-K sums are left to the next norm
             return self.down.forward_partials(ctx, gu, "down", silu_gate=True)
+        # many rows: a separate SiLU-multiply pass (fused into the tiled kernel's tile loads it would
+        # be recomputed once per column tile, which costs more than the pass)
         act = ctx.scratch("ffn.act", (n, self.intermediate))
         ops.silu_mul(gu, act)
         self.down.forward(ctx, act, x, residual=x)

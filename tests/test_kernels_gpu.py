@@ -197,6 +197,21 @@ def test_linear_partials_and_fused_silu(ops, device, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(65, 48, 64), (200, 389, 320), (300, 130, 1032)])
+def test_linear_silu_many_rows(ops, device, dtype, m, n, k):
+    gu = rand((m, 2 * k), dtype, device, 1.0, seed=3)
+    w = rand((n, k), dtype, device, 0.05, seed=2)
+    res = rand((m, n), torch.float32, device, 1.0, seed=4)
+    act = torch.empty(m, k, dtype=dtype, device=device)
+    ops.silu_mul(gu, act)
+    want = res.clone()
+    ops.linear(act, w, want, residual=want, force=ops.GEMM_TILED)
+    got = res.clone()
+    ops.linear_silu(gu, w, got, residual=got)
+    torch.testing.assert_close(got, want, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_odd_k_uses_generic(ops, device, dtype):
     m, n, k = 5, 37, 101
     x, w = rand((m, k), dtype, device, seed=1), rand((n, k), dtype, device, 0.1, seed=2)
