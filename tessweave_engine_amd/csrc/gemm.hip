@@ -30,7 +30,8 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_silu_mul_frag(typename Elem
 #define TW_LDS_ROW 144
 
 // SILU: A is [M][2K] = [gate | up] and silu(gate) * up (rounded to T) stands in for the activations.
-template <typename T, typename OutT, int WM, int WN, bool SILU>
+// KCH: 16-byte chunks of K per row and stage (8: 128 bytes, 4: 64 bytes).
+template <typename T, typename OutT, int WM, int WN, int KCH, bool SILU>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A, long lda,
                                                          const T* __restrict__ W, long ldw,
                                                          const float* __restrict__ bias,
@@ -39,9 +40,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
                                                          int n_blocks) {
   typedef typename Elem<T>::Frag Frag;
   constexpr int EPF = Elem<T>::kPerFrag;
-  constexpr int BK = 8 * EPF;
+  constexpr int BK = KCH * EPF;
   constexpr int BM = 64 * WM, BN = 64 * WN;
-  constexpr int A_LOADS = BM / 32, W_LOADS = BN / 32;
+  constexpr int LROW = KCH * 16 + 16;                       // LDS bytes per row of a stage, padded
+  constexpr int A_LOADS = BM * KCH / 256, W_LOADS = BN * KCH / 256;
+  constexpr int STAGE = (BM + BN) * LROW;                   // bytes of one stage: A rows then W rows
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
   // Blocks are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
@@ -56,8 +59,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
   const int wm0 = (wave >> 1) * 32 * WM, wn0 = (wave & 1) * 32 * WN;
   const int r = lane & 31, g = lane >> 5;
 
-  constexpr int STAGE = (BM + BN) * TW_LDS_ROW;            // bytes of one stage: A rows then W rows
-
   f32x16 acc[WM][WN];
 #pragma unroll
   for (int i = 0; i < WM; ++i)
@@ -66,82 +67,168 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  Frag a_reg[A_LOADS], w_reg[W_LOADS];
+  // Global addressing: a tile base that is the same for every lane, plus per-thread element
+  // offsets fixed for the whole K loop. Rows past the end are clamped to the last valid row
+  // (what they produce is never stored), so whole k-tiles need no predicate.
+  const T* a_tile = A + (size_t)m0 * lda;
+  const T* w_tile = W + (size_t)n0 * ldw;
+  unsigned a_off[A_LOADS], w_off[W_LOADS];
+  int st_off[A_LOADS > W_LOADS ? A_LOADS : W_LOADS];
+#pragma unroll
+  for (int i = 0; i < A_LOADS; ++i) {
+    const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
+    a_off[i] = (unsigned)(min(m0 + row, M - 1) - m0) * (unsigned)lda + kc * EPF;
+  }
+#pragma unroll
+  for (int i = 0; i < W_LOADS; ++i) {
+    const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
+    w_off[i] = (unsigned)(min(n0 + row, N - 1) - n0) * (unsigned)ldw + kc * EPF;
+  }
+#pragma unroll
+  for (int i = 0; i < (A_LOADS > W_LOADS ? A_LOADS : W_LOADS); ++i) {
+    const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
+    st_off[i] = row * LROW + kc * 16;                // same layout for the A rows and the W rows
+  }
+  const int kc_mine = tid % KCH;
+
+  // Two register sets: the global loads of k-tile kt+2 are issued while k-tile kt is multiplied,
+  // so two k-tiles per workgroup are on their way from memory at any time.
+  Frag a_regs[2][A_LOADS], w_regs[2][W_LOADS];
   const int k_tiles = (K + BK - 1) / BK;
+  const int whole_tiles = K / BK;
 
-  auto load_global = [&](int kt) {
+  auto load_global = [&](int kt, Frag* a_reg, Frag* w_reg) {
+    const T* ab = a_tile + (size_t)kt * BK;
+    const T* wb = w_tile + (size_t)kt * BK;
+    if (kt < whole_tiles) {
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
-      const int gm = m0 + row, gk = kt * BK + kc * EPF;
-      if (SILU) {
-        a_reg[i] = (gm < M && gk < K) ? tw_silu_mul_frag<T>(tw_load_frag(A + (size_t)gm * lda + gk),
-                                                            tw_load_frag(A + (size_t)gm * lda + K + gk))
-                                      : Elem<T>::zero();
-      } else {
-        a_reg[i] = (gm < M && gk < K) ? tw_load_frag(A + (size_t)gm * lda + gk) : Elem<T>::zero();
+      for (int i = 0; i < A_LOADS; ++i) {
+        if (SILU) a_reg[i] = tw_silu_mul_frag<T>(tw_load_frag(ab + a_off[i]), tw_load_frag(ab + K + a_off[i]));
+        else a_reg[i] = tw_load_frag(ab + a_off[i]);
       }
-    }
 #pragma unroll
-    for (int i = 0; i < W_LOADS; ++i) {
-      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
-      const int gn = n0 + row, gk = kt * BK + kc * EPF;
-      w_reg[i] = (gn < N && gk < K) ? tw_load_frag(W + (size_t)gn * ldw + gk) : Elem<T>::zero();
+      for (int i = 0; i < W_LOADS; ++i) w_reg[i] = tw_load_frag(wb + w_off[i]);
+    } else {                                                // the last, partial k-tile: chunks past K are zeros
+      const bool ok = kt * BK + kc_mine * EPF < K;
+#pragma unroll
+      for (int i = 0; i < A_LOADS; ++i) {
+        if (SILU) a_reg[i] = ok ? tw_silu_mul_frag<T>(tw_load_frag(ab + a_off[i]), tw_load_frag(ab + K + a_off[i])) : Elem<T>::zero();
+        else a_reg[i] = ok ? tw_load_frag(ab + a_off[i]) : Elem<T>::zero();
+      }
+#pragma unroll
+      for (int i = 0; i < W_LOADS; ++i) w_reg[i] = ok ? tw_load_frag(wb + w_off[i]) : Elem<T>::zero();
     }
   };
-  auto store_lds = [&](int buf) {
+  auto store_lds = [&](int buf, const Frag* a_reg, const Frag* w_reg) {
+    char* base = lds + buf * STAGE;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
-      *reinterpret_cast<Frag*>(lds + buf * STAGE + row * TW_LDS_ROW + kc * 16) = a_reg[i];
-    }
+    for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<Frag*>(base + st_off[i]) = a_reg[i];
 #pragma unroll
-    for (int i = 0; i < W_LOADS; ++i) {
-      const int c = tid + i * 256, row = c >> 3, kc = c & 7;
-      *reinterpret_cast<Frag*>(lds + buf * STAGE + (BM + row) * TW_LDS_ROW + kc * 16) = w_reg[i];
+    for (int i = 0; i < W_LOADS; ++i) *reinterpret_cast<Frag*>(base + BM * LROW + st_off[i]) = w_reg[i];
+  };
+
+  // this lane's fragment addresses in stage 0 (k-chunk pair cc adds 32 bytes)
+  const char* a_frag = lds + (wm0 + r) * LROW + g * 16;
+  const char* w_frag = lds + (BM + wn0 + r) * LROW + g * 16;
+  auto read_frags = [&](int buf, int cc, Frag* af, Frag* wf) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+      af[i] = *reinterpret_cast<const Frag*>(a_frag + buf * STAGE + i * 32 * LROW + cc * 32);
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+      wf[j] = *reinterpret_cast<const Frag*>(w_frag + buf * STAGE + j * 32 * LROW + cc * 32);
+  };
+
+  auto multiply = [&](int buf) {
+    // the fragments of the next k-chunk pair are read from LDS while this one is multiplied
+    Frag af[2][WM], wf[2][WN];
+    read_frags(buf, 0, af[0], wf[0]);
+#pragma unroll
+    for (int cc = 0; cc < KCH / 2; ++cc) {
+      if (cc + 1 < KCH / 2) read_frags(buf, cc + 1, af[(cc + 1) & 1], wf[(cc + 1) & 1]);
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[cc & 1][i], wf[cc & 1][j]);
     }
   };
 
-  load_global(0);
-  store_lds(0);
+  load_global(0, a_regs[0], w_regs[0]);
+  if (k_tiles > 1) load_global(1, a_regs[1], w_regs[1]);
+  store_lds(0, a_regs[0], w_regs[0]);
   __syncthreads();
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < k_tiles) load_global(kt + 1);
-#pragma unroll
-    for (int cc = 0; cc < 4; ++cc) {
-      Frag af[WM], wf[WN];
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-        af[i] = *reinterpret_cast<const Frag*>(lds + buf * STAGE + (wm0 + i * 32 + r) * TW_LDS_ROW + (2 * cc + g) * 16);
-#pragma unroll
-      for (int j = 0; j < WN; ++j)
-        wf[j] = *reinterpret_cast<const Frag*>(lds + buf * STAGE + (BM + wn0 + j * 32 + r) * TW_LDS_ROW + (2 * cc + g) * 16);
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[i], wf[j]);
-    }
-    if (kt + 1 < k_tiles) store_lds(buf ^ 1);
+  for (int kt = 0; kt < k_tiles; kt += 2) {
+    // even k-tile: LDS stage 0, register set 0 is free for k-tile kt+2
+    if (kt + 2 < k_tiles) load_global(kt + 2, a_regs[0], w_regs[0]);
+    multiply(0);
+    if (kt + 1 < k_tiles) store_lds(1, a_regs[1], w_regs[1]);
+    __syncthreads();
+    if (kt + 1 >= k_tiles) break;
+    // odd k-tile: LDS stage 1, register set 1 is free for k-tile kt+3
+    if (kt + 3 < k_tiles) load_global(kt + 3, a_regs[1], w_regs[1]);
+    multiply(1);
+    if (kt + 2 < k_tiles) store_lds(0, a_regs[0], w_regs[0]);
     __syncthreads();
   }
 
+  // ---- epilogue: each wave passes its tile through LDS (32 rows at a time) so that a lane
+  // stores 8 consecutive columns of one row: whole cache lines instead of 2- or 4-byte pieces.
+  constexpr int WCOLS = 32 * WN;                             // columns of a wave tile
+  constexpr int EROW = WCOLS + 4;                            // floats per staged row, padded
+  // (the launcher asks for max(pipeline stages, 4 waves x 32 rows x EROW floats) bytes of LDS)
+  float* stage = reinterpret_cast<float*>(lds) + wave * 32 * EROW;
+  constexpr int CPR = WCOLS / 8;                             // 8-column groups per row
+  const bool vec_ok = (ldc % 8 == 0) && (residual == nullptr || ldr % 4 == 0) &&
+                      ((uintptr_t)C % 16 == 0) && ((uintptr_t)residual % 16 == 0);
 #pragma unroll
-  for (int i = 0; i < WM; ++i)
+  for (int i = 0; i < WM; ++i) {
+    __syncthreads();                                          // the pipeline's (or the last round's) LDS reads are done
 #pragma unroll
-    for (int j = 0; j < WN; ++j) {
-      const int col = n0 + wn0 + j * 32 + r;
-      if (col >= N) continue;
-      const float b = bias ? bias[col] : 0.f;
+    for (int j = 0; j < WN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm0 + i * 32 + 8 * (e / 4) + 4 * g + (e % 4);
-        if (row >= M) continue;
-        float v = acc[i][j][e] + b;
-        if (residual) v += residual[(size_t)row * ldr + col];
-        C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
+      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * g + (e % 4)) * EROW + j * 32 + r] = acc[i][j][e];
+    __syncthreads();
+#pragma unroll
+    for (int q = lane; q < 32 * CPR; q += 64) {
+      const int lr = q / CPR, lc = (q % CPR) * 8;
+      const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
+      if (row >= M || col >= N) continue;
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = stage[lr * EROW + lc + e];
+      if (bias) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) v[e] += bias[col + e];
+      }
+      if (vec_ok && col + 8 <= N) {
+        if (residual) {
+          const f32x4 r0 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col);
+          const f32x4 r1 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { v[e] += r0[e]; v[4 + e] += r1[e]; }
+        }
+        OutT* dst = C + (size_t)row * ldc + col;
+        if (sizeof(OutT) == 4) {
+          *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+          *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
+        } else {
+          bf16x8 o;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
+          *reinterpret_cast<bf16x8*>(dst) = o;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) {
+            float x = v[e];
+            if (residual) x += residual[(size_t)row * ldr + col + e];
+            C[(size_t)row * ldc + col + e] = tw_from_float<OutT>(x);
+          }
       }
     }
+  }
 }
 
 // =====================================================================================
@@ -446,7 +533,7 @@ __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* 
 // =====================================================================================
 // Host side
 // =====================================================================================
-template <typename T, typename OutT, int WM, int WN, bool SILU = false>
+template <typename T, typename OutT, int WM, int WN, int KCH = 8, bool SILU = false>
 static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
                         const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
                         hipStream_t stream) {
@@ -454,9 +541,12 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
   const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
   const long n_blocks = (long)tiles_m * tiles_n;
   TW_REQUIRE(n_blocks < (1L << 30));
+  TW_REQUIRE((long)BM * lda < (1L << 31) && (long)BN * ldw < (1L << 31));     // per-tile offsets are 32-bit
   const int grid = (int)((n_blocks + 7) / 8 * 8);
-  const size_t lds_bytes = 2 * (size_t)(BM + BN) * TW_LDS_ROW;
-  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, SILU>;
+  const size_t pipeline_bytes = 2 * (size_t)(BM + BN) * (KCH * 16 + 16);
+  const size_t epilogue_bytes = 4 * 32 * (size_t)(32 * WN + 4) * 4;
+  const size_t lds_bytes = pipeline_bytes > epilogue_bytes ? pipeline_bytes : epilogue_bytes;
+  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, KCH, SILU>;
   static bool attribute_set = false;   // per instantiation
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -573,7 +663,7 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
   const bool aligned = K % EPF == 0 && lda % EPF == 0 && ldw % EPF == 0 &&
                        ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
   // force: 0 = choose, 1 = generic, 2 = skinny (per-wave), 3 = tiled 128x128, 4 = tiled 128x256,
-  //        5 = skinny (workgroup-cooperative)
+  //        5 = skinny (workgroup-cooperative), 6..8 = tiled with 64-byte stages (256x128, 128x128, 128x256)
   if (force == 1 || !aligned) {
     TW_REQUIRE(force <= 1);
     gemm_generic_kernel<T, OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(A, lda, W, ldw, bias, residual,
@@ -593,6 +683,12 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
   }
   if (force == 4)
     return launch_tiled<T, OutT, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+  if (force == 6)      // 256x128 tile, 64-byte stages
+    return launch_tiled<T, OutT, 4, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+  if (force == 7)      // 128x128 tile, 64-byte stages
+    return launch_tiled<T, OutT, 2, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+  if (force == 8)      // 128x256 tile, 64-byte stages
+    return launch_tiled<T, OutT, 2, 4, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
   return launch_tiled<T, OutT, 2, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
 }
 
@@ -658,13 +754,13 @@ extern "C" int tw_linear_silu(int dtype, int out_f32, const void* A, long lda, c
   TW_REQUIRE(K % epf == 0 && lda % epf == 0 && ldw % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
   if (M == 0) return 0;
   if (dtype == TW_DTYPE_F32)
-    return launch_tiled<float, float, 2, 2, true>((const float*)A, lda, (const float*)W, ldw, nullptr, residual, ldr,
+    return launch_tiled<float, float, 2, 2, 8, true>((const float*)A, lda, (const float*)W, ldw, nullptr, residual, ldr,
                                                   (float*)C, ldc, M, N, K, stream);
   if (dtype == TW_DTYPE_BF16) {
     if (out_f32)
-      return launch_tiled<bf16_t, float, 2, 2, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
+      return launch_tiled<bf16_t, float, 2, 2, 8, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
                                                      ldr, (float*)C, ldc, M, N, K, stream);
-    return launch_tiled<bf16_t, bf16_t, 2, 2, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
+    return launch_tiled<bf16_t, bf16_t, 2, 2, 8, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
                                                     ldr, (bf16_t*)C, ldc, M, N, K, stream);
   }
   return TW_ERR_BAD_ARGUMENT;
