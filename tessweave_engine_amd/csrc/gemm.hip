@@ -6,7 +6,25 @@
 //   gemm_skinny  - few rows (decode): weights streamed once from HBM straight
 //                  into 16x16 MFMA fragments, split over K when N is small
 //   gemm_generic - any K (rows not 16-byte aligned): one output per thread
+//
+// Weight layouts. Row-major [N][K] as in the checkpoint, or SHUFFLED (an exact permutation,
+// zero padded): blocks of 16 rows x 4 sixteen-byte chunks stored in the order the MFMA units
+// read them, [N/16][K/(4*EPF)][chunk 0..3][row 0..15][EPF]. Element (n, k) is at
+//   ((n/16 * k_steps + (k/EPF)/4) * 64 + ((k/EPF)%4) * 16 + n%16) * EPF + k%EPF.
+// A wave's load of one block is 1 KB of consecutive memory: the decode kernels stream weights
+// as whole cache lines and may skip the caches (non-temporal), the tiled kernel copies blocks.
 #include "tw_common.h"
+
+// element offset of (row n, 16-byte chunk c) in the shuffled layout
+__device__ __forceinline__ size_t tw_shuffled_chunk(int n, int c, int k_steps, int epf) {
+  return ((size_t)((size_t)(n >> 4) * k_steps + (c >> 2)) * 64 + (c & 3) * 16 + (n & 15)) * epf;
+}
+
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p) {
+  // weights are read once per step: do not keep them in the caches
+  return __builtin_nontemporal_load(reinterpret_cast<const typename Elem<T>::Frag*>(p));
+}
 
 // silu(g) * u on a fragment pair, float32 arithmetic, one rounding to T
 template <typename T>
@@ -31,7 +49,8 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_silu_mul_frag(typename Elem
 
 // SILU: A is [M][2K] = [gate | up] and silu(gate) * up (rounded to T) stands in for the activations.
 // KCH: 16-byte chunks of K per row and stage (8: 128 bytes, 4: 64 bytes).
-template <typename T, typename OutT, int WM, int WN, int KCH, bool SILU>
+// SHUF: W is in the shuffled layout and ldw is its k_steps.
+template <typename T, typename OutT, int WM, int WN, int KCH, bool SILU, bool SHUF>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A, long lda,
                                                          const T* __restrict__ W, long ldw,
                                                          const float* __restrict__ bias,
@@ -71,23 +90,39 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
   // offsets fixed for the whole K loop. Rows past the end are clamped to the last valid row
   // (what they produce is never stored), so whole k-tiles need no predicate.
   const T* a_tile = A + (size_t)m0 * lda;
-  const T* w_tile = W + (size_t)n0 * ldw;
+  const T* w_tile = SHUF ? W + (size_t)(n0 / 16) * ldw * 64 * EPF : W + (size_t)n0 * ldw;
+  const int k_steps_w = SHUF ? (int)ldw : 0;
   unsigned a_off[A_LOADS], w_off[W_LOADS];
-  int st_off[A_LOADS > W_LOADS ? A_LOADS : W_LOADS];
+  int st_off[A_LOADS];
 #pragma unroll
   for (int i = 0; i < A_LOADS; ++i) {
     const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
     a_off[i] = (unsigned)(min(m0 + row, M - 1) - m0) * (unsigned)lda + kc * EPF;
   }
+  constexpr int SPT = KCH / 4;                             // shuffled k-steps per k-tile
+  int w_st_off[W_LOADS], w_ks[W_LOADS];
+  const int n_blocks_w = (N + 15) / 16;
 #pragma unroll
   for (int i = 0; i < W_LOADS; ++i) {
-    const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
-    w_off[i] = (unsigned)(min(n0 + row, N - 1) - n0) * (unsigned)ldw + kc * EPF;
+    const int c = tid + i * 256;
+    if (SHUF) {
+      // piece c of the tile: block (16 rows x 4 chunks) c / 64, lane c % 64 of that block
+      const int blk = c >> 6, ln = c & 63, nblk = blk / SPT, ks = blk % SPT;
+      const int gblk = min(n0 / 16 + nblk, n_blocks_w - 1);
+      w_off[i] = (unsigned)(gblk - n0 / 16) * (unsigned)ldw * 64 * EPF + (ks * 64 + ln) * EPF;
+      w_ks[i] = ks;
+      w_st_off[i] = (nblk * 16 + (ln & 15)) * LROW + (ks * 4 + (ln >> 4)) * 16;
+    } else {
+      const int row = c / KCH, kc = c % KCH;
+      w_off[i] = (unsigned)(min(n0 + row, N - 1) - n0) * (unsigned)ldw + kc * EPF;
+      w_ks[i] = 0;
+      w_st_off[i] = row * LROW + kc * 16;
+    }
   }
 #pragma unroll
-  for (int i = 0; i < (A_LOADS > W_LOADS ? A_LOADS : W_LOADS); ++i) {
+  for (int i = 0; i < A_LOADS; ++i) {
     const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
-    st_off[i] = row * LROW + kc * 16;                // same layout for the A rows and the W rows
+    st_off[i] = row * LROW + kc * 16;
   }
   const int kc_mine = tid % KCH;
 
@@ -97,18 +132,24 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
   const int k_tiles = (K + BK - 1) / BK;
   const int whole_tiles = K / BK;
 
-  auto load_global = [&](int kt, Frag* a_reg, Frag* w_reg) {
+  // whole k-tiles need no predicate at all; the main loop below runs only those
+  auto load_whole = [&](int kt, Frag* a_reg, Frag* w_reg) {
     const T* ab = a_tile + (size_t)kt * BK;
-    const T* wb = w_tile + (size_t)kt * BK;
+    const T* wb = SHUF ? w_tile + (size_t)kt * SPT * 64 * EPF : w_tile + (size_t)kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+      if (SILU) a_reg[i] = tw_silu_mul_frag<T>(tw_load_frag(ab + a_off[i]), tw_load_frag(ab + K + a_off[i]));
+      else a_reg[i] = tw_load_frag(ab + a_off[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) w_reg[i] = tw_load_frag(wb + w_off[i]);
+  };
+  auto load_global = [&](int kt, Frag* a_reg, Frag* w_reg) {
     if (kt < whole_tiles) {
-#pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) {
-        if (SILU) a_reg[i] = tw_silu_mul_frag<T>(tw_load_frag(ab + a_off[i]), tw_load_frag(ab + K + a_off[i]));
-        else a_reg[i] = tw_load_frag(ab + a_off[i]);
-      }
-#pragma unroll
-      for (int i = 0; i < W_LOADS; ++i) w_reg[i] = tw_load_frag(wb + w_off[i]);
+      load_whole(kt, a_reg, w_reg);
     } else {                                                // the last, partial k-tile: chunks past K are zeros
+      const T* ab = a_tile + (size_t)kt * BK;
+      const T* wb = SHUF ? w_tile + (size_t)kt * SPT * 64 * EPF : w_tile + (size_t)kt * BK;
       const bool ok = kt * BK + kc_mine * EPF < K;
 #pragma unroll
       for (int i = 0; i < A_LOADS; ++i) {
@@ -116,7 +157,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
         else a_reg[i] = ok ? tw_load_frag(ab + a_off[i]) : Elem<T>::zero();
       }
 #pragma unroll
-      for (int i = 0; i < W_LOADS; ++i) w_reg[i] = ok ? tw_load_frag(wb + w_off[i]) : Elem<T>::zero();
+      for (int i = 0; i < W_LOADS; ++i) {
+        const bool w_ok = SHUF ? kt * SPT + w_ks[i] < k_steps_w : ok;     // the shuffled layout is zero padded
+        w_reg[i] = w_ok ? tw_load_frag(wb + w_off[i]) : Elem<T>::zero();
+      }
     }
   };
   auto store_lds = [&](int buf, const Frag* a_reg, const Frag* w_reg) {
@@ -124,7 +168,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<Frag*>(base + st_off[i]) = a_reg[i];
 #pragma unroll
-    for (int i = 0; i < W_LOADS; ++i) *reinterpret_cast<Frag*>(base + BM * LROW + st_off[i]) = w_reg[i];
+    for (int i = 0; i < W_LOADS; ++i) *reinterpret_cast<Frag*>(base + BM * LROW + w_st_off[i]) = w_reg[i];
   };
 
   // this lane's fragment addresses in stage 0 (k-chunk pair cc adds 32 bytes)
@@ -157,14 +201,26 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
   if (k_tiles > 1) load_global(1, a_regs[1], w_regs[1]);
   store_lds(0, a_regs[0], w_regs[0]);
   __syncthreads();
-  for (int kt = 0; kt < k_tiles; kt += 2) {
-    // even k-tile: LDS stage 0, register set 0 is free for k-tile kt+2
+  int kt = 0;
+  // Main loop: two k-tiles per round, every load whole and unconditional, so that the register
+  // sets are plain loop-carried values (conditional loads cost a register copy per loaded dword).
+  for (; kt + 3 < whole_tiles; kt += 2) {
+    load_whole(kt + 2, a_regs[0], w_regs[0]);               // LDS stage 0, register set 0 is free
+    multiply(0);
+    store_lds(1, a_regs[1], w_regs[1]);
+    __syncthreads();
+    load_whole(kt + 3, a_regs[1], w_regs[1]);               // LDS stage 1, register set 1 is free
+    multiply(1);
+    store_lds(0, a_regs[0], w_regs[0]);
+    __syncthreads();
+  }
+  // The last few k-tiles (kt is even here): the same rounds with every step conditional.
+  for (; kt < k_tiles; kt += 2) {
     if (kt + 2 < k_tiles) load_global(kt + 2, a_regs[0], w_regs[0]);
     multiply(0);
     if (kt + 1 < k_tiles) store_lds(1, a_regs[1], w_regs[1]);
     __syncthreads();
     if (kt + 1 >= k_tiles) break;
-    // odd k-tile: LDS stage 1, register set 1 is free for k-tile kt+3
     if (kt + 3 < k_tiles) load_global(kt + 3, a_regs[1], w_regs[1]);
     multiply(1);
     if (kt + 2 < k_tiles) store_lds(0, a_regs[0], w_regs[0]);
@@ -364,7 +420,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const T* __restrict__ 
 // SILU: the activations are [M][2K] = [gate | up]; the kernel multiplies silu(gate) * up by W
 // (the rounded product is what a separate SiLU-multiply kernel would have written).
 // PARTIAL: always write float32 partial sums partial[split][M][N] (splits >= 1), no epilogue.
-template <typename T, typename OutT, int MT, int U, bool SILU, bool PARTIAL>
+// SHUF: W is in the shuffled layout (ldw = its k_steps): every weight load is 1 KB of consecutive
+// memory, needs no predicate (the layout is zero padded) and bypasses the caches.
+template <typename T, typename OutT, int MT, int U, bool SILU, bool PARTIAL, bool SHUF>
 __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restrict__ A, long lda,
                                                               const T* __restrict__ W, long ldw,
                                                               const float* __restrict__ bias,
@@ -395,7 +453,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const T* w_row = W + (size_t)min(n0 + r, N - 1) * ldw;
+  const T* w_row = SHUF ? W + ((size_t)min(n0 / 16, (N + 15) / 16 - 1) * ldw * 64 + lane) * EPF
+                        : W + (size_t)min(n0 + r, N - 1) * ldw;
   // this thread's share of the activation slice: fragment f = i*256 + tid -> (row f / (4U), chunk f % (4U))
   const T* x_src[XLOADS];
   int x_dst[XLOADS], x_chunk[XLOADS];
@@ -412,7 +471,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int chunk = (s0 + u) * 4 + g;
-      if (whole || ((s0 + u) < step_end && chunk < chunks))
+      if (SHUF) {
+        if (whole || (s0 + u) < step_end)
+          wf[buf][u] = tw_load_frag_stream(w_row + (size_t)(s0 + u) * 64 * EPF);
+        else
+          wf[buf][u] = Elem<T>::zero();
+      } else if (whole || ((s0 + u) < step_end && chunk < chunks))
         wf[buf][u] = tw_load_frag(w_row + (size_t)chunk * EPF);
       else
         wf[buf][u] = Elem<T>::zero();
@@ -517,13 +581,18 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int spli
 template <typename T, typename OutT>
 __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* __restrict__ W, long ldw,
                                     const float* __restrict__ bias, const float* residual, long ldr,
-                                    OutT* C, long ldc, int M, int N, int K) {
+                                    OutT* C, long ldc, int M, int N, int K, int shuffled) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= (long)M * N) return;
   const int row = (int)(i / N), col = (int)(i % N);
   const T* a = A + (size_t)row * lda;
   const T* w = W + (size_t)col * ldw;
+  constexpr int EPF = Elem<T>::kPerFrag;
   float v = 0.f;
+  if (shuffled) {
+    for (int k = 0; k < K; ++k)
+      v = fmaf(tw_to_float(a[k]), tw_to_float(W[tw_shuffled_chunk(col, k / EPF, (int)ldw, EPF) + k % EPF]), v);
+  } else
   for (int k = 0; k < K; ++k) v = fmaf(tw_to_float(a[k]), tw_to_float(w[k]), v);
   if (bias) v += bias[col];
   if (residual) v += residual[(size_t)row * ldr + col];
@@ -533,20 +602,23 @@ __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* 
 // =====================================================================================
 // Host side
 // =====================================================================================
-template <typename T, typename OutT, int WM, int WN, int KCH = 8, bool SILU = false>
+template <typename T, typename OutT, int WM, int WN, bool SHUF>
 static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
                         const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
                         hipStream_t stream) {
-  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int BM = 64 * WM, BN = 64 * WN, KCH = 8;
+  constexpr int EPF = Elem<T>::kPerFrag;
   const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
   const long n_blocks = (long)tiles_m * tiles_n;
   TW_REQUIRE(n_blocks < (1L << 30));
-  TW_REQUIRE((long)BM * lda < (1L << 31) && (long)BN * ldw < (1L << 31));     // per-tile offsets are 32-bit
+  // per-tile offsets are 32-bit
+  TW_REQUIRE((long)BM * lda < (1L << 31));
+  TW_REQUIRE(SHUF ? (long)(BN / 16) * ldw * 64 * EPF < (1L << 31) : (long)BN * ldw < (1L << 31));
   const int grid = (int)((n_blocks + 7) / 8 * 8);
   const size_t pipeline_bytes = 2 * (size_t)(BM + BN) * (KCH * 16 + 16);
   const size_t epilogue_bytes = 4 * 32 * (size_t)(32 * WN + 4) * 4;
   const size_t lds_bytes = pipeline_bytes > epilogue_bytes ? pipeline_bytes : epilogue_bytes;
-  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, KCH, SILU>;
+  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, KCH, false, SHUF>;
   static bool attribute_set = false;   // per instantiation
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -559,12 +631,12 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
   return TW_LAUNCH_RESULT();
 }
 
-// Output tiles per wave of the skinny kernel (they share the activation fragments).
+// Output tiles per wave of the per-wave skinny kernel (they share the activation fragments).
 static int skinny_tiles_per_wave(int N) { return N >= 16384 ? 2 : 1; }
 
-// How many K ranges the skinny kernel uses for an [N, K] weight: enough waves
-// to fill 256 CUs several times over, each range at least 16 MFMA steps long.
-// The choice depends on N and K only, never on the rows of a batch.
+// How many K ranges the skinny kernels use for an [N, K] weight: enough waves to fill 256 CUs
+// several times over, each range at least 16 MFMA steps long. The choice depends on N and K
+// only, never on the rows of a batch.
 static int skinny_splits(int N, int K, int epf) {
   const int groups = tw_div_up(N, 16 * skinny_tiles_per_wave(N));
   const int steps = tw_div_up(K / epf, 4);
@@ -614,7 +686,16 @@ static int launch_skinny_tw(const T* A, long lda, const T* W, long ldw, const fl
   return TW_LAUNCH_RESULT();
 }
 
-template <typename T, typename OutT, int MT, bool SILU, bool PARTIAL>
+template <typename T, typename OutT, int MT>
+static int launch_skinny(const T* A, long lda, const T* W, long ldw, const float* bias,
+                         const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                         long partial_bytes, int M, int N, int K, hipStream_t stream) {
+  if (skinny_tiles_per_wave(N) == 2)
+    return launch_skinny_tw<T, OutT, MT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  return launch_skinny_tw<T, OutT, MT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+}
+
+template <typename T, typename OutT, int MT, bool SILU, bool PARTIAL, bool SHUF>
 static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const float* bias,
                              const float* residual, long ldr, OutT* C, long ldc, float* partial,
                              long partial_bytes, int M, int N, int K, hipStream_t stream) {
@@ -627,7 +708,7 @@ static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const f
   } else if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) {
     splits = 1;
   }
-  gemm_skinny_lds_kernel<T, OutT, MT, U, SILU, PARTIAL><<<groups * splits, 256, 0, stream>>>(
+  gemm_skinny_lds_kernel<T, OutT, MT, U, SILU, PARTIAL, SHUF><<<groups * splits, 256, 0, stream>>>(
       A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
   int err = TW_LAUNCH_RESULT();
   if (err || splits == 1 || PARTIAL) return err;
@@ -636,81 +717,80 @@ static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const f
   return TW_LAUNCH_RESULT();
 }
 
-template <typename T, typename OutT, bool SILU, bool PARTIAL>
+template <typename T, typename OutT, bool SILU, bool PARTIAL, bool SHUF>
 static int launch_skinny_lds_m(const T* A, long lda, const T* W, long ldw, const float* bias,
                                const float* residual, long ldr, OutT* C, long ldc, float* partial,
                                long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  if (M <= 16) return launch_skinny_lds<T, OutT, 1, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  if (M <= 32) return launch_skinny_lds<T, OutT, 2, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  if (M <= 48) return launch_skinny_lds<T, OutT, 3, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  return launch_skinny_lds<T, OutT, 4, SILU, PARTIAL>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 16) return launch_skinny_lds<T, OutT, 1, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 32) return launch_skinny_lds<T, OutT, 2, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 48) return launch_skinny_lds<T, OutT, 3, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  return launch_skinny_lds<T, OutT, 4, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
 }
 
-template <typename T, typename OutT, int MT>
-static int launch_skinny(const T* A, long lda, const T* W, long ldw, const float* bias,
-                         const float* residual, long ldr, OutT* C, long ldc, float* partial,
-                         long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  if (skinny_tiles_per_wave(N) == 2)
-    return launch_skinny_tw<T, OutT, MT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  return launch_skinny_tw<T, OutT, MT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-}
-
-template <typename T, typename OutT>
+template <typename T, typename OutT, bool SHUF>
 static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const float* bias,
                            const float* residual, long ldr, OutT* C, long ldc, float* partial,
                            long partial_bytes, int M, int N, int K, int force, hipStream_t stream) {
   constexpr int EPF = Elem<T>::kPerFrag;
-  const bool aligned = K % EPF == 0 && lda % EPF == 0 && ldw % EPF == 0 &&
-                       ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
-  // force: 0 = choose, 1 = generic, 2 = skinny (per-wave), 3 = tiled 128x128, 4 = tiled 128x256,
-  //        5 = skinny (workgroup-cooperative), 6..8 = tiled with 64-byte stages (256x128, 128x128, 128x256)
+  // the shuffled layout exists only for K that is a multiple of 16 bytes and is always aligned
+  const bool aligned = K % EPF == 0 && lda % EPF == 0 && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) &&
+                       (SHUF || ldw % EPF == 0);
+  // force: 0 = choose, 1 = generic, 2 = skinny (per-wave, row-major weights only), 3 = tiled 128x128,
+  //        4 = tiled 128x256, 5 = skinny (workgroup-cooperative)
   if (force == 1 || !aligned) {
     TW_REQUIRE(force <= 1);
+    TW_REQUIRE(!SHUF || K % EPF == 0);
     gemm_generic_kernel<T, OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(A, lda, W, ldw, bias, residual,
-                                                                               ldr, C, ldc, M, N, K);
+                                                                               ldr, C, ldc, M, N, K, SHUF ? 1 : 0);
     return TW_LAUNCH_RESULT();
   }
   if (force == 5 || (force == 0 && M <= 64)) {
     TW_REQUIRE(M <= 64);
-    return launch_skinny_lds_m<T, OutT, false, false>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny_lds_m<T, OutT, false, false, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
   if (force == 2) {
-    TW_REQUIRE(M <= 64);
+    TW_REQUIRE(M <= 64 && !SHUF);
     if (M <= 16) return launch_skinny<T, OutT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
     if (M <= 32) return launch_skinny<T, OutT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
     if (M <= 48) return launch_skinny<T, OutT, 3>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
     return launch_skinny<T, OutT, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
   if (force == 4)
-    return launch_tiled<T, OutT, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
-  if (force == 6)      // 256x128 tile, 64-byte stages
-    return launch_tiled<T, OutT, 4, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
-  if (force == 7)      // 128x128 tile, 64-byte stages
-    return launch_tiled<T, OutT, 2, 2, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
-  if (force == 8)      // 128x256 tile, 64-byte stages
-    return launch_tiled<T, OutT, 2, 4, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
-  return launch_tiled<T, OutT, 2, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+    return launch_tiled<T, OutT, 2, 4, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+  return launch_tiled<T, OutT, 2, 2, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
 }
 
-// C = A W^T (+bias) (+residual). out_f32 != 0: C is float32 whatever the input
-// type (residual stream, logits); else C has the input type. `residual` may be
-// C itself. `partial` is scratch for split-K (tw_linear_workspace_bytes).
-extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const void* W, long ldw,
+template <typename T, typename OutT>
+static int linear_layout(int shuffled, const T* A, long lda, const T* W, long ldw, const float* bias,
+                         const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                         long partial_bytes, int M, int N, int K, int force, hipStream_t stream) {
+  if (shuffled)
+    return linear_dispatch<T, OutT, true>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, force, stream);
+  return linear_dispatch<T, OutT, false>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, force, stream);
+}
+
+// C = A W^T (+bias) (+residual). out_f32 != 0: C is float32 whatever the input type (residual
+// stream, logits); else C has the input type. `residual` may be C itself. `partial` is scratch
+// for split-K (tw_linear_workspace_bytes). shuffled != 0: W is in the shuffled layout and ldw
+// is its number of k-steps, ceil(K / (4 * elements per 16 bytes)).
+extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const void* W, long ldw, int shuffled,
                          const float* bias, const float* residual, long ldr, void* C, long ldc,
                          float* partial, long partial_bytes, int M, int N, int K, int force,
                          hipStream_t stream) {
-  TW_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K && ldw >= K && ldc >= N);
+  TW_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K && ldc >= N);
+  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
+  TW_REQUIRE(shuffled ? ldw >= (K / epf + 3) / 4 && K % epf == 0 : ldw >= K);
   TW_REQUIRE(residual == nullptr || (ldr >= N && out_f32));
   if (M == 0) return 0;
   if (dtype == TW_DTYPE_F32)
-    return linear_dispatch<float, float>((const float*)A, lda, (const float*)W, ldw, bias, residual, ldr,
-                                         (float*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
+    return linear_layout<float, float>(shuffled, (const float*)A, lda, (const float*)W, ldw, bias, residual, ldr,
+                                       (float*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
   if (dtype == TW_DTYPE_BF16) {
     if (out_f32)
-      return linear_dispatch<bf16_t, float>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, residual, ldr,
-                                            (float*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
-    return linear_dispatch<bf16_t, bf16_t>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, residual, ldr,
-                                           (bf16_t*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
+      return linear_layout<bf16_t, float>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, residual, ldr,
+                                          (float*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
+    return linear_layout<bf16_t, bf16_t>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, residual, ldr,
+                                         (bf16_t*)C, ldc, partial, partial_bytes, M, N, K, force, stream);
   }
   return TW_ERR_BAD_ARGUMENT;
 }
@@ -723,45 +803,31 @@ extern "C" int tw_linear_partial_splits(int dtype, int N, int K) {
   return skinny_lds_splits(N, K, epf);
 }
 
+template <typename T, bool SILU>
+static int partials_layout(int shuffled, const T* A, long lda, const T* W, long ldw, float* partial,
+                           long partial_bytes, int M, int N, int K, hipStream_t stream) {
+  if (shuffled)
+    return launch_skinny_lds_m<T, float, SILU, true, true>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+  return launch_skinny_lds_m<T, float, SILU, true, false>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+}
+
 // partial[split][M][N] (float32) = A[:, K range of split] W[:, same]^T for every split; the caller's
 // next kernel adds the splits up (with bias, residual, norm or rotation as it needs).
 // silu != 0: A is [M][2K] = [gate | up] and silu(gate) * up stands in for the activations.
 extern "C" int tw_linear_partials(int dtype, int silu, const void* A, long lda, const void* W, long ldw,
-                                  float* partial, long partial_bytes, int M, int N, int K,
+                                  int shuffled, float* partial, long partial_bytes, int M, int N, int K,
                                   hipStream_t stream) {
-  TW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && ldw >= K && lda >= (silu ? 2L * K : (long)K));
+  TW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && lda >= (silu ? 2L * K : (long)K));
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
-  TW_REQUIRE(K % epf == 0 && lda % epf == 0 && ldw % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
+  TW_REQUIRE(K % epf == 0 && lda % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
+  TW_REQUIRE(shuffled ? ldw >= (K / epf + 3) / 4 : (ldw >= K && ldw % epf == 0));
   if (dtype == TW_DTYPE_F32) {
-    if (silu) return launch_skinny_lds_m<float, float, true, true>((const float*)A, lda, (const float*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
-    return launch_skinny_lds_m<float, float, false, true>((const float*)A, lda, (const float*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+    if (silu) return partials_layout<float, true>(shuffled, (const float*)A, lda, (const float*)W, ldw, partial, partial_bytes, M, N, K, stream);
+    return partials_layout<float, false>(shuffled, (const float*)A, lda, (const float*)W, ldw, partial, partial_bytes, M, N, K, stream);
   }
   if (dtype == TW_DTYPE_BF16) {
-    if (silu) return launch_skinny_lds_m<bf16_t, float, true, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
-    return launch_skinny_lds_m<bf16_t, float, false, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
-  }
-  return TW_ERR_BAD_ARGUMENT;
-}
-
-// C = (silu(gate) * up) W^T (+ residual) for any number of rows with A = [gate | up] ([M][2K]) and
-// 16-byte aligned K: the tiled kernel forms the product while it loads its A tiles.
-extern "C" int tw_linear_silu(int dtype, int out_f32, const void* A, long lda, const void* W, long ldw,
-                              const float* residual, long ldr, void* C, long ldc, int M, int N, int K,
-                              hipStream_t stream) {
-  TW_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= 2L * K && ldw >= K && ldc >= N);
-  TW_REQUIRE(residual == nullptr || (ldr >= N && out_f32));
-  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
-  TW_REQUIRE(K % epf == 0 && lda % epf == 0 && ldw % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
-  if (M == 0) return 0;
-  if (dtype == TW_DTYPE_F32)
-    return launch_tiled<float, float, 2, 2, 8, true>((const float*)A, lda, (const float*)W, ldw, nullptr, residual, ldr,
-                                                  (float*)C, ldc, M, N, K, stream);
-  if (dtype == TW_DTYPE_BF16) {
-    if (out_f32)
-      return launch_tiled<bf16_t, float, 2, 2, 8, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
-                                                     ldr, (float*)C, ldc, M, N, K, stream);
-    return launch_tiled<bf16_t, bf16_t, 2, 2, 8, true>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, nullptr, residual,
-                                                    ldr, (bf16_t*)C, ldc, M, N, K, stream);
+    if (silu) return partials_layout<bf16_t, true>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, partial, partial_bytes, M, N, K, stream);
+    return partials_layout<bf16_t, false>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, partial, partial_bytes, M, N, K, stream);
   }
   return TW_ERR_BAD_ARGUMENT;
 }

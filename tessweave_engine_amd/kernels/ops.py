@@ -146,6 +146,62 @@ def silu_mul(gate_up, out):
     return out
 
 
+class ShuffledWeight:
+    """An [n, k] weight in the kernels' own layout: an exact permutation of the matrix, zero padded.
+
+    Blocks of 16 rows x 4 sixteen-byte chunks, stored in the order MFMA fragments are read:
+    [ceil(n/16)][k_steps][chunk 0..3][row 0..15][elements of 16 bytes]. One wave-wide load of a
+    block is 1 KB of consecutive memory.
+    """
+
+    def __init__(self, data, n, k, k_steps, dtype):
+        self.data, self.n, self.k, self.k_steps, self.dtype = data, n, k, k_steps, dtype
+
+    @property
+    def shape(self):
+        return (self.n, self.k)
+
+    def numel(self):
+        return self.data.numel()
+
+    def element_size(self):
+        return self.data.element_size()
+
+    def to_rows(self):
+        """The matrix back in row-major order (for tests)."""
+        epf = 16 // self.data.element_size()
+        blocks = self.data.view(-1, self.k_steps, 4, 16, epf)
+        return blocks.permute(0, 3, 1, 2, 4).reshape(blocks.shape[0] * 16, self.k_steps * 4 * epf)[:self.n, :self.k]
+
+
+def can_shuffle(weight):
+    return weight.dim() == 2 and weight.shape[1] % (16 // weight.element_size()) == 0
+
+
+def shuffle_weight(weight):
+    """The shuffled copy of a row-major [n, k] weight (k must be a multiple of 16 bytes)."""
+    _need(can_shuffle(weight), "only weights whose rows are a multiple of 16 bytes can be shuffled")
+    n, k = weight.shape
+    epf = 16 // weight.element_size()
+    k_steps = (k // epf + 3) // 4
+    n_pad, k_pad = (n + 15) // 16 * 16, k_steps * 4 * epf
+    if (n_pad, k_pad) != (n, k):
+        padded = weight.new_zeros((n_pad, k_pad))
+        padded[:n, :k] = weight
+    else:
+        padded = weight
+    data = padded.view(n_pad // 16, 16, k_steps, 4, epf).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+    return ShuffledWeight(data, n, k, k_steps, weight.dtype)
+
+
+def _weight_args(weight):
+    """(n, k, pointer, ldw, shuffled flag, dtype) of a row-major tensor or a ShuffledWeight."""
+    if isinstance(weight, ShuffledWeight):
+        return weight.n, weight.k, _dev(weight.data), weight.k_steps, 1, weight.dtype
+    n, k, ldw = _rows(weight, "weight")
+    return n, k, _dev(weight), ldw, 0, weight.dtype
+
+
 def linear_workspace_bytes(dtype, max_rows, n, k):
     return int(library().tw_linear_workspace_bytes(dtype_id(dtype), int(max_rows), int(n), int(k)))
 
@@ -162,36 +218,16 @@ def linear_partials(x, weight, partial, silu_gate=False):
     silu(gate) * up (rounded to x's type) stands in for the activations.
     """
     m, kx, lda = _rows(x, "x")
-    n, k, ldw = _rows(weight, "weight")
+    n, k, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
     _need(kx == (2 * k if silu_gate else k), "linear_partials shapes do not agree")
-    _need(x.dtype == weight.dtype and 1 <= m <= 64, "linear_partials takes 1..64 rows of the weight's type")
-    splits = linear_partial_splits(weight.dtype, n, k)
+    _need(x.dtype == w_dtype and 1 <= m <= 64, "linear_partials takes 1..64 rows of the weight's type")
+    splits = linear_partial_splits(w_dtype, n, k)
     _need(splits > 0, "linear_partials needs K to be a multiple of 16 bytes")
     _need(partial.is_contiguous() and tuple(partial.shape) == (splits, m, n), f"partial must be [{splits}, {m}, {n}]")
-    check(library().tw_linear_partials(dtype_id(x.dtype), 1 if silu_gate else 0, _dev(x), lda, _dev(weight), ldw,
+    check(library().tw_linear_partials(dtype_id(x.dtype), 1 if silu_gate else 0, _dev(x), lda, w_ptr, ldw, shuffled,
                                        _dev(partial, torch.float32, "partial"), partial.numel() * 4, m, n, k,
                                        _stream()), "linear_partials")
     return partial
-
-
-def linear_silu(gate_up, weight, out, residual=None):
-    """out = (silu(gate) * up) @ weight.T (+ residual) with gate_up = [gate | up] ([m, 2k]); K 16-byte aligned."""
-    m, k2, lda = _rows(gate_up, "gate_up")
-    n, k, ldw = _rows(weight, "weight")
-    mo, no, ldc = _rows(out, "out")
-    _need(k2 == 2 * k and (mo, no) == (m, n) and gate_up.dtype == weight.dtype, "linear_silu shapes or types do not agree")
-    _need(k % (8 if weight.dtype == torch.bfloat16 else 4) == 0, "linear_silu needs K to be a multiple of 16 bytes")
-    out_f32 = out.dtype == torch.float32
-    _need(out_f32 or out.dtype == weight.dtype, "out must be float32 or the input type")
-    ldr = 0
-    if residual is not None:
-        _need(out_f32, "a residual needs a float32 output")
-        mr, nr, ldr = _rows(residual, "residual")
-        _need((mr, nr) == (m, n), "residual shape differs from the output")
-    check(library().tw_linear_silu(dtype_id(weight.dtype), 1 if out_f32 else 0, _dev(gate_up), lda, _dev(weight), ldw,
-                                   _dev(residual, torch.float32, "residual") if residual is not None else None, ldr,
-                                   _dev(out), ldc, m, n, k, _stream()), "linear_silu")
-    return out
 
 
 GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY_COOP = 0, 1, 2, 3, 4, 5
@@ -200,15 +236,15 @@ GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY_C
 def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_AUTO):
     """out = x @ weight.T (+ bias) (+ residual).
 
-    x [m, k] and weight [n, k] share a type (float32 or bfloat16); out is float32
-    (required with a residual; the residual may be `out` itself) or that type.
-    bias is float32 [n]; workspace is a float32/byte scratch tensor for split-K.
+    x [m, k] and weight [n, k] (a row-major tensor or a ShuffledWeight) share a type (float32 or
+    bfloat16); out is float32 (required with a residual; the residual may be `out` itself) or that
+    type. bias is float32 [n]; workspace is a float32/byte scratch tensor for split-K.
     """
     m, k, lda = _rows(x, "x")
-    n, k2, ldw = _rows(weight, "weight")
+    n, k2, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
     mo, no, ldc = _rows(out, "out")
     _need(k == k2 and mo == m and no == n, f"linear shapes do not agree: x {tuple(x.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
-    _need(x.dtype == weight.dtype, "x and weight types differ")
+    _need(x.dtype == w_dtype, "x and weight types differ")
     out_f32 = out.dtype == torch.float32
     _need(out_f32 or out.dtype == x.dtype, "out must be float32 or the input type")
     ldr = 0
@@ -221,7 +257,7 @@ def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_
     ws_ptr, ws_bytes = None, 0
     if workspace is not None:
         ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
-    check(library().tw_linear(dtype_id(x.dtype), 1 if out_f32 else 0, _dev(x), lda, _dev(weight), ldw,
+    check(library().tw_linear(dtype_id(x.dtype), 1 if out_f32 else 0, _dev(x), lda, w_ptr, ldw, shuffled,
                               _dev(bias, torch.float32, "bias") if bias is not None else None,
                               _dev(residual, torch.float32, "residual") if residual is not None else None, ldr,
                               _dev(out), ldc, ws_ptr, ws_bytes, m, n, k, int(force), _stream()), "linear")

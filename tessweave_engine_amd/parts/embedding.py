@@ -43,11 +43,16 @@ class OutputHead(Part):
         return [TensorSpec(self.name + ".weight", (self.vocab, self.hidden), MATRIX, NORMAL)]
 
     def bind(self, tensors, dtype, device):
-        if self.tied_to is None:
-            self.weight = tensors.pop(self.name + ".weight").contiguous()
+        # The head's matrix is kept in the matrix kernels' shuffled layout; a tied head makes its own
+        # shuffled copy of the embedding (the gather reads rows, the head streams MFMA blocks).
+        source = self.tied_to.weight if self.tied_to is not None else tensors.pop(self.name + ".weight").contiguous()
+        if torch.device(device).type == "cuda" and ops.can_shuffle(source):
+            self.weight = ops.shuffle_weight(source)
+        else:
+            self.weight = source
 
     def matrix(self):
-        return self.tied_to.weight if self.tied_to is not None else self.weight
+        return self.weight
 
     def forward(self, ctx, h):
         # The logits live in a shared scratch buffer: they are valid until the next step.

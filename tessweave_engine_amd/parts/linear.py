@@ -42,15 +42,23 @@ class Linear(Part):
         weights = [tensors.pop(name + ".weight") for name in self.names]
         biases = [tensors.pop(name + ".bias") for name in self.names] if self.has_bias else []
         if self.packed and len(weights) > 1:
-            self.weights = [torch.cat(weights, 0).contiguous()]
-            self.biases = [torch.cat(biases, 0).contiguous()] if biases else []
-        else:
-            self.weights = [w.contiguous() for w in weights]
-            self.biases = [b.contiguous() for b in biases]
+            weights = [torch.cat(weights, 0)]
+            biases = [torch.cat(biases, 0)] if biases else []
+        # On a GPU the matrices are kept in the kernels' shuffled layout (an exact permutation)
+        # whenever their rows are a multiple of 16 bytes; otherwise row-major for the generic kernel.
+        on_gpu = torch.device(device).type == "cuda"
+        self.weights = [ops.shuffle_weight(w.contiguous()) if on_gpu and ops.can_shuffle(w) else w.contiguous()
+                        for w in weights]
+        self.biases = [b.contiguous() for b in biases]
         del weights, biases
 
     def weight_bytes(self):
         return sum(w.numel() * w.element_size() for w in self.weights)
+
+    def row_major(self, i=0):
+        """Weight i as a row-major [out, in] tensor (a copy if it is held shuffled)."""
+        w = self.weights[i]
+        return w.to_rows() if isinstance(w, ops.ShuffledWeight) else w
 
     def forward(self, ctx, x, out, residual=None):
         """out[:, columns] = x @ W.T (+ bias) (+ residual); out may be float32 or x's type."""

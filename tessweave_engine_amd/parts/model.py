@@ -68,6 +68,7 @@ class DecoderModel(Part):
             for value in vars(part).values():
                 items = value if isinstance(value, (list, tuple)) else [value]
                 for t in items:
+                    t = getattr(t, "data", t) if type(t).__name__ == "ShuffledWeight" else t
                     if isinstance(t, torch.Tensor) and t.is_floating_point() and id(t) not in seen and t.dim() >= 1:
                         if getattr(part, "inv_freq", None) is t:
                             continue

@@ -158,7 +158,14 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
         forces += [ops.GEMM_SKINNY, ops.GEMM_SKINNY_COOP]
     scale = math.sqrt(k) * 0.05
     t = dict(atol=2e-5 * scale, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2 * scale, rtol=2e-2)
-    for force in forces:
+    shuffled = ops.shuffle_weight(w)
+    torch.testing.assert_close(shuffled.to_rows(), w, atol=0, rtol=0)          # an exact permutation
+    for force in forces + [("shuffled", f) for f in (ops.GEMM_AUTO, ops.GEMM_GENERIC, ops.GEMM_TILED, ops.GEMM_TILED_WIDE)
+                           + ((ops.GEMM_SKINNY_COOP,) if m <= 64 else ())]:
+        wt = w
+        if isinstance(force, tuple):
+            wt, force = shuffled, force[1]
+        w_rows, w = w, wt
         # plain output in the input type
         out = torch.full((m, n), float("nan"), dtype=dtype, device=device)
         ops.linear(x, w, out, workspace=ws, force=force)
@@ -173,6 +180,7 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
         ops.linear(x, w, out2, bias=bias, force=force)
         torch.testing.assert_close(out2.double().cpu(), want + bias.double().cpu(),
                                    atol=t["atol"] if dtype == torch.float32 else 2e-5 * scale + 1e-5, rtol=1e-5)
+        w = w_rows
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -186,6 +194,11 @@ def test_linear_partials_and_fused_silu(ops, device, dtype, m, n, k):
     want = x.double().cpu() @ w.double().cpu().T
     scale = math.sqrt(k) * 0.05
     torch.testing.assert_close(part.double().sum(0).cpu(), want, atol=3e-5 * scale, rtol=1e-5)
+    rows_sum = part.sum(0).clone()
+    w = ops.shuffle_weight(w)                    # the same from the shuffled layout: identical bits
+    part.fill_(float("nan"))
+    ops.linear_partials(x, w, part)
+    torch.testing.assert_close(part.sum(0), rows_sum, atol=0, rtol=0)
     # [gate | up] input: silu(gate) * up, rounded to the input type, is what gets multiplied
     gu = rand((m, 2 * k), dtype, device, 1.0, seed=3)
     act = torch.empty(m, k, dtype=dtype, device=device)
@@ -194,21 +207,6 @@ def test_linear_partials_and_fused_silu(ops, device, dtype, m, n, k):
     plain_sum = part.sum(0).clone()
     ops.linear_partials(gu, w, part, silu_gate=True)
     torch.testing.assert_close(part.sum(0), plain_sum, atol=0, rtol=0)
-
-
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,n,k", [(65, 48, 64), (200, 389, 320), (300, 130, 1032)])
-def test_linear_silu_many_rows(ops, device, dtype, m, n, k):
-    gu = rand((m, 2 * k), dtype, device, 1.0, seed=3)
-    w = rand((n, k), dtype, device, 0.05, seed=2)
-    res = rand((m, n), torch.float32, device, 1.0, seed=4)
-    act = torch.empty(m, k, dtype=dtype, device=device)
-    ops.silu_mul(gu, act)
-    want = res.clone()
-    ops.linear(act, w, want, residual=want, force=ops.GEMM_TILED)
-    got = res.clone()
-    ops.linear_silu(gu, w, got, residual=got)
-    torch.testing.assert_close(got, want, atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
