@@ -2,17 +2,22 @@
 // A and W are both contiguous along K (the checkpoint's [out, in] layout), in
 // float32 or bfloat16; accumulation is float32 on the MFMA units (true float32
 // MFMA for float32 inputs, no reduced-precision matrix mode). Three kernels:
-//   gemm_tiled   - many rows (prompt portions): LDS-staged 32x32 MFMA tiles
-//   gemm_skinny  - few rows (decode): weights streamed once from HBM straight
-//                  into 16x16 MFMA fragments, split over K when N is small
-//   gemm_generic - any K (rows not 16-byte aligned): one output per thread
+//   gemm_tiled      - many rows (prompt portions): LDS-staged 32x32 MFMA tiles
+//   gemm_skinny_lds - few rows (decode): weights streamed once from HBM straight
+//                     into 16x16 MFMA fragments, split over K when N is small
+//   gemm_generic    - any K (rows not 16-byte aligned): one output per thread
 //
 // Weight layouts. Row-major [N][K] as in the checkpoint, or SHUFFLED (an exact permutation,
 // zero padded): blocks of 16 rows x 4 sixteen-byte chunks stored in the order the MFMA units
 // read them, [N/16][K/(4*EPF)][chunk 0..3][row 0..15][EPF]. Element (n, k) is at
 //   ((n/16 * k_steps + (k/EPF)/4) * 64 + ((k/EPF)%4) * 16 + n%16) * EPF + k%EPF.
-// A wave's load of one block is 1 KB of consecutive memory: the decode kernels stream weights
-// as whole cache lines and may skip the caches (non-temporal), the tiled kernel copies blocks.
+// A wave's load of one block is 1 KB of consecutive memory: the decode kernel streams weights
+// as whole cache lines past the caches (non-temporal), the tiled kernel copies blocks.
+//
+// GLU (gated linear unit) form: the N rows of W are the gate and up projections interleaved in
+// blocks of 16 rows (gate rows 16j.., then up rows 16j.., for j = 0, 1, ...). The kernels form
+// C[M, N/2][.., 16j + i] = silu(gate_j[i]) * up_j[i] in their epilogues, in float32 from the
+// accumulators, so the [M, N] intermediate never reaches memory.
 #include "tw_common.h"
 
 // element offset of (row n, 16-byte chunk c) in the shuffled layout
@@ -26,17 +31,7 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p
   return __builtin_nontemporal_load(reinterpret_cast<const typename Elem<T>::Frag*>(p));
 }
 
-// silu(g) * u on a fragment pair, float32 arithmetic, one rounding to T
-template <typename T>
-__device__ __forceinline__ typename Elem<T>::Frag tw_silu_mul_frag(typename Elem<T>::Frag gf, typename Elem<T>::Frag uf) {
-  typename Elem<T>::Frag out;
-#pragma unroll
-  for (int e = 0; e < Elem<T>::kPerFrag; ++e) {
-    const float gv = tw_to_float(gf[e]), uv = tw_to_float(uf[e]);
-    out[e] = tw_from_float<T>(gv / (1.0f + expf(-gv)) * uv);
-  }
-  return out;
-}
+__device__ __forceinline__ float tw_silu(float g) { return g / (1.0f + expf(-g)); }
 
 // =====================================================================================
 // Tiled kernel. Workgroup = 4 waves in a 2x2 grid, wave tile (32*WM) x (32*WN).
@@ -47,10 +42,8 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_silu_mul_frag(typename Elem
 // =====================================================================================
 #define TW_LDS_ROW 144
 
-// SILU: A is [M][2K] = [gate | up] and silu(gate) * up (rounded to T) stands in for the activations.
-// KCH: 16-byte chunks of K per row and stage (8: 128 bytes, 4: 64 bytes).
-// SHUF: W is in the shuffled layout and ldw is its k_steps.
-template <typename T, typename OutT, int WM, int WN, int KCH, bool SILU, bool SHUF>
+// SHUF: W is in the shuffled layout and ldw is its k_steps. GLU: see the top of the file.
+template <typename T, typename OutT, int WM, int WN, bool SHUF, bool GLU>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A, long lda,
                                                          const T* __restrict__ W, long ldw,
                                                          const float* __restrict__ bias,
@@ -59,6 +52,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
                                                          int n_blocks) {
   typedef typename Elem<T>::Frag Frag;
   constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr int KCH = 8;                                    // 16-byte chunks of K per row and stage
   constexpr int BK = KCH * EPF;
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int LROW = KCH * 16 + 16;                       // LDS bytes per row of a stage, padded
@@ -137,10 +131,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
     const T* ab = a_tile + (size_t)kt * BK;
     const T* wb = SHUF ? w_tile + (size_t)kt * SPT * 64 * EPF : w_tile + (size_t)kt * BK;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      if (SILU) a_reg[i] = tw_silu_mul_frag<T>(tw_load_frag(ab + a_off[i]), tw_load_frag(ab + K + a_off[i]));
-      else a_reg[i] = tw_load_frag(ab + a_off[i]);
-    }
+    for (int i = 0; i < A_LOADS; ++i) a_reg[i] = tw_load_frag(ab + a_off[i]);
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) w_reg[i] = tw_load_frag(wb + w_off[i]);
   };
@@ -152,10 +143,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
       const T* wb = SHUF ? w_tile + (size_t)kt * SPT * 64 * EPF : w_tile + (size_t)kt * BK;
       const bool ok = kt * BK + kc_mine * EPF < K;
 #pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) {
-        if (SILU) a_reg[i] = ok ? tw_silu_mul_frag<T>(tw_load_frag(ab + a_off[i]), tw_load_frag(ab + K + a_off[i])) : Elem<T>::zero();
-        else a_reg[i] = ok ? tw_load_frag(ab + a_off[i]) : Elem<T>::zero();
-      }
+      for (int i = 0; i < A_LOADS; ++i) a_reg[i] = ok ? tw_load_frag(ab + a_off[i]) : Elem<T>::zero();
 #pragma unroll
       for (int i = 0; i < W_LOADS; ++i) {
         const bool w_ok = SHUF ? kt * SPT + w_ks[i] < k_steps_w : ok;     // the shuffled layout is zero padded
@@ -244,6 +232,40 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 #pragma unroll
       for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * g + (e % 4)) * EROW + j * 32 + r] = acc[i][j][e];
     __syncthreads();
+    if (GLU) {
+      // a wave tile's columns are [gate 16 | up 16] pairs; a lane forms 8 outputs of one row
+      constexpr int GPR = WCOLS / 16;                         // 8-output groups per row
+#pragma unroll
+      for (int q = lane; q < 32 * GPR; q += 64) {
+        const int lr = q / GPR, og = q % GPR;
+        const int lc = (og >> 1) * 32 + (og & 1) * 8;         // gate columns lc.., up columns lc + 16..
+        const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
+        if (row >= M || col + 24 > N) continue;               // N is a multiple of 32: groups are whole
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float gv = stage[lr * EROW + lc + e], uv = stage[lr * EROW + lc + 16 + e];
+          if (bias) { gv += bias[col + e]; uv += bias[col + 16 + e]; }
+          v[e] = tw_silu(gv) * uv;
+        }
+        OutT* dst = C + (size_t)row * ldc + (n0 + wn0) / 2 + (og >> 1) * 16 + (og & 1) * 8;
+        if (ldc % 8 == 0 && (uintptr_t)C % 16 == 0) {
+          if (sizeof(OutT) == 4) {
+            *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
+          } else {
+            bf16x8 o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
+            *reinterpret_cast<bf16x8*>(dst) = o;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dst[e] = tw_from_float<OutT>(v[e]);
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int q = lane; q < 32 * CPR; q += 64) {
       const int lr = q / CPR, lc = (q % CPR) * 8;
@@ -288,141 +310,22 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 }
 
 // =====================================================================================
-// Skinny kernel: M <= 16*MT rows. Each wave owns 16 output columns (16 rows of
-// W) and one K range; it loads weight fragments straight from global memory
-// (every weight byte is read by exactly one wave, 64 contiguous bytes per row
-// per load instruction) and the matching activation fragments from L2.
-// SPLITS == 1: the epilogue runs here. SPLITS > 1: float32 partial sums go to
-// `partial[split][M][N]` and `splitk_reduce_kernel` finishes, always in the
-// same order, so results do not depend on timing.
-// =====================================================================================
-template <typename T, typename OutT, int MT, int TW, int U>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const T* __restrict__ A, long lda,
-                                                          const T* __restrict__ W, long ldw,
-                                                          const float* __restrict__ bias,
-                                                          const float* residual, long ldr, OutT* C,
-                                                          long ldc, float* __restrict__ partial, int M,
-                                                          int N, int K, int n_groups, int splits) {
-  // A wave owns TW tiles of 16 output columns (16*TW rows of W) and one K range.
-  typedef typename Elem<T>::Frag Frag;
-  constexpr int EPF = Elem<T>::kPerFrag;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int unit = blockIdx.x * 4 + wave;
-  if (unit >= n_groups * splits) return;
-  const int group = unit % n_groups, split = unit / n_groups;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = group * 16 * TW;
-
-  const int chunks = K / EPF;                              // 16-byte chunks per row
-  const int steps = (chunks + 3) / 4;                      // MFMA steps over all of K
-  const int steps_per_split = (steps + splits - 1) / splits;
-  const int step_begin = split * steps_per_split;
-  const int step_end = min(steps, step_begin + steps_per_split);
-
-  f32x4 acc[TW][MT];
-#pragma unroll
-  for (int t = 0; t < TW; ++t)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // Rows past the end are clamped to the last valid row: what they produce is
-  // never stored, and the main loop needs no per-load predicate.
-  const T* w_row[TW];
-#pragma unroll
-  for (int t = 0; t < TW; ++t) w_row[t] = W + (size_t)min(n0 + t * 16 + r, N - 1) * ldw + g * EPF;
-  const T* a_row[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) a_row[mt] = A + (size_t)min(mt * 16 + r, M - 1) * lda + g * EPF;
-
-  // Two register stages of U MFMA steps each: the loads of one stage are in
-  // flight while the other is multiplied.
-  Frag wf[2][U][TW], xf[2][U][MT];
-  auto load = [&](const int buf, int s0) {          // all U steps lie inside [step_begin, full_end)
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const size_t off = (size_t)(s0 + u) * 4 * EPF;
-#pragma unroll
-      for (int t = 0; t < TW; ++t) wf[buf][u][t] = tw_load_frag(w_row[t] + off);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xf[buf][u][mt] = tw_load_frag(a_row[mt] + off);
-    }
-  };
-  auto multiply = [&](const int buf) {
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int t = 0; t < TW; ++t)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) tw_mma16(acc[t][mt], wf[buf][u][t], xf[buf][u][mt]);
-  };
-  // steps whose four chunks all exist, in whole stages
-  const int whole_steps = min(step_end, chunks / 4);
-  const int n_stages = whole_steps > step_begin ? (whole_steps - step_begin) / U : 0;
-  const int full_end = step_begin + n_stages * U;
-  if (n_stages > 0) {
-    load(0, step_begin);
-    int s0 = step_begin;
-    for (int i = 0; i + 2 <= n_stages; i += 2, s0 += 2 * U) {
-      load(1, s0 + U);
-      multiply(0);
-      if (i + 2 < n_stages) load(0, s0 + 2 * U);
-      multiply(1);
-    }
-    if (n_stages & 1) multiply(0);
-  }
-  // tail: single steps with per-chunk predicates
-  for (int s = full_end; s < step_end; ++s) {
-    const int chunk = s * 4 + g;
-    const bool ok = chunk < chunks;
-    const size_t off = (size_t)s * 4 * EPF;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const Frag af = ok ? tw_load_frag(a_row[mt] + off) : Elem<T>::zero();
-#pragma unroll
-      for (int t = 0; t < TW; ++t) {
-        const Frag wfrag = ok ? tw_load_frag(w_row[t] + off) : Elem<T>::zero();
-        tw_mma16(acc[t][mt], wfrag, af);
-      }
-    }
-  }
-
-  // acc[t][mt][j] = sum_k W[n0 + 16 t + 4g + j][k] * A[16 mt + r][k]
-#pragma unroll
-  for (int t = 0; t < TW; ++t)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int row = mt * 16 + r;
-      if (row >= M) continue;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int col = n0 + t * 16 + 4 * g + j;
-        if (col >= N) continue;
-        if (splits > 1) {
-          partial[((size_t)split * M + row) * N + col] = acc[t][mt][j];
-        } else {
-          float v = acc[t][mt][j] + (bias ? bias[col] : 0.f);
-          if (residual) v += residual[(size_t)row * ldr + col];
-          C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
-        }
-      }
-    }
-}
-
-// =====================================================================================
-// Skinny kernel, workgroup-cooperative form. The 4 waves of a workgroup own 4
+// Skinny kernel (M <= 16*MT rows), workgroup-cooperative. The 4 waves of a workgroup own 4
 // neighbouring tiles of 16 output columns and the SAME K range. Per stage of U
 // MFMA steps the workgroup copies the activations' K slice [16*MT rows][U*64 B]
 // to LDS once (instead of every wave reading it from L2); each wave streams its
-// own 16 weight rows from global memory into registers. Two stages in flight.
+// own 16 weight rows from global memory into registers (every weight byte is read by exactly
+// one wave). Two stages in flight. splits == 1: the epilogue runs here. splits > 1: float32
+// partial sums go to partial[split][M][N] and splitk_reduce_kernel (or the caller's next
+// kernel) adds them, always in the same order, so results do not depend on timing.
 // =====================================================================================
 #define TW_XROW(U) ((U) * 64 + 16)          /* LDS bytes per activation row of a stage, padded */
 
-// SILU: the activations are [M][2K] = [gate | up]; the kernel multiplies silu(gate) * up by W
-// (the rounded product is what a separate SiLU-multiply kernel would have written).
 // PARTIAL: always write float32 partial sums partial[split][M][N] (splits >= 1), no epilogue.
 // SHUF: W is in the shuffled layout (ldw = its k_steps): every weight load is 1 KB of consecutive
 // memory, needs no predicate (the layout is zero padded) and bypasses the caches.
-template <typename T, typename OutT, int MT, int U, bool SILU, bool PARTIAL, bool SHUF>
+// GLU (splits == 1 only): the workgroup's 4 tiles are gate, up, gate, up; C gets 32 columns.
+template <typename T, typename OutT, int MT, int U, bool PARTIAL, bool SHUF, bool GLU>
 __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restrict__ A, long lda,
                                                               const T* __restrict__ W, long ldw,
                                                               const float* __restrict__ bias,
@@ -466,7 +369,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
     x_dst[i] = row * XROW + c * 16;
   }
 
-  Frag wf[2][U], xg[XLOADS], xu[SILU ? XLOADS : 1];
+  Frag wf[2][U], xg[XLOADS];
   auto load_w = [&](const int buf, int s0, bool whole) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -486,19 +389,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
       const int chunk = s0 * 4 + x_chunk[i];
-      if (whole || (chunk < step_end * 4 && chunk < chunks)) {
+      if (whole || (chunk < step_end * 4 && chunk < chunks))
         xg[i] = tw_load_frag(x_src[i] + (size_t)chunk * EPF);
-        if (SILU) xu[i] = tw_load_frag(x_src[i] + (size_t)K + (size_t)chunk * EPF);
-      } else {
+      else
         xg[i] = Elem<T>::zero();
-        if (SILU) xu[i] = Elem<T>::zero();
-      }
     }
   };
   auto store_x = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i)
-      *reinterpret_cast<Frag*>(lds + buf * XSTAGE + x_dst[i]) = SILU ? tw_silu_mul_frag<T>(xg[i], xu[i]) : xg[i];
+      *reinterpret_cast<Frag*>(lds + buf * XSTAGE + x_dst[i]) = xg[i];
   };
   auto multiply = [&](const int buf) {
 #pragma unroll
@@ -542,6 +442,31 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
     }
   }
 
+  // acc[mt][j] = sum_k W[n0 + 4g + j][k] * A[16 mt + r][k]
+  if (GLU) {
+    // the waves swap their tiles through LDS (every wave is past its last LDS read: the loop
+    // ends with a barrier), then each thread forms outputs from a (gate, up) pair
+    constexpr int GROW = 17;                                  // floats per staged row, padded
+    static_assert(4 * MT * 16 * GROW * 4 <= 2 * XSTAGE, "the GLU exchange fits the pipeline's LDS");
+    float* ex = reinterpret_cast<float*>(lds);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = n0 + 4 * g + j;
+        ex[(wave * MT * 16 + mt * 16 + r) * GROW + 4 * g + j] = acc[mt][j] + (bias && col < N ? bias[col] : 0.f);
+      }
+    __syncthreads();
+    for (int o = tid; o < MT * 16 * 32; o += 256) {
+      const int row = o >> 5, c = o & 31, pair = c >> 4, i = c & 15;
+      const int col = group * 32 + c;                         // output column
+      if (row >= M || col >= N / 2) continue;
+      const float gv = ex[((2 * pair) * MT * 16 + row) * GROW + i];
+      const float uv = ex[((2 * pair + 1) * MT * 16 + row) * GROW + i];
+      C[(size_t)row * ldc + col] = tw_from_float<OutT>(tw_silu(gv) * uv);
+    }
+    return;
+  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int row = mt * 16 + r;
@@ -578,22 +503,38 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int spli
 // =====================================================================================
 // Generic kernel: any K. One thread per output element, float32 accumulation.
 // =====================================================================================
-template <typename T, typename OutT>
-__global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* __restrict__ W, long ldw,
-                                    const float* __restrict__ bias, const float* residual, long ldr,
-                                    OutT* C, long ldc, int M, int N, int K, int shuffled) {
-  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= (long)M * N) return;
-  const int row = (int)(i / N), col = (int)(i % N);
-  const T* a = A + (size_t)row * lda;
-  const T* w = W + (size_t)col * ldw;
+template <typename T>
+__device__ __forceinline__ float tw_generic_dot(const T* a, const T* W, long ldw, int col, int K, int shuffled) {
   constexpr int EPF = Elem<T>::kPerFrag;
   float v = 0.f;
   if (shuffled) {
     for (int k = 0; k < K; ++k)
       v = fmaf(tw_to_float(a[k]), tw_to_float(W[tw_shuffled_chunk(col, k / EPF, (int)ldw, EPF) + k % EPF]), v);
-  } else
-  for (int k = 0; k < K; ++k) v = fmaf(tw_to_float(a[k]), tw_to_float(w[k]), v);
+  } else {
+    const T* w = W + (size_t)col * ldw;
+    for (int k = 0; k < K; ++k) v = fmaf(tw_to_float(a[k]), tw_to_float(w[k]), v);
+  }
+  return v;
+}
+
+// glu: C has N / 2 columns (see the top of the file)
+template <typename T, typename OutT>
+__global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* __restrict__ W, long ldw,
+                                    const float* __restrict__ bias, const float* residual, long ldr,
+                                    OutT* C, long ldc, int M, int N, int K, int shuffled, int glu) {
+  const int n_out = glu ? N / 2 : N;
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)M * n_out) return;
+  const int row = (int)(i / n_out), col = (int)(i % n_out);
+  const T* a = A + (size_t)row * lda;
+  if (glu) {
+    const int gate = (col / 16) * 32 + col % 16, up = gate + 16;
+    const float gv = tw_generic_dot(a, W, ldw, gate, K, shuffled) + (bias ? bias[gate] : 0.f);
+    const float uv = tw_generic_dot(a, W, ldw, up, K, shuffled) + (bias ? bias[up] : 0.f);
+    C[(size_t)row * ldc + col] = tw_from_float<OutT>(tw_silu(gv) * uv);
+    return;
+  }
+  float v = tw_generic_dot(a, W, ldw, col, K, shuffled);
   if (bias) v += bias[col];
   if (residual) v += residual[(size_t)row * ldr + col];
   C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
@@ -602,7 +543,7 @@ __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* 
 // =====================================================================================
 // Host side
 // =====================================================================================
-template <typename T, typename OutT, int WM, int WN, bool SHUF>
+template <typename T, typename OutT, int WM, int WN, bool SHUF, bool GLU>
 static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
                         const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
                         hipStream_t stream) {
@@ -618,7 +559,7 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
   const size_t pipeline_bytes = 2 * (size_t)(BM + BN) * (KCH * 16 + 16);
   const size_t epilogue_bytes = 4 * 32 * (size_t)(32 * WN + 4) * 4;
   const size_t lds_bytes = pipeline_bytes > epilogue_bytes ? pipeline_bytes : epilogue_bytes;
-  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, KCH, false, SHUF>;
+  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, SHUF, GLU>;
   static bool attribute_set = false;   // per instantiation
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -631,22 +572,9 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
   return TW_LAUNCH_RESULT();
 }
 
-// Output tiles per wave of the per-wave skinny kernel (they share the activation fragments).
-static int skinny_tiles_per_wave(int N) { return N >= 16384 ? 2 : 1; }
-
-// How many K ranges the skinny kernels use for an [N, K] weight: enough waves to fill 256 CUs
-// several times over, each range at least 16 MFMA steps long. The choice depends on N and K
-// only, never on the rows of a batch.
-static int skinny_splits(int N, int K, int epf) {
-  const int groups = tw_div_up(N, 16 * skinny_tiles_per_wave(N));
-  const int steps = tw_div_up(K / epf, 4);
-  int splits = tw_div_up(2048, groups);
-  const int max_by_k = steps / 16 > 0 ? steps / 16 : 1;
-  if (splits > max_by_k) splits = max_by_k;
-  if (splits > 16) splits = 16;
-  return splits < 1 ? 1 : splits;
-}
-
+// How many K ranges the skinny kernel uses for an [N, K] weight: enough workgroups to fill 256
+// CUs twice, each range at least 16 MFMA steps long. The choice depends on N and K only, never
+// on the rows of a batch.
 static int skinny_lds_splits(int N, int K, int epf) {
   const int groups = tw_div_up(N, 64);
   const int steps = tw_div_up(K / epf, 4);
@@ -661,54 +589,24 @@ extern "C" long tw_linear_workspace_bytes(int dtype, int max_rows, int N, int K)
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
   if (K % epf) return 0;
   const int rows = max_rows < 64 ? max_rows : 64;
-  int splits = skinny_splits(N, K, epf);
-  const int coop = skinny_lds_splits(N, K, epf);
-  if (coop > splits) splits = coop;
+  const int splits = skinny_lds_splits(N, K, epf);
   return splits > 1 ? (long)splits * rows * N * 4 : 0;
 }
 
-template <typename T, typename OutT, int MT, int TW>
-static int launch_skinny_tw(const T* A, long lda, const T* W, long ldw, const float* bias,
-                            const float* residual, long ldr, OutT* C, long ldc, float* partial,
-                            long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  constexpr int EPF = Elem<T>::kPerFrag;
-  constexpr int U = (MT * TW <= 2) ? 8 : 4;
-  const int groups = tw_div_up(N, 16 * TW);
-  int splits = skinny_splits(N, K, EPF);
-  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) splits = 1;
-  const int units = groups * splits;
-  gemm_skinny_kernel<T, OutT, MT, TW, U><<<tw_div_up(units, 4), 256, 0, stream>>>(
-      A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
-  int err = TW_LAUNCH_RESULT();
-  if (err || splits == 1) return err;
-  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
-                                                                             ldr, C, ldc, M, N);
-  return TW_LAUNCH_RESULT();
-}
-
-template <typename T, typename OutT, int MT>
-static int launch_skinny(const T* A, long lda, const T* W, long ldw, const float* bias,
-                         const float* residual, long ldr, OutT* C, long ldc, float* partial,
-                         long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  if (skinny_tiles_per_wave(N) == 2)
-    return launch_skinny_tw<T, OutT, MT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  return launch_skinny_tw<T, OutT, MT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-}
-
-template <typename T, typename OutT, int MT, bool SILU, bool PARTIAL, bool SHUF>
+template <typename T, typename OutT, int MT, bool PARTIAL, bool SHUF, bool GLU>
 static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const float* bias,
                              const float* residual, long ldr, OutT* C, long ldc, float* partial,
                              long partial_bytes, int M, int N, int K, hipStream_t stream) {
   constexpr int EPF = Elem<T>::kPerFrag;
   constexpr int U = MT == 1 ? 8 : 4;
   const int groups = tw_div_up(N, 64);
-  int splits = skinny_lds_splits(N, K, EPF);
+  int splits = GLU ? 1 : skinny_lds_splits(N, K, EPF);
   if (PARTIAL) {
     TW_REQUIRE(partial != nullptr && partial_bytes >= (long)splits * M * N * 4);
   } else if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) {
     splits = 1;
   }
-  gemm_skinny_lds_kernel<T, OutT, MT, U, SILU, PARTIAL, SHUF><<<groups * splits, 256, 0, stream>>>(
+  gemm_skinny_lds_kernel<T, OutT, MT, U, PARTIAL, SHUF, GLU><<<groups * splits, 256, 0, stream>>>(
       A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
   int err = TW_LAUNCH_RESULT();
   if (err || splits == 1 || PARTIAL) return err;
@@ -717,47 +615,41 @@ static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const f
   return TW_LAUNCH_RESULT();
 }
 
-template <typename T, typename OutT, bool SILU, bool PARTIAL, bool SHUF>
+template <typename T, typename OutT, bool PARTIAL, bool SHUF, bool GLU>
 static int launch_skinny_lds_m(const T* A, long lda, const T* W, long ldw, const float* bias,
                                const float* residual, long ldr, OutT* C, long ldc, float* partial,
                                long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  if (M <= 16) return launch_skinny_lds<T, OutT, 1, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  if (M <= 32) return launch_skinny_lds<T, OutT, 2, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  if (M <= 48) return launch_skinny_lds<T, OutT, 3, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  return launch_skinny_lds<T, OutT, 4, SILU, PARTIAL, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 16) return launch_skinny_lds<T, OutT, 1, PARTIAL, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 32) return launch_skinny_lds<T, OutT, 2, PARTIAL, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if (M <= 48) return launch_skinny_lds<T, OutT, 3, PARTIAL, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  return launch_skinny_lds<T, OutT, 4, PARTIAL, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
 }
 
-template <typename T, typename OutT, bool SHUF>
+// force: 0 = choose, 1 = generic, 3 = tiled 128x128, 4 = tiled 128x256, 5 = skinny
+template <typename T, typename OutT, bool SHUF, bool GLU>
 static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const float* bias,
                            const float* residual, long ldr, OutT* C, long ldc, float* partial,
                            long partial_bytes, int M, int N, int K, int force, hipStream_t stream) {
   constexpr int EPF = Elem<T>::kPerFrag;
+  TW_REQUIRE(force == 0 || force == 1 || force == 3 || force == 4 || force == 5);
   // the shuffled layout exists only for K that is a multiple of 16 bytes and is always aligned
   const bool aligned = K % EPF == 0 && lda % EPF == 0 && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) &&
                        (SHUF || ldw % EPF == 0);
-  // force: 0 = choose, 1 = generic, 2 = skinny (per-wave, row-major weights only), 3 = tiled 128x128,
-  //        4 = tiled 128x256, 5 = skinny (workgroup-cooperative)
   if (force == 1 || !aligned) {
     TW_REQUIRE(force <= 1);
     TW_REQUIRE(!SHUF || K % EPF == 0);
-    gemm_generic_kernel<T, OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(A, lda, W, ldw, bias, residual,
-                                                                               ldr, C, ldc, M, N, K, SHUF ? 1 : 0);
+    const long outputs = (long)M * (GLU ? N / 2 : N);
+    gemm_generic_kernel<T, OutT><<<tw_div_up(outputs, 256), 256, 0, stream>>>(A, lda, W, ldw, bias, residual, ldr, C,
+                                                                            ldc, M, N, K, SHUF ? 1 : 0, GLU ? 1 : 0);
     return TW_LAUNCH_RESULT();
   }
   if (force == 5 || (force == 0 && M <= 64)) {
     TW_REQUIRE(M <= 64);
-    return launch_skinny_lds_m<T, OutT, false, false, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  }
-  if (force == 2) {
-    TW_REQUIRE(M <= 64 && !SHUF);
-    if (M <= 16) return launch_skinny<T, OutT, 1>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-    if (M <= 32) return launch_skinny<T, OutT, 2>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-    if (M <= 48) return launch_skinny<T, OutT, 3>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-    return launch_skinny<T, OutT, 4>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny_lds_m<T, OutT, false, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
   if (force == 4)
-    return launch_tiled<T, OutT, 2, 4, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
-  return launch_tiled<T, OutT, 2, 2, SHUF>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
 }
 
 template <typename T, typename OutT>
@@ -765,21 +657,25 @@ static int linear_layout(int shuffled, const T* A, long lda, const T* W, long ld
                          const float* residual, long ldr, OutT* C, long ldc, float* partial,
                          long partial_bytes, int M, int N, int K, int force, hipStream_t stream) {
   if (shuffled)
-    return linear_dispatch<T, OutT, true>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, force, stream);
-  return linear_dispatch<T, OutT, false>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, force, stream);
+    return linear_dispatch<T, OutT, true, false>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, force, stream);
+  return linear_dispatch<T, OutT, false, false>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, force, stream);
+}
+
+static bool weight_layout_ok(int dtype, int shuffled, long ldw, int K) {
+  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
+  return shuffled ? (K % epf == 0 && ldw >= (K / epf + 3) / 4) : ldw >= K;
 }
 
 // C = A W^T (+bias) (+residual). out_f32 != 0: C is float32 whatever the input type (residual
 // stream, logits); else C has the input type. `residual` may be C itself. `partial` is scratch
 // for split-K (tw_linear_workspace_bytes). shuffled != 0: W is in the shuffled layout and ldw
-// is its number of k-steps, ceil(K / (4 * elements per 16 bytes)).
+// is the number of k-steps between its row blocks, at least ceil(K / (4 * elements per 16 bytes)).
 extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const void* W, long ldw, int shuffled,
                          const float* bias, const float* residual, long ldr, void* C, long ldc,
                          float* partial, long partial_bytes, int M, int N, int K, int force,
                          hipStream_t stream) {
   TW_REQUIRE(M >= 0 && N > 0 && K > 0 && lda >= K && ldc >= N);
-  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
-  TW_REQUIRE(shuffled ? ldw >= (K / epf + 3) / 4 && K % epf == 0 : ldw >= K);
+  TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K));
   TW_REQUIRE(residual == nullptr || (ldr >= N && out_f32));
   if (M == 0) return 0;
   if (dtype == TW_DTYPE_F32)
@@ -795,7 +691,30 @@ extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const 
   return TW_ERR_BAD_ARGUMENT;
 }
 
-// ---- decode-path forms: few rows, 16-byte aligned K ------------------------------------
+template <typename T>
+static int glu_layout(int shuffled, const T* A, long lda, const T* W, long ldw, const float* bias, T* C, long ldc,
+                      int M, int N, int K, int force, hipStream_t stream) {
+  if (shuffled)
+    return linear_dispatch<T, T, true, true>(A, lda, W, ldw, bias, nullptr, 0, C, ldc, nullptr, 0, M, N, K, force, stream);
+  return linear_dispatch<T, T, false, true>(A, lda, W, ldw, bias, nullptr, 0, C, ldc, nullptr, 0, M, N, K, force, stream);
+}
+
+// Gated linear unit: W [N, K] holds gate and up rows interleaved in blocks of 16 (N a multiple
+// of 32); C [M, N / 2] = silu(gate) * up in the input type. bias (may be null) is indexed like W's rows.
+extern "C" int tw_linear_glu(int dtype, const void* A, long lda, const void* W, long ldw, int shuffled,
+                             const float* bias, void* C, long ldc, int M, int N, int K, int force,
+                             hipStream_t stream) {
+  TW_REQUIRE(M >= 0 && N > 0 && N % 32 == 0 && K > 0 && lda >= K && ldc >= N / 2);
+  TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K));
+  if (M == 0) return 0;
+  if (dtype == TW_DTYPE_F32)
+    return glu_layout<float>(shuffled, (const float*)A, lda, (const float*)W, ldw, bias, (float*)C, ldc, M, N, K, force, stream);
+  if (dtype == TW_DTYPE_BF16)
+    return glu_layout<bf16_t>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, force, stream);
+  return TW_ERR_BAD_ARGUMENT;
+}
+
+// ---- decode-path form: few rows, 16-byte aligned K ------------------------------------
 // Number of K ranges tw_linear_partials uses for an [N, K] weight (0: shape not supported).
 extern "C" int tw_linear_partial_splits(int dtype, int N, int K) {
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
@@ -803,31 +722,25 @@ extern "C" int tw_linear_partial_splits(int dtype, int N, int K) {
   return skinny_lds_splits(N, K, epf);
 }
 
-template <typename T, bool SILU>
+template <typename T>
 static int partials_layout(int shuffled, const T* A, long lda, const T* W, long ldw, float* partial,
                            long partial_bytes, int M, int N, int K, hipStream_t stream) {
   if (shuffled)
-    return launch_skinny_lds_m<T, float, SILU, true, true>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
-  return launch_skinny_lds_m<T, float, SILU, true, false>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+    return launch_skinny_lds_m<T, float, true, true, false>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
+  return launch_skinny_lds_m<T, float, true, false, false>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
 }
 
 // partial[split][M][N] (float32) = A[:, K range of split] W[:, same]^T for every split; the caller's
 // next kernel adds the splits up (with bias, residual, norm or rotation as it needs).
-// silu != 0: A is [M][2K] = [gate | up] and silu(gate) * up stands in for the activations.
-extern "C" int tw_linear_partials(int dtype, int silu, const void* A, long lda, const void* W, long ldw,
-                                  int shuffled, float* partial, long partial_bytes, int M, int N, int K,
-                                  hipStream_t stream) {
-  TW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && lda >= (silu ? 2L * K : (long)K));
+extern "C" int tw_linear_partials(int dtype, const void* A, long lda, const void* W, long ldw, int shuffled,
+                                  float* partial, long partial_bytes, int M, int N, int K, hipStream_t stream) {
+  TW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && lda >= K);
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
   TW_REQUIRE(K % epf == 0 && lda % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
-  TW_REQUIRE(shuffled ? ldw >= (K / epf + 3) / 4 : (ldw >= K && ldw % epf == 0));
-  if (dtype == TW_DTYPE_F32) {
-    if (silu) return partials_layout<float, true>(shuffled, (const float*)A, lda, (const float*)W, ldw, partial, partial_bytes, M, N, K, stream);
-    return partials_layout<float, false>(shuffled, (const float*)A, lda, (const float*)W, ldw, partial, partial_bytes, M, N, K, stream);
-  }
-  if (dtype == TW_DTYPE_BF16) {
-    if (silu) return partials_layout<bf16_t, true>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, partial, partial_bytes, M, N, K, stream);
-    return partials_layout<bf16_t, false>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, partial, partial_bytes, M, N, K, stream);
-  }
+  TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K) && (shuffled || ldw % epf == 0));
+  if (dtype == TW_DTYPE_F32)
+    return partials_layout<float>(shuffled, (const float*)A, lda, (const float*)W, ldw, partial, partial_bytes, M, N, K, stream);
+  if (dtype == TW_DTYPE_BF16)
+    return partials_layout<bf16_t>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, partial, partial_bytes, M, N, K, stream);
   return TW_ERR_BAD_ARGUMENT;
 }

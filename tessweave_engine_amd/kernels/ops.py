@@ -211,26 +211,53 @@ def linear_partial_splits(dtype, n, k):
     return int(library().tw_linear_partial_splits(dtype_id(dtype), int(n), int(k)))
 
 
-def linear_partials(x, weight, partial, silu_gate=False):
+def linear_partials(x, weight, partial):
     """partial[s] = x[:, K range s] @ weight[:, K range s].T in float32, for at most 64 rows.
 
-    The caller's next kernel adds the splits up. silu_gate: x is [m, 2k] = [gate | up] and
-    silu(gate) * up (rounded to x's type) stands in for the activations.
+    The caller's next kernel adds the splits up.
     """
     m, kx, lda = _rows(x, "x")
     n, k, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
-    _need(kx == (2 * k if silu_gate else k), "linear_partials shapes do not agree")
+    _need(kx == k, "linear_partials shapes do not agree")
     _need(x.dtype == w_dtype and 1 <= m <= 64, "linear_partials takes 1..64 rows of the weight's type")
     splits = linear_partial_splits(w_dtype, n, k)
     _need(splits > 0, "linear_partials needs K to be a multiple of 16 bytes")
     _need(partial.is_contiguous() and tuple(partial.shape) == (splits, m, n), f"partial must be [{splits}, {m}, {n}]")
-    check(library().tw_linear_partials(dtype_id(x.dtype), 1 if silu_gate else 0, _dev(x), lda, w_ptr, ldw, shuffled,
+    check(library().tw_linear_partials(dtype_id(x.dtype), _dev(x), lda, w_ptr, ldw, shuffled,
                                        _dev(partial, torch.float32, "partial"), partial.numel() * 4, m, n, k,
                                        _stream()), "linear_partials")
     return partial
 
 
-GEMM_AUTO, GEMM_GENERIC, GEMM_SKINNY, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY_COOP = 0, 1, 2, 3, 4, 5
+def interleave_glu_rows(gate, up):
+    """[2n, k] with the rows of gate and up [n, k] alternating in blocks of 16 (n a multiple of 16).
+
+    The same order applies to biases ([n] each). This is the row order `linear_glu` expects.
+    """
+    _need(gate.shape == up.shape and gate.shape[0] % 16 == 0, "gate and up must have equally many rows, a multiple of 16")
+    n = gate.shape[0]
+    rest = tuple(gate.shape[1:])
+    return torch.stack([gate.reshape(n // 16, 16, *rest), up.reshape(n // 16, 16, *rest)], 1).reshape(2 * n, *rest).contiguous()
+
+
+def linear_glu(x, weight, out, bias=None, force=0):
+    """out[m, n/2] = silu(x @ gate.T) * (x @ up.T), weight [n, k] holding gate and up rows
+    interleaved by `interleave_glu_rows` (row-major or shuffled); out has x's type."""
+    m, k, lda = _rows(x, "x")
+    n, k2, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
+    mo, no, ldc = _rows(out, "out")
+    _need(n % 32 == 0, "a gated weight has a multiple of 32 rows")
+    _need(k == k2 and mo == m and no == n // 2, f"linear_glu shapes do not agree: x {tuple(x.shape)}, weight {(n, k2)}, out {tuple(out.shape)}")
+    _need(x.dtype == w_dtype and out.dtype == x.dtype, "x, weight and out types differ")
+    if bias is not None:
+        _need(bias.numel() == n, "bias has the wrong size")
+    check(library().tw_linear_glu(dtype_id(x.dtype), _dev(x), lda, w_ptr, ldw, shuffled,
+                                  _dev(bias, torch.float32, "bias") if bias is not None else None,
+                                  _dev(out), ldc, m, n, k, force, _stream()), "linear_glu")
+    return out
+
+
+GEMM_AUTO, GEMM_GENERIC, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY = 0, 1, 3, 4, 5
 
 
 def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_AUTO):

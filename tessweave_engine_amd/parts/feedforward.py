@@ -10,7 +10,7 @@ class SwiGLU(FeedForward):
     def __init__(self, prefix, hidden, intermediate, packed=True):
         self.hidden, self.intermediate = int(hidden), int(intermediate)
         self.gate_up = Linear([prefix + "gate_proj", prefix + "up_proj"], hidden, [intermediate, intermediate],
-                              packed=packed)
+                              packed=packed, glu=True)
         self.down = Linear([prefix + "down_proj"], intermediate, [hidden])
 
     def parts(self):
@@ -25,15 +25,16 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx, h, x):
         n = h.shape[0]
-        gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
-        self.gate_up.forward(ctx, h, gu)
-        if self.down.deferrable(n):
-            # few rows: silu(gate) * up is formed while the down projection stages its input,
-            # and its split-K sums are left to the next norm
-            return self.down.forward_partials(ctx, gu, "down", silu_gate=True)
-        # many rows: a separate SiLU-multiply pass (fused into the tiled kernel's tile loads it would
-        # be recomputed once per column tile, which costs more than the pass)
         act = ctx.scratch("ffn.act", (n, self.intermediate))
-        ops.silu_mul(gu, act)
+        if self.gate_up.gated:
+            # silu(gate) * up is formed in the projection's epilogue; [n, 2 * intermediate] is never stored
+            self.gate_up.forward_glu(ctx, h, act)
+        else:
+            gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
+            self.gate_up.forward(ctx, h, gu)
+            ops.silu_mul(gu, act)
+        if self.down.deferrable(n):
+            # few rows: the down projection's split-K sums are left to the next norm
+            return self.down.forward_partials(ctx, act, "down")
         self.down.forward(ctx, act, x, residual=x)
         return None

@@ -15,13 +15,19 @@ from .base import Part
 
 
 class Linear(Part):
-    def __init__(self, names, in_features, out_features, bias=False, packed=True):
-        """names[i] is the checkpoint prefix of the i-th matrix ("...q_proj"), out_features[i] its rows."""
+    def __init__(self, names, in_features, out_features, bias=False, packed=True, glu=False):
+        """names[i] is the checkpoint prefix of the i-th matrix ("...q_proj"), out_features[i] its rows.
+
+        glu: the two matrices are a gate and an up projection; if they can be packed with their
+        rows interleaved (`gated` is then true after bind), `forward_glu` gives silu(gate) * up.
+        """
         self.names = list(names)
         self.in_features = int(in_features)
         self.out_features = [int(o) for o in out_features]
         self.has_bias = bool(bias)
         self.packed = bool(packed)
+        self.glu = bool(glu)
+        self.gated = False
         self.weights = []       # one tensor if packed, else one per name
         self.biases = []
         self._ws_floats = {}
@@ -41,7 +47,12 @@ class Linear(Part):
     def bind(self, tensors, dtype, device):
         weights = [tensors.pop(name + ".weight") for name in self.names]
         biases = [tensors.pop(name + ".bias") for name in self.names] if self.has_bias else []
-        if self.packed and len(weights) > 1:
+        self.gated = (self.glu and self.packed and len(weights) == 2 and
+                      self.out_features[0] == self.out_features[1] and self.out_features[0] % 16 == 0)
+        if self.gated:
+            weights = [ops.interleave_glu_rows(*weights)]
+            biases = [ops.interleave_glu_rows(*biases)] if biases else []
+        elif self.packed and len(weights) > 1:
             weights = [torch.cat(weights, 0)]
             biases = [torch.cat(biases, 0)] if biases else []
         # On a GPU the matrices are kept in the kernels' shuffled layout (an exact permutation)
@@ -56,12 +67,18 @@ class Linear(Part):
         return sum(w.numel() * w.element_size() for w in self.weights)
 
     def row_major(self, i=0):
-        """Weight i as a row-major [out, in] tensor (a copy if it is held shuffled)."""
+        """Weight i as a row-major [out, in] tensor (a copy if it is held shuffled; a gated pair keeps its interleaved rows)."""
         w = self.weights[i]
         return w.to_rows() if isinstance(w, ops.ShuffledWeight) else w
 
+    def forward_glu(self, ctx, x, out):
+        """out [n, rows of one matrix] = silu(x @ gate.T + b) * (x @ up.T + b), in x's type (needs `gated`)."""
+        return ops.linear_glu(x, self.weights[0], out, bias=self.biases[0] if self.biases else None)
+
     def forward(self, ctx, x, out, residual=None):
         """out[:, columns] = x @ W.T (+ bias) (+ residual); out may be float32 or x's type."""
+        if self.gated:
+            raise RuntimeError("a gated pair of matrices has interleaved rows; use forward_glu")
         col = 0
         for i, w in enumerate(self.weights):
             rows = w.shape[0]
@@ -90,10 +107,10 @@ class Linear(Part):
             self._ws_floats["splits"] = ops.linear_partial_splits(w.dtype, w.shape[0], w.shape[1])
         return self._ws_floats["splits"] > 0
 
-    def forward_partials(self, ctx, x, tag, silu_gate=False):
+    def forward_partials(self, ctx, x, tag):
         """float32 [splits, n, out] partial sums of x @ W.T (bias NOT added); see ops.linear_partials."""
         w = self.weights[0]
         splits = self._ws_floats["splits"]
         buf = ctx.workspace.get("linear.partial." + tag, (splits, 64, w.shape[0]), torch.float32)
         partial = buf.view(-1)[:splits * x.shape[0] * w.shape[0]].view(splits, x.shape[0], w.shape[0])
-        return ops.linear_partials(x, w, partial, silu_gate=silu_gate)
+        return ops.linear_partials(x, w, partial)

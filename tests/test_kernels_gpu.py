@@ -155,13 +155,13 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
     ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=device)
     forces = [ops.GEMM_AUTO, ops.GEMM_GENERIC, ops.GEMM_TILED, ops.GEMM_TILED_WIDE]
     if m <= 64:
-        forces += [ops.GEMM_SKINNY, ops.GEMM_SKINNY_COOP]
+        forces += [ops.GEMM_SKINNY]
     scale = math.sqrt(k) * 0.05
     t = dict(atol=2e-5 * scale, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2 * scale, rtol=2e-2)
     shuffled = ops.shuffle_weight(w)
     torch.testing.assert_close(shuffled.to_rows(), w, atol=0, rtol=0)          # an exact permutation
     for force in forces + [("shuffled", f) for f in (ops.GEMM_AUTO, ops.GEMM_GENERIC, ops.GEMM_TILED, ops.GEMM_TILED_WIDE)
-                           + ((ops.GEMM_SKINNY_COOP,) if m <= 64 else ())]:
+                           + ((ops.GEMM_SKINNY,) if m <= 64 else ())]:
         wt = w
         if isinstance(force, tuple):
             wt, force = shuffled, force[1]
@@ -185,7 +185,7 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 389, 2048), (17, 130, 4096), (64, 96, 9472)])
-def test_linear_partials_and_fused_silu(ops, device, dtype, m, n, k):
+def test_linear_partials(ops, device, dtype, m, n, k):
     x = rand((m, k), dtype, device, 1.0, seed=1)
     w = rand((n, k), dtype, device, 0.05, seed=2)
     splits = ops.linear_partial_splits(dtype, n, k)
@@ -199,14 +199,36 @@ def test_linear_partials_and_fused_silu(ops, device, dtype, m, n, k):
     part.fill_(float("nan"))
     ops.linear_partials(x, w, part)
     torch.testing.assert_close(part.sum(0), rows_sum, atol=0, rtol=0)
-    # [gate | up] input: silu(gate) * up, rounded to the input type, is what gets multiplied
-    gu = rand((m, 2 * k), dtype, device, 1.0, seed=3)
-    act = torch.empty(m, k, dtype=dtype, device=device)
-    ops.silu_mul(gu, act)
-    ops.linear_partials(act, w, part)
-    plain_sum = part.sum(0).clone()
-    ops.linear_partials(gu, w, part, silu_gate=True)
-    torch.testing.assert_close(part.sum(0), plain_sum, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,inter,k", [(1, 16, 64), (8, 208, 320), (17, 48, 1032), (64, 1040, 256), (65, 80, 64),
+                                       (200, 400, 320), (130, 16, 101)])
+def test_linear_glu(ops, device, dtype, m, inter, k):
+    """silu(x gate^T + b) * (x up^T + b) from interleaved rows, every kernel and both layouts."""
+    x = rand((m, k), dtype, device, 1.0, seed=1)
+    gate, up = rand((inter, k), dtype, device, 0.08, seed=2), rand((inter, k), dtype, device, 0.08, seed=3)
+    bg, bu = rand((inter,), torch.float32, device, 0.5, seed=4), rand((inter,), torch.float32, device, 0.5, seed=5)
+    w = ops.interleave_glu_rows(gate, up)
+    bias = ops.interleave_glu_rows(bg, bu)
+    assert torch.equal(w[:16], gate[:16]) and torch.equal(w[16:32], up[:16])
+    xd = x.double().cpu()
+    scale = math.sqrt(k) * 0.08
+    t = dict(atol=3e-5 * scale, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2 * scale, rtol=2e-2)
+    aligned = k % (16 // x.element_size()) == 0
+    forces = [ops.GEMM_AUTO, ops.GEMM_GENERIC] + ([ops.GEMM_TILED, ops.GEMM_TILED_WIDE] if aligned else [])
+    if m <= 64 and aligned:
+        forces.append(ops.GEMM_SKINNY)
+    layouts = [w] + ([ops.shuffle_weight(w)] if aligned else [])
+    for b in (None, bias):
+        g = xd @ gate.double().cpu().T + (bg.double().cpu() if b is not None else 0)
+        u = xd @ up.double().cpu().T + (bu.double().cpu() if b is not None else 0)
+        want = torch.nn.functional.silu(g) * u
+        for weight in layouts:
+            for force in forces:
+                out = torch.full((m, inter), float("nan"), dtype=dtype, device=device)
+                ops.linear_glu(x, weight, out, bias=b, force=force)
+                torch.testing.assert_close(out.double().cpu(), want, **t)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

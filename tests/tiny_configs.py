@@ -10,7 +10,7 @@ TINY_A_PAGE, TINY_A_SEED = 16, 0
 TINY_B = dict(
     architectures=["Qwen2ForCausalLM"], model_type="qwen2",
     num_hidden_layers=3, hidden_size=192, num_attention_heads=6, num_key_value_heads=1, head_dim=32,
-    intermediate_size=320, vocab_size=389, rope_theta=1e6, rms_norm_eps=1e-5,
+    intermediate_size=328, vocab_size=389, rope_theta=1e6, rms_norm_eps=1e-5,
     tie_word_embeddings=False, use_sliding_window=False, max_position_embeddings=1024, hidden_act="silu")
 TINY_B_PAGE, TINY_B_SEED = 8, 1
 
