@@ -387,6 +387,50 @@ def test_attn_far_key_among_hundreds(ops, device):
         torch.testing.assert_close(out.cpu().reshape(1, heads, d), want, atol=3e-5, rtol=3e-5)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page,window", [(16, 0), (8, 0), (64, 0), (16, 70), (4, 33)])
+def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
+    """Each head's query points at ONE key that sits on an edge (of a page, of a 32-key block, of a split,
+    of the window, of the sequence): a kernel that drops, doubles or misplaces that key is wrong by O(1),
+    also in bfloat16, where random keys would hide it in the tolerance."""
+    d, n, q_len = 64, 300, 48
+    targets = [0, 1, 7, 8, 15, 16, 17, 31, 32, 33, 63, 64, 127, 128, 159, 160, 255, 256, n - q_len - 1, n - q_len,
+               n - 2, n - 1]
+    if window:
+        targets += [n - window - 1, n - window, n - window + 1, n - q_len - window, n - q_len - window + 1]
+    heads = len(targets)
+    gen = torch.Generator().manual_seed(77)
+    unit = torch.nn.functional.normalize(torch.randn(heads, d, generator=gen), dim=1)
+    k = (torch.randn(n, 1, d, generator=gen) * 0.1)
+    v = torch.randn(n, 1, d, generator=gen)
+    for h, p in enumerate(targets):
+        k[p, 0] = unit[h] * 30.0
+    k, v = k.to(dtype).float(), v.to(dtype).float()
+    q_one = (unit * 8.0).to(dtype)                                     # score of the target: 30, of the rest: ~0
+    keys, values, table = build_paged([k], [v], [n], page, 320 // page + 8, device, dtype, seed=21)
+    kv_len = torch.tensor([n], dtype=torch.int32, device=device)
+    # decode: the last position asks
+    want = plain.attention(q_one[None].float(), k, v, torch.tensor([n - 1]), window=window or None)
+    seen = [h for h, p in enumerate(targets) if not window or p > n - 1 - window]
+    assert all((want[0, h] - v[targets[h], 0]).abs().max() < 2e-2 for h in seen)    # the vectors do what they are for
+    q_start = torch.tensor([0, 1], dtype=torch.int32, device=device)
+    for splits, generic in ((1, False), (2, False), (3, False), (7, False), (1, True), (4, True)):
+        out = torch.full((1, heads * d), float("nan"), dtype=dtype, device=device)
+        ws = torch.empty(max(1, ops.attn_decode_workspace_floats(1, heads, d, splits)), device=device)
+        ops.attn_decode(q_one.reshape(1, -1).to(device), keys, values, table, q_start, kv_len, 0, 1, out, heads, 1, d,
+                        d ** -0.5, window=window, splits=splits, workspace=ws, generic=generic)
+        torch.testing.assert_close(out.float().cpu().reshape(1, heads, d), want, **ATTN_TOL[dtype])
+    # prefill: the last q_len positions ask the same questions; early rows do not see late keys
+    q = q_one[None].expand(q_len, heads, d).contiguous()
+    want = plain.attention(q.float(), k, v, torch.arange(n - q_len, n), window=window or None)
+    q_start = torch.tensor([0, q_len], dtype=torch.int32, device=device)
+    for generic in (False, True):
+        out = torch.full((q_len, heads * d), float("nan"), dtype=dtype, device=device)
+        ops.attn_prefill(q.reshape(q_len, -1).to(device), keys, values, table, q_start, kv_len, 0, 1, q_len, out, heads, 1,
+                         d, d ** -0.5, window=window, generic=generic)
+        torch.testing.assert_close(out.float().cpu().reshape(q_len, heads, d), want, **ATTN_TOL[dtype])
+
+
 # ---------------------------------------------------------------------------------------
 def test_sampling_greedy_ties_and_distribution(ops, device):
     vocab = 389
