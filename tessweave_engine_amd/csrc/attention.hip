@@ -258,7 +258,12 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 // (8a + 4 + j), so lane group g ends up with the probabilities of the 8
 // CONSECUTIVE keys 8g .. 8g+7: they are the B operand of one 16x16x32 MFMA per
 // 16 output dims, whose A operand is a single 16-byte load of values[d][8g..8g+7].
-// The keys and values of the next block are loaded while this one is computed.
+//
+// A wave keeps two blocks in registers: the loads of the next block are in flight while
+// this one is computed. Loads carry no predicate: a key outside the sequence or the window
+// is read from a page the block does hold (its score is then selected to -inf and its value
+// to zero), and only the first and last block of a range pay for those selects.
+// EXACT: head_dim == 16 * DTMAX (no per-chunk checks at all).
 // =====================================================================================
 template <int DTMAX>
 struct KVBlock {
@@ -267,7 +272,9 @@ struct KVBlock {
   bf16x8 v[DTMAX];
 };
 
-template <int DTMAX>
+template <bool V> struct BoolTag { static constexpr bool value = V; };
+
+template <int DTMAX, bool EXACT>
 __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
   constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
   __shared__ float lds_o[3][16][DTMAX * 16];
@@ -283,7 +290,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
   const int token = a.q_start[seq];
   const int t = kv_len - 1;
   const int* table = a.block_table + (size_t)seq * a.table_stride;
-  const int D = a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
+  const int D = EXACT ? DTMAX * 16 : a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
   const bf16_t* keys = (const bf16_t*)a.keys;
   const bf16_t* values = (const bf16_t*)a.values;
 
@@ -296,7 +303,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
 #pragma unroll
     for (int st = 0; st < NSMAX; ++st) {
       const int chunk = st * 4 + g;
-      qf[st] = (row_ok && chunk < chunks) ? tw_load_frag(q_row + chunk * 8) : Elem<bf16_t>::zero();
+      qf[st] = (row_ok && (EXACT || chunk < chunks)) ? tw_load_frag(q_row + chunk * 8) : Elem<bf16_t>::zero();
     }
   }
   f32x4 acc[DTMAX];
@@ -310,68 +317,80 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
   const int begin = blk_lo + split * per_split;
   const int end = min(blk_hi, begin + per_split);
 
-  // Page ids of a 32-key block are the same for every lane: they are read with
-  // scalar loads (blk is made wave-uniform), off the vector-memory queue.
+  // Per-lane constants of the loads. A 32-key block spans 1, 2 or 4 pages (pages of 8 keys
+  // or more, powers of two); p0 is a multiple of 32, so for pages smaller than a block the
+  // in-page index of a key does not depend on the block.
   const int pshift = a.page_shift, pmask = P - 1;
-  const int ppb = P >= 32 ? 1 : (32 >> pshift);                    // pages per block: 1, 2 or 4
-  const unsigned head_stride = (unsigned)P * D;                      // elements of one (page, kv head)
+  const int ppb = P >= 32 ? 1 : (32 >> pshift);                    // pages per block
+  const size_t head_stride = (size_t)P * D;                          // elements of one (page, kv head)
+  int k_pi[2];
+  unsigned k_off[2];
+#pragma unroll
+  for (int tile = 0; tile < 2; ++tile) {
+    const int ko = 8 * (r >> 2) + 4 * tile + (r & 3);                // the key this lane's row stands for
+    k_pi[tile] = P >= 32 ? 0 : (ko >> pshift);
+    k_off[tile] = (unsigned)(P >= 32 ? ko : (ko & pmask)) * D + g * 8;
+  }
+  const int kv0 = 8 * g;                                              // this lane's 8 consecutive keys
+  const int v_pi = P >= 32 ? 0 : (kv0 >> pshift);
+  const unsigned v_off = (unsigned)r * P + (P >= 32 ? kv0 : (kv0 & pmask));
+
+  // Page ids of a block are the same for every lane: scalar loads (blk is wave-uniform).
+  // A page that holds no key of [lo, kv_len) may not be held at all: it is replaced by one
+  // of the block that is, so that every load has an address inside the pool.
   auto issue = [&](int blk_v, KVBlock<DTMAX>& L) {
     const int blk = __builtin_amdgcn_readfirstlane(blk_v);
     const int p0 = blk * 32;
     const int first = p0 >> pshift;
     int pg[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pg[i] = (i < ppb && p0 + (i << pshift) < kv_len) ? table[first + i] : -1;
-    auto page_of = [&](int ko) {                                     // ko: key offset inside the block
-      const int i = P >= 32 ? 0 : (ko >> pshift);
-      return i == 0 ? pg[0] : (i == 1 ? pg[1] : (i == 2 ? pg[2] : pg[3]));
-    };
+    for (int i = 0; i < 4; ++i) {
+      const int a0 = P >= 32 ? p0 : p0 + (i << pshift);              // first key of the block in page i
+      const int a1 = P >= 32 ? p0 + 31 : a0 + P - 1;                 // last one
+      pg[i] = (i < ppb && a0 < kv_len && a1 >= lo) ? table[first + i] : -1;
+    }
+    int safe = pg[0] >= 0 ? pg[0] : (pg[1] >= 0 ? pg[1] : (pg[2] >= 0 ? pg[2] : pg[3]));
+    if (safe < 0) safe = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (pg[i] < 0) pg[i] = safe;
+    auto page_of = [&](int i) { return i == 0 ? pg[0] : (i == 1 ? pg[1] : (i == 2 ? pg[2] : pg[3])); };
+    const unsigned pb = P >= 32 ? (unsigned)(p0 & pmask) : 0u;      // the block's first key inside its page
 #pragma unroll
     for (int tile = 0; tile < 2; ++tile) {
-      const int ko = 8 * (r >> 2) + 4 * tile + (r & 3);              // the key this lane's row stands for
-      const int p = p0 + ko;
-      int page = page_of(ko);
-      if (p >= kv_len || p < lo) page = -1;
-      const size_t base = ((size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh) * head_stride;
-      const bf16_t* k_row = keys + base + (unsigned)(p & pmask) * D + g * 8;
+      const bf16_t* k_row = keys + ((size_t)page_of(k_pi[tile]) * a.kv_heads + kvh) * head_stride + pb * D + k_off[tile];
 #pragma unroll
       for (int st = 0; st < NSMAX; ++st)
-        L.k[tile][st] = (page >= 0 && st * 4 + g < chunks) ? tw_load_frag(k_row + st * 32) : Elem<bf16_t>::zero();
+        L.k[tile][st] = (EXACT || st * 4 + g < chunks) ? tw_load_frag(k_row + st * 32) : Elem<bf16_t>::zero();
     }
-    const int kv0 = 8 * g;                                            // this lane's 8 consecutive keys
-    int vpage = page_of(kv0);
-    if (p0 + kv0 >= kv_len || p0 + kv0 + 7 < lo) vpage = -1;
-    const size_t vbase = ((size_t)(vpage < 0 ? 0 : vpage) * a.kv_heads + kvh) * head_stride;
-    const bf16_t* v_base = values + vbase + ((p0 + kv0) & pmask) + (unsigned)r * P;
+    const bf16_t* v_base = values + ((size_t)page_of(v_pi) * a.kv_heads + kvh) * head_stride + pb + v_off;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts)
-        L.v[dt] = vpage >= 0 ? tw_load_frag(v_base + (unsigned)(dt * 16) * P) : Elem<bf16_t>::zero();
+      if (EXACT || dt < dts) L.v[dt] = tw_load_frag(v_base + (size_t)(dt * 16) * P);
   };
 
-  auto compute = [&](int blk, KVBlock<DTMAX>& L) {
+  auto compute_as = [&](int blk, KVBlock<DTMAX>& L, auto edge_tag) {
+    constexpr bool EDGE = decltype(edge_tag)::value;
     const int p0 = blk * 32;
     f32x4 s[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
     for (int tile = 0; tile < 2; ++tile)
 #pragma unroll
       for (int st = 0; st < NSMAX; ++st)
-        if (st * 4 < chunks) tw_mma16(s[tile], L.k[tile][st], qf[st]);
-    // this lane: row r (a head), keys p0 + 8g + e, e = 4*tile + j
+        if (EXACT || st * 4 < chunks) tw_mma16(s[tile], L.k[tile][st], qf[st]);
+    // this lane: row r (a head), keys p0 + 8g + e, e = 4*tile + j; every cached key is at or before t
     float pr[8];
     float mx = -INFINITY;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int p = p0 + 8 * g + e;
-      const bool ok = row_ok && p < kv_len && p >= lo;                  // decode: every cached key is at or before t
-      pr[e] = ok ? s[e >> 2][e & 3] * a.scale : -INFINITY;
+      pr[e] = (!EDGE || (p < kv_len && p >= lo)) ? s[e >> 2][e & 3] * a.scale : -INFINITY;
       mx = fmaxf(mx, pr[e]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
     const float m_new = fmaxf(m, mx);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = __expf(m - m_use);
     float sum = 0.f;
     bf16x8 pb;
 #pragma unroll
@@ -382,32 +401,55 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
     }
     sum += __shfl_xor(sum, 16, TW_WAVE);
     sum += __shfl_xor(sum, 32, TW_WAVE);
-    l = l * alpha + sum;
-    m = m_new;
-    const bool edge = p0 + 32 > kv_len || p0 < lo;                      // only edge blocks hold keys to blank out
+    // the running maximum of a row rarely moves after the first blocks: rescale only then
+    if (__any(m_new > m)) {
+      const float alpha = __expf(m - m_use);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DTMAX; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[dt][j] *= alpha;
+      m = m_new;
+    }
+    l += sum;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts) {
+      if (EXACT || dt < dts) {
         bf16x8 vq = L.v[dt];
-        if (edge) {
+        if (EDGE) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const int p = p0 + 8 * g + e;
             if (p >= kv_len || p < lo) vq[e] = (bf16_t)0.f;
           }
         }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[dt][j] *= alpha;
         tw_mma16(acc[dt], vq, pb);
       }
   };
+  auto compute = [&](int blk, KVBlock<DTMAX>& L) {
+    if (blk * 32 + 32 > kv_len || blk * 32 < lo) compute_as(blk, L, BoolTag<true>());
+    else compute_as(blk, L, BoolTag<false>());
+  };
 
   {
-    // One block in registers per wave; several waves per SIMD hide each other's memory latency.
-    KVBlock<DTMAX> A;
-    for (int blk = begin + wave; blk < end; blk += 4) {
+    KVBlock<DTMAX> A, B;
+    int blk = begin + wave;                                     // this wave's blocks: blk, blk + 4, ...
+    if (blk < end) {
       issue(blk, A);
-      compute(blk, A);
+      while (blk + 8 < end) {                                   // blocks blk + 4 and blk + 8 exist
+        issue(blk + 4, B);
+        compute(blk, A);
+        issue(blk + 8, A);
+        compute(blk + 4, B);
+        blk += 8;
+      }
+      if (blk + 4 < end) {
+        issue(blk + 4, B);
+        compute(blk, A);
+        compute(blk + 4, B);
+      } else {
+        compute(blk, A);
+      }
     }
   }
 
@@ -415,7 +457,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
   if (wave > 0) {
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts)
+      if (EXACT || dt < dts)
 #pragma unroll
         for (int j = 0; j < 4; ++j) lds_o[wave - 1][r][dt * 16 + 4 * g + j] = acc[dt][j];
     if (g == 0) {
@@ -441,7 +483,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
     l += lds_ml[w][r][1] * f;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts)
+      if (EXACT || dt < dts)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[dt][j] += lds_o[w][r][dt * 16 + 4 * g + j] * f;
   }
@@ -451,7 +493,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
     bf16_t* dst = (bf16_t*)a.out + (size_t)token * a.ldo + (size_t)head * D;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts)
+      if (EXACT || dt < dts)
 #pragma unroll
         for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = (bf16_t)(acc[dt][j] * inv);
   } else {
@@ -459,7 +501,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
     float* dst = a.part_o + slot * D;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts)
+      if (EXACT || dt < dts)
 #pragma unroll
         for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = acc[dt][j];
     if (g == 0) {
@@ -566,7 +608,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 // =====================================================================================
 #define TW_PF_VROW 80                       /* LDS bytes per value row (32 keys = 64 B, padded) */
 
-template <bool V> struct BoolTag { static constexpr bool value = V; };
 
 template <int DTMAX>
 __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
@@ -876,7 +917,8 @@ static int check_common(const AttnArgs& a) {
 extern "C" int tw_attn_decode_splits(int n_seqs, int q_heads, int kv_heads, int max_kv_len) {
   const int G = q_heads / kv_heads;
   const int units = n_seqs * kv_heads * ((G + 15) / 16);
-  int splits = tw_div_up(1024, units > 0 ? units : 1);
+  // one workgroup per CU is enough: a wave keeps two 16 KB blocks in flight
+  int splits = tw_div_up(256, units > 0 ? units : 1);
   const int by_len = tw_div_up(max_kv_len, 256);
   if (splits > by_len) splits = by_len;
   if (splits > 64) splits = 64;
@@ -895,12 +937,16 @@ static int decode_launch(AttnArgs a, int n_seqs, int generic, hipStream_t stream
   const int G = a.q_heads / a.kv_heads;
   dim3 grid(a.splits, a.kv_heads * ((G + 15) / 16), n_seqs);
   if (IsBf16<T>::value && a.page_shift >= 3 && !generic) {
-    if (a.head_dim <= 64)
-      attn_decode_bf16_kernel<4><<<grid, 256, 0, stream>>>(a);
-    else if (a.head_dim <= 128)
-      attn_decode_bf16_kernel<8><<<grid, 256, 0, stream>>>(a);
+    if (a.head_dim == 64)
+      attn_decode_bf16_kernel<4, true><<<grid, 256, 0, stream>>>(a);
+    else if (a.head_dim < 64)
+      attn_decode_bf16_kernel<4, false><<<grid, 256, 0, stream>>>(a);
+    else if (a.head_dim == 128)
+      attn_decode_bf16_kernel<8, true><<<grid, 256, 0, stream>>>(a);
+    else if (a.head_dim < 128)
+      attn_decode_bf16_kernel<8, false><<<grid, 256, 0, stream>>>(a);
     else
-      attn_decode_bf16_kernel<16><<<grid, 256, 0, stream>>>(a);
+      attn_decode_bf16_kernel<16, false><<<grid, 256, 0, stream>>>(a);
   } else if (a.head_dim <= 64)
     attn_decode_kernel<T, 4><<<grid, 256, 0, stream>>>(a);
   else if (a.head_dim <= 128)
