@@ -73,10 +73,12 @@ def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, s
             engine.stepper.step([StepEntry(r.seq, r.prompt[i:min(prompt_len - 1, i + chunk)], [])])
     for _ in range(warmup):
         engine.step()
+    engine.flush()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         engine.step()
+    engine.flush()                 # the last step's tokens are read inside the timed region too
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     assert all(len(r.output) == warmup + steps for r in requests), [len(r.output) for r in requests]

@@ -189,7 +189,8 @@ class CacheManager:
         for g, pool in enumerate(self.pools):
             table = seq.tables[g]
             blocks = math.ceil(n_tokens / self.page_size)
-            first = self.first_needed_block(g, seq.computed)
+            # positions below seq.computed are held already (or a window has passed them)
+            first = max(self.first_needed_block(g, seq.computed), seq.computed // self.page_size)
             missing = [b for b in range(first, blocks) if b >= len(table) or table[b] < 0]
             plans.append((g, blocks, missing))
         taken = []

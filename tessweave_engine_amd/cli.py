@@ -41,6 +41,7 @@ def _engine_options(p):
     p.add_argument("--max-step-tokens", type=int, default=0, help="token budget of one step (0: max-active + prefill-chunk)")
     p.add_argument("--adaptive-chunk", action="store_true", help="size prompt portions by measured step time")
     p.add_argument("--no-graphs", action="store_true", help="never replay decode steps from HIP graphs")
+    p.add_argument("--no-lookahead", action="store_true", help="read every turn's tokens before the next turn is put on the device")
 
 
 def build_parser():
@@ -105,7 +106,7 @@ def make_engine(args):
         max_active=args.max_active, prefill_chunk=args.prefill_chunk,
         min_prefill_chunk=min(16, args.prefill_chunk), target_step_ms=args.target_step_ms,
         prefix_cache=not args.no_prefix_cache, dtype=dtype, max_step_tokens=args.max_step_tokens,
-        adaptive_chunk=args.adaptive_chunk, use_graphs=not args.no_graphs)
+        adaptive_chunk=args.adaptive_chunk, use_graphs=not args.no_graphs, lookahead=not args.no_lookahead)
     tokenizer = None
     if getattr(args, "prompt", None):
         from transformers import AutoTokenizer          # tokenizer files only; no model code of the library runs

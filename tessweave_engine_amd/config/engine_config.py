@@ -4,7 +4,7 @@ Names, defaults and meanings follow flow_engine/config.py:68-92 where the
 reference has them. Left out: `attention` (one backend here) and `draft_*`
 (speculation is not built). Added: `dtype`, `max_step_tokens` (token budget of
 one step), `adaptive_chunk` (the reference's wall-clock feedback on the prompt
-portion, off by default so runs are reproducible) and `use_graphs`.
+portion, off by default so runs are reproducible), `use_graphs` and `lookahead`.
 """
 from __future__ import annotations
 
@@ -26,6 +26,7 @@ class EngineConfig:
     max_step_tokens: int = 0        # 0: max_active + prefill_chunk
     adaptive_chunk: bool = False    # flow_engine/engine.py:262-268 feedback controller
     use_graphs: bool = True         # replay decode-only steps from HIP graphs
+    lookahead: bool = True          # put a turn on the device before the tokens of the turn before are read
 
     def __post_init__(self):
         for key in ("block_size", "kv_blocks", "max_context", "max_active", "max_queue",

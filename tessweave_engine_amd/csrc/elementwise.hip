@@ -4,11 +4,15 @@
 #include "tw_common.h"
 
 // ---- embedding: x[n, :] = float(E[ids[n], :]) ------------------------------------
+// A negative id -1 - k stands for feed[k]: a token that an earlier kernel on this stream wrote
+// (the sampler's output of the step before), which the host has not read yet.
 template <typename T>
 __global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                    float* __restrict__ out, int hidden, int vocab) {
+                                    float* __restrict__ out, int hidden, int vocab,
+                                    const int* __restrict__ feed, int feed_count) {
   const int n = blockIdx.x;
   int id = ids[n];
+  if (id < 0 && feed != nullptr && -1 - id < feed_count) id = feed[-1 - id];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // ids are validated on the host; never read outside
   const T* row = table + (size_t)id * hidden;
   float* dst = out + (size_t)n * hidden;
@@ -16,13 +20,13 @@ __global__ void embed_gather_kernel(const int* __restrict__ ids, const T* __rest
 }
 
 extern "C" int tw_embed_gather(int dtype, const int* ids, const void* table, float* out, int n,
-                               int hidden, int vocab, hipStream_t stream) {
-  TW_REQUIRE(n >= 0 && hidden > 0 && vocab > 0);
+                               int hidden, int vocab, const int* feed, int feed_count, hipStream_t stream) {
+  TW_REQUIRE(n >= 0 && hidden > 0 && vocab > 0 && feed_count >= 0);
   if (n == 0) return 0;
   if (dtype == TW_DTYPE_F32)
-    embed_gather_kernel<float><<<n, 256, 0, stream>>>(ids, (const float*)table, out, hidden, vocab);
+    embed_gather_kernel<float><<<n, 256, 0, stream>>>(ids, (const float*)table, out, hidden, vocab, feed, feed_count);
   else if (dtype == TW_DTYPE_BF16)
-    embed_gather_kernel<bf16_t><<<n, 256, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab);
+    embed_gather_kernel<bf16_t><<<n, 256, 0, stream>>>(ids, (const bf16_t*)table, out, hidden, vocab, feed, feed_count);
   else
     return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();

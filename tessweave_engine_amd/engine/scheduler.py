@@ -15,6 +15,15 @@ batch for the step function, under a token budget (`max_step_tokens`); several
 prompts may advance in a turn if the budget allows; the portion size is fixed
 unless `adaptive_chunk` asks for the reference's wall-clock feedback
 (engine.py:262-268); sampling runs on the device.
+
+Lookahead (`EngineConfig.lookahead`, on the GPU): a turn is put on the device
+BEFORE the tokens of the turn before it are read. A request's newest token is then
+named by its row in the sampler's output and resolved on the device, and the host
+reads and commits tokens one turn late, while the device already runs the next
+turn; the host's work between turns no longer leaves the device idle. A request
+that turns out to have ended (EOS) has then run one token too far: that token is
+dropped, and what it wrote lies beyond anything the prefix index publishes. The
+tokens a request gets are the same with and without lookahead.
 """
 from __future__ import annotations
 
@@ -47,6 +56,8 @@ class Request:
     tokens: list = field(default_factory=list)       # prompt + generated
     output: list = field(default_factory=list)       # generated
     seq: object = None                               # cache.Sequence while admitted
+    issued: int = 0                                  # generated tokens, those still on the device included
+    feed_row: int = -1                               # row of the newest token in the sampler's output while unread
     cached: int = 0                                  # prompt tokens taken from the prefix index
     status: str = "waiting"
     created: float = field(default_factory=time.perf_counter)
@@ -100,6 +111,9 @@ class Engine:
         self.running = False
         self.thread = None
         self.fatal = None
+        self.lookahead = (bool(getattr(self.config, "lookahead", True)) and hasattr(self.sampler, "sample_async")
+                          and getattr(self.stepper, "accepts_token_feed", False))
+        self._inflight = None            # (PendingTokens, [(request, row)]) of the turn whose tokens are unread
         self.prefill_cursor = 0
         self.chunk = self.config.prefill_chunk
         self.prefill_ms_per_token = None
@@ -154,7 +168,7 @@ class Engine:
     def plan(self):
         """Which admitted requests run how many tokens in the next step (decisions only, no side effects
         beyond the round-robin cursor)."""
-        decode = [r for r in self.active if not r.prefilling]
+        decode = [r for r in self.active if not r.prefilling and r.issued < r.max_tokens]
         portions = [Portion(r, 1, True) for r in decode]
         prefill = [r for r in self.active if r.prefilling]
         if prefill:
@@ -175,37 +189,77 @@ class Engine:
         return portions
 
     def step(self):
-        """One scheduler turn; False when nothing is admitted."""
+        """One scheduler turn; False when nothing is admitted and no token is unread."""
         with self.lock:
             self._admit()
-            if not self.active:
-                return False
+            portions = self.plan() if self.active else []
+            if not portions:
+                if self._inflight is None:
+                    return False
+                self._collect()              # nothing new to run: read what the last turn sampled
+                return True
             started = time.perf_counter()
-            portions = self.plan()
+            if self.lookahead:
+                feed = self.sampler.out_buffer
+                if getattr(self.stepper, "token_feed", None) is not feed:
+                    self.stepper.set_token_feed(feed)
             entries = []
             for p in portions:
                 r = p.request
                 begin = r.computed
-                entries.append(StepEntry(r.seq, r.tokens[begin:begin + p.count], [p.count - 1] if p.samples else []))
+                if begin == len(r.tokens):   # its newest token is still on the device: name it by its row
+                    tokens = [-1 - r.feed_row]
+                else:
+                    tokens = r.tokens[begin:begin + p.count]
+                entries.append(StepEntry(r.seq, tokens, [p.count - 1] if p.samples else []))
             logits = self.stepper.step(entries)
             sampled = [p for p in portions if p.samples]
-            ids = self.sampler.sample(logits, [p.request.temperature for p in sampled],
-                                      [p.request.seed for p in sampled],
-                                      [len(p.request.output) for p in sampled]) if sampled else []
-            if not sampled and self.config.adaptive_chunk and hasattr(self.stepper, "synchronize"):
+            arguments = (logits, [p.request.temperature for p in sampled], [p.request.seed for p in sampled],
+                         [p.request.issued for p in sampled])
+            previous = self._inflight
+            if not sampled:
+                self._inflight = None
+            elif self.lookahead:
+                self._inflight = (self.sampler.sample_async(*arguments), [(p.request, i) for i, p in enumerate(sampled)])
+            else:
+                ids = self.sampler.sample(*arguments)
+                self._inflight = (ids, [(p.request, i) for i, p in enumerate(sampled)])
+            for i, p in enumerate(sampled):
+                p.request.issued += 1
+                p.request.feed_row = i
+            if previous is not None:
+                self._collect(previous)      # the turn before, read while the device runs this one
+            if not self.lookahead:
+                self._collect()
+            elif not sampled and self.config.adaptive_chunk and hasattr(self.stepper, "synchronize"):
                 self.stepper.synchronize()      # nothing was read back: wait so that the timing is real
             elapsed = (time.perf_counter() - started) * 1000
             self.counters["steps"] += 1
             n_prompt = sum(p.count for p in portions if p.prompt)
             self.counters["prefill_tokens"] += n_prompt
-            for p, token in zip(sampled, ids):
-                self._commit(p.request, int(token))
             self.trace.emit("step", request_ids=[p.request.id for p in portions], batch=len(portions),
                             tokens=sum(p.count for p in portions), prompt_tokens=n_prompt,
                             elapsed_ms=elapsed, prefill_chunk=self.chunk, **self.cache.stats())
             if self.config.adaptive_chunk and n_prompt:
                 self._adapt_chunk(elapsed, n_prompt)
             return True
+
+    def flush(self):
+        """Read and commit the tokens of the last turn, if they are still unread (lookahead)."""
+        with self.lock:
+            self._collect()
+
+    def _collect(self, turn=None):
+        """Read the tokens a turn sampled (waiting for them if need be) and commit them to their requests."""
+        if turn is None:
+            turn, self._inflight = self._inflight, None
+        if turn is None:
+            return
+        pending, rows = turn
+        ids = pending.result() if hasattr(pending, "result") else pending
+        for r, row in rows:
+            if r.id in self.requests and r.status == "active":     # else it ended meanwhile: the token is dropped
+                self._commit(r, int(ids[row]))
 
     def _adapt_chunk(self, elapsed_ms, prompt_tokens):
         # The reference's feedback (engine.py:262-268): EMA of prompt ms/token, portion sized to the turn budget.

@@ -36,9 +36,14 @@ def _round_up(v, m):
     return (v + m - 1) // m * m
 
 
+GRAPH_SEGMENT_RUNS = 8       # layer runs per captured graph after the first
+
+
 class _Graph:
-    def __init__(self, handle, logits, generation):
-        self.handle, self.logits, self.generation = handle, logits, generation
+    """A captured decode step: several graphs launched one after the other (see Stepper._capture)."""
+
+    def __init__(self, handles, logits, generation):
+        self.handles, self.logits, self.generation = handles, logits, generation
 
 
 class Stepper:
@@ -56,6 +61,7 @@ class Stepper:
         self.max_seqs = 0
         self._graphs = {}
         self._warm = set()
+        self.token_feed = None
         self._staging = []
         self._staging_events = []
         self._staging_next = 0
@@ -102,12 +108,27 @@ class Stepper:
             torch.cuda.synchronize(self.device)
             lib = library()
             for graph in self._graphs.values():
-                lib.tw_graph_destroy(graph.handle)
+                for handle in graph.handles:
+                    lib.tw_graph_destroy(handle)
         self._graphs = {}
         self._warm = set()
 
     def close(self):
         self._drop_graphs()
+
+    accepts_token_feed = True
+
+    def set_token_feed(self, feed):
+        """FEED (int32, on the device, or None): from now on a token id -1 - k in a step entry stands for
+        feed[k] as it is when the step runs, e.g. a token sampled by the step before that the host has not read."""
+        if feed is not None and (feed.dtype != torch.int32 or feed.device.type != "cuda" or not feed.is_contiguous()):
+            raise ValueError("the token feed must be a contiguous int32 tensor on the model's device")
+        same = (feed is None and self.token_feed is None) or \
+            (feed is not None and self.token_feed is not None and feed.data_ptr() == self.token_feed.data_ptr()
+             and feed.numel() == self.token_feed.numel())
+        if not same:
+            self._drop_graphs()          # captured steps hold the old pointer
+            self.token_feed = feed
 
     def synchronize(self):
         self.stream.synchronize()
@@ -154,6 +175,7 @@ class Stepper:
         Returns (context, entries in batch order, whether the step can be replayed from a graph).
         """
         vocab, seen = self.model.vocab_size, set()
+        feed = self.token_feed.numel() if self.token_feed is not None else 0     # ids -1 .. -feed name fed tokens
         for e in entries:
             if not e.tokens:
                 raise ValueError("a step entry needs at least one token")
@@ -162,7 +184,7 @@ class Stepper:
             seen.add(id(e.seq))
             if e.seq.closed:
                 raise ValueError(f"request {e.seq.id!r} is closed")
-            if any(type(t) is not int or t < 0 or t >= vocab for t in e.tokens):
+            if any(type(t) is not int or t >= vocab or t < -feed for t in e.tokens):
                 raise ValueError(f"request {e.seq.id!r}: token ids must be integers in [0, {vocab})")
             if any(type(w) is not int or w < 0 or w >= len(e.tokens) for w in e.want):
                 raise ValueError(f"request {e.seq.id!r}: wanted places must index this step's tokens")
@@ -242,6 +264,7 @@ class Stepper:
         ctx.kv_capacity = width * page
         ctx.max_tokens = self.max_tokens
         ctx.cache, ctx.workspace = self.cache, self.workspace
+        ctx.token_feed = self.token_feed
 
         graphable = (self.use_graphs and n_decode == n_seqs and n_logits == n_seqs
                      and rows == list(range(n_seqs)))
@@ -257,6 +280,50 @@ class Stepper:
         return np.maximum(0, computed - window + 1) // self.cache.page_size * self.cache.page_size
 
     # ---- HIP graphs for decode-only steps ------------------------------------------------
+    def _capture(self, ctx):
+        """Capture model.forward(ctx) as a chain of graphs.
+
+        Launching a graph costs host time per node before its first kernel starts. The step is
+        therefore cut after the first layer run and then every GRAPH_SEGMENT_RUNS runs: the
+        first graph is short and starts at once, and every later one is launched while its
+        predecessor still runs.
+        """
+        lib = library()
+        stream = self.stream.cuda_stream
+        generation = self.workspace.generation
+        handles = []
+        n_runs = len(self.model.schedule)
+
+        def end_segment():
+            handle = ctypes.c_void_p()
+            code = lib.tw_graph_end(stream, ctypes.byref(handle))
+            if code == 0:
+                handles.append(handle)
+            return code
+
+        def segment_end(i):
+            if i + 1 < n_runs and (i == 0 or (i + 1) % GRAPH_SEGMENT_RUNS == 0):
+                check(end_segment(), "graph capture end")
+                check(lib.tw_graph_begin(stream), "graph capture begin")
+
+        check(lib.tw_graph_begin(stream), "graph capture begin")
+        ctx.segment_end = segment_end
+        try:
+            logits = self.model.forward(ctx)
+        except BaseException:
+            end_segment()
+            for handle in handles:
+                lib.tw_graph_destroy(handle)
+            raise
+        finally:
+            ctx.segment_end = None
+        check(end_segment(), "graph capture end")
+        if self.workspace.generation != generation:
+            for handle in handles:
+                lib.tw_graph_destroy(handle)
+            raise RuntimeError("a scratch buffer was allocated during graph capture")
+        return _Graph(handles, logits, generation)
+
     def _run_graphable(self, ctx, n_seqs):
         graph = self._graphs.get(n_seqs)
         if graph is not None and graph.generation != self.workspace.generation:
@@ -267,19 +334,9 @@ class Stepper:
                 # First time at this batch size: run eagerly so every scratch buffer exists.
                 self._warm.add(n_seqs)
                 return self.model.forward(ctx)
-            lib = library()
-            generation = self.workspace.generation
-            handle = ctypes.c_void_p()
-            check(lib.tw_graph_begin(self.stream.cuda_stream), "graph capture begin")
-            try:
-                logits = self.model.forward(ctx)
-            finally:
-                code = lib.tw_graph_end(self.stream.cuda_stream, ctypes.byref(handle))
-            check(code, "graph capture end")
-            if self.workspace.generation != generation:
-                lib.tw_graph_destroy(handle)
-                raise RuntimeError("a scratch buffer was allocated during graph capture")
-            graph = self._graphs[n_seqs] = _Graph(handle, logits, generation)
-        check(library().tw_graph_launch(graph.handle, self.stream.cuda_stream), "graph launch")
+            graph = self._graphs[n_seqs] = self._capture(ctx)
+        lib = library()
+        for handle in graph.handles:
+            check(lib.tw_graph_launch(handle, self.stream.cuda_stream), "graph launch")
         self.graph_replays += 1
         return graph.logits

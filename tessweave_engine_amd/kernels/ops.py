@@ -44,14 +44,16 @@ def dtype_id(dtype):
     return _DTYPE_ID[dtype]
 
 
-def embed_gather(ids, table, out):
-    """out[n, :] = float32(table[ids[n], :])."""
+def embed_gather(ids, table, out, feed=None):
+    """out[n, :] = float32(table[ids[n], :]); an id -1 - k stands for feed[k] (int32, on the device)."""
     n = ids.numel()
     vocab, hidden = table.shape
     _need(table.is_contiguous() and out.is_contiguous(), "embedding operands must be contiguous")
     _need(tuple(out.shape) == (n, hidden), "embedding output has the wrong shape")
     check(library().tw_embed_gather(dtype_id(table.dtype), _dev(ids, torch.int32, "ids"), _dev(table),
-                                    _dev(out, torch.float32, "out"), n, hidden, vocab, _stream()),
+                                    _dev(out, torch.float32, "out"), n, hidden, vocab,
+                                    _dev(feed, torch.int32, "feed") if feed is not None else None,
+                                    feed.numel() if feed is not None else 0, _stream()),
           "embed_gather")
     return out
 

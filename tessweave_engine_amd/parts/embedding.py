@@ -27,7 +27,7 @@ class TokenEmbedding(Part):
 
     def forward(self, ctx):
         x = ctx.scratch("residual", (ctx.n_tokens, self.hidden), torch.float32)
-        return ops.embed_gather(ctx.token_ids, self.weight, x)
+        return ops.embed_gather(ctx.token_ids, self.weight, x, feed=ctx.token_feed)
 
 
 class OutputHead(Part):

@@ -99,8 +99,10 @@ class DecoderModel(Part):
         """Run the step's tokens; float32 logits [n_logits, vocab] at ctx.logit_rows."""
         x = self.embedding.forward(ctx)
         pending = None              # partial sums a block left for the next norm to add into x
-        for run in self.schedule:
+        for i, run in enumerate(self.schedule):
             pending = self.blocks[run.block].forward(ctx, run, x, pending)
+            if ctx.segment_end is not None:
+                ctx.segment_end(i)
         if ctx.n_logits == 0:
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=ctx.device)
         h = self.final_norm.forward(ctx, x, rows=ctx.logit_rows, add=pending, tag="norm.final")

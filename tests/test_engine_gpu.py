@@ -1,5 +1,6 @@
 """The engine on the GPU: generation through the entry point, long decoding, sampling, prefix reuse,
 each part alone, schedules that name a layer twice or share a cache, and a toy mixer with its own state."""
+import dataclasses
 import json
 import math
 
@@ -109,6 +110,34 @@ def test_sampling_seed_is_independent_of_other_requests(tiny):
     e.drain()
     assert cold.output == plain.greedy(tiny["config"], tiny["weights"], p[0], 7)
     e.close()
+
+
+def test_lookahead_and_reading_every_turn_give_the_same_tokens(tiny):
+    """Turns put on the device before the last turn's tokens are read (the default) against reading every turn:
+    greedy and sampled requests, staggered arrivals, and a request that ends on EOS one turn before the host knows."""
+    prompts = prompts_for(tiny, [3, 21, 40, 8], seed=31)
+    greedy = plain.greedy(tiny["config"], tiny["weights"], prompts[0], 12)
+    first = {}
+    for i, t in enumerate(greedy):
+        first.setdefault(t, i)
+    eos = max(first, key=first.get)                  # the token that first appears latest ends the request there
+    outs = []
+    for look in (True, False):
+        e = engine(tiny, no_lookahead=not look)
+        assert e.lookahead == look
+        e.model_config = dataclasses.replace(e.model_config, eos_token_ids=(eos,))
+        rs = [e.submit(prompts[0], 12), e.submit(prompts[1], 9, temperature=0.7, seed=4, ignore_eos=True)]
+        for _ in range(3):
+            e.step()
+        rs += [e.submit(prompts[2], 5, ignore_eos=True), e.submit(prompts[3], 11, temperature=1.3, seed=6, ignore_eos=True)]
+        e.drain()
+        outs.append([(r.output, r.status) for r in rs])
+        stats = e.stats()
+        assert stats["free_blocks"] == stats["physical_blocks"]
+        e.close()
+    assert outs[0] == outs[1]
+    assert outs[0][0] == (greedy[:greedy.index(eos) + 1], "stop")
+    assert outs[0][2] == (plain.greedy(tiny["config"], tiny["weights"], prompts[2], 5), "length")
 
 
 def test_prefix_pages_are_reused_on_the_gpu(tiny):

@@ -299,3 +299,142 @@ def test_generate_convenience_and_worker_thread():
         got.append(ev["token_id"])
     assert got == expected([5, 5, 5], 3) and e.stats()["finished"] == 3
     e.close()
+
+
+# ---- lookahead: a turn is put on the device before the tokens of the turn before are read ----------
+class FeedStepper(FakeStepper):
+    """A step function that knows prompt tokens only; a negative id -1 - k is read from the token feed when
+    the step runs, as the device does. Its logits come from the tokens IT has seen, not from the host's list."""
+    accepts_token_feed = True
+    token_feed = None
+
+    def set_token_feed(self, feed):
+        self.token_feed = feed
+
+    def step(self, entries):
+        rows = []
+        self.batches.append([(e.seq.id, e.seq.computed, len(e.tokens), list(e.want)) for e in entries])
+        for e in entries:
+            self.cache.ensure(e.seq, e.seq.computed + len(e.tokens))
+            h = self.history.setdefault(e.seq.id, [])
+            h.extend(self.full[e.seq.id][len(h):e.seq.computed])          # prefix-shared prompt tokens never ran here
+            assert len(h) == e.seq.computed
+            for t in e.tokens:
+                assert t >= 0 or self.token_feed is not None
+                h.append(t if t >= 0 else self.token_feed[-1 - t])
+            self.fed += sum(t < 0 for t in e.tokens)
+            for w in e.want:
+                rows.append((e, e.seq.computed + w + 1))
+        logits = torch.zeros(len(rows), VOCAB)
+        for i, (e, upto) in enumerate(rows):
+            logits[i, next_token(self.history[e.seq.id][:upto])] = 1.0
+        for e in entries:
+            self.cache.advance(e.seq, e.seq.computed + len(e.tokens))
+        return logits
+
+    fed = 0
+
+
+class FeedSampler(FakeSampler):
+    """Writes ids into one buffer that every call overwrites (the device's), hands back a copy later."""
+
+    def __init__(self):
+        self.out_buffer = [0] * 16
+        self.unread = 0
+
+    def sample_async(self, logits, temperatures, seeds, counters):
+        ids = self.sample(logits, temperatures, seeds, counters)
+        self.out_buffer[:len(ids)] = ids
+        self.unread += 1
+        sampler = self
+
+        class Pending:
+            def result(self):
+                sampler.unread -= 1
+                return list(ids)
+        return Pending()
+
+
+def make_lookahead(cfg=CFG, **kw):
+    defaults = dict(block_size=4, kv_blocks=32, max_context=64, prefill_chunk=4, min_prefill_chunk=1, dtype="float32")
+    defaults.update(kw)
+    config = EngineConfig(**defaults)
+    model = build_model(config_from_dict(cfg))
+    cache = CacheManager(model.cache_layout(), config.block_size, config.kv_blocks, config.max_active,
+                         prefix_cache=config.prefix_cache, max_request_tokens=config.max_context)
+    stepper = FeedStepper(cache)
+    stepper.full = {}
+    engine = Engine(model, config, stepper=stepper, cache=cache, sampler=FeedSampler())
+    submit = engine.submit
+
+    def tracked(tokens, *a, **k):
+        r = submit(tokens, *a, **k)
+        stepper.full[r.id] = list(tokens)                              # the prompt only
+        return r
+    engine.submit = tracked
+    return engine, stepper
+
+
+def test_lookahead_gives_the_same_tokens_one_turn_late():
+    e, s = make_lookahead()
+    assert e.lookahead
+    prompts = [[4, 5, 6, 7, 8], [2, 3, 4, 5, 6, 7, 8, 9, 10], [9]]
+    counts = [7, 3, 1]
+    rs = [e.submit(p, n) for p, n in zip(prompts, counts)]
+    seen_unread = 0
+    for _ in range(200):
+        if not e.step():
+            break
+        seen_unread = max(seen_unread, e.sampler.unread)
+        assert e.sampler.unread <= 1                                   # at most one turn's tokens are unread
+    assert seen_unread == 1 and s.fed > 0                              # turns did run ahead of the host
+    for r, p, n in zip(rs, prompts, counts):
+        assert r.output == expected(p, n) and r.status == "length" and r.issued == n
+    assert e._inflight is None and not e.requests
+    e.cache.check()
+    # no request ever ran past prompt + max_tokens - 1 positions
+    for r, p, n in zip(rs, prompts, counts):
+        assert len(s.history[r.id]) == len(p) + n - 1
+    e.close()
+    assert len(e.cache.pools[0].free) == 32
+    # the same schedule of batches as without lookahead, apart from the reading
+    e2, s2 = make(lookahead=False)
+    for p, n in zip(prompts, counts):
+        e2.submit(p, n)
+    drain(e2)
+    shape = lambda batches: [[(start, n, w) for _, start, n, w in b] for b in batches]
+    assert shape(s.batches)[:3] == shape(s2.batches)[:3]
+    e2.close()
+
+
+def test_lookahead_drops_the_token_after_eos_and_frees_the_pages():
+    prompt = [3, 4, 5, 6, 7]
+    want = expected(prompt, 12)
+    end = next(i for i in range(2, 12) if want[i] not in want[:i])
+    e, s = make_lookahead(cfg=dict(CFG, eos_token_id=want[end]))
+    r = e.submit(prompt, 12)
+    other = e.submit([11, 12, 13], 12, ignore_eos=True)
+    drain(e)
+    assert r.status == "stop" and r.output == want[:end + 1]            # EOS is part of the output, nothing after it
+    assert len(s.history[r.id]) == len(prompt) + end + 1               # ... though the device ran EOS's own step
+    assert other.status == "length" and other.output == expected([11, 12, 13], 12)
+    e.cache.check()
+    e.close()
+    assert len(e.cache.pools[0].free) == 32
+
+
+def test_lookahead_with_cancel_failure_and_prefix_reuse():
+    e, s = make_lookahead(prefix_cache=True)
+    shared = list(range(1, 13))
+    a = e.submit(shared + [20], 4)
+    drain(e)
+    b = e.submit(shared + [21], 4)                                      # 12 tokens = 3 pages come from the index
+    c = e.submit([5, 6], 8)
+    e.step(); e.step()
+    e.cancel(c.id)                                                      # while one of its tokens is unread
+    drain(e)
+    assert b.cached == 12 and b.output == expected(shared + [21], 4) and a.output == expected(shared + [20], 4)
+    assert c.status == "cancelled"
+    e.cache.check()
+    e.close()
+    assert len(e.cache.pools[0].free) == 32
