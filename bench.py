@@ -165,7 +165,8 @@ def main():
         points[f"decode_b{b}"] = round(tps, 1)
 
     line = {
-        "metric": "decode tok/s @ batch 8, Qwen2.5-7B shape bf16 (+ prefill tok/s @ 2048, decode @ batch 1/64)",
+        "metric": f"decode tok/s @ batch {args.batch}, Qwen2.5-7B shape {'bf16' if args.dtype == 'bfloat16' else 'fp32'} "
+                  f"(+ prefill tok/s @ {t}, decode @ batch {args.points or '-'})",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",

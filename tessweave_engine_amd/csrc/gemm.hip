@@ -33,6 +33,108 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p
 
 __device__ __forceinline__ float tw_silu(float g) { return g / (1.0f + expf(-g)); }
 
+// Epilogue of the tiled kernels: each wave passes its tile through LDS (32 rows at a time) so
+// that a lane stores 8 consecutive columns of one row, whole cache lines instead of 2- or 4-byte
+// pieces; bias, residual, the output type and the SiLU-multiply of GLU pairs are applied here.
+// `lds` must hold 4 waves x 32 rows x (32 * WN + 4) floats and no wave may still read its old contents
+// (the first __syncthreads below sees to that).
+template <typename OutT, int WM, int WN, bool GLU>
+__device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* lds, const float* __restrict__ bias,
+                                                  const float* residual, long ldr, OutT* C, long ldc, int M, int N,
+                                                  int m0, int n0, int wm0, int wn0, int wave, int lane) {
+  const int r = lane & 31, g = lane >> 5;
+  constexpr int WCOLS = 32 * WN;                             // columns of a wave tile
+  constexpr int EROW = WCOLS + 4;                            // floats per staged row, padded
+  // (the launcher asks for max(pipeline stages, 4 waves x 32 rows x EROW floats) bytes of LDS)
+  float* stage = reinterpret_cast<float*>(lds) + wave * 32 * EROW;
+  constexpr int CPR = WCOLS / 8;                             // 8-column groups per row
+  const bool vec_ok = (ldc % 8 == 0) && (residual == nullptr || ldr % 4 == 0) &&
+                      ((uintptr_t)C % 16 == 0) && ((uintptr_t)residual % 16 == 0);
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    __syncthreads();                                          // the pipeline's (or the last round's) LDS reads are done
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * g + (e % 4)) * EROW + j * 32 + r] = acc[i][j][e];
+    __syncthreads();
+    if (GLU) {
+      // a wave tile's columns are [gate 16 | up 16] pairs; a lane forms 8 outputs of one row
+      constexpr int GPR = WCOLS / 16;                         // 8-output groups per row
+#pragma unroll
+      for (int q = lane; q < 32 * GPR; q += 64) {
+        const int lr = q / GPR, og = q % GPR;
+        const int lc = (og >> 1) * 32 + (og & 1) * 8;         // gate columns lc.., up columns lc + 16..
+        const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
+        if (row >= M || col + 24 > N) continue;               // N is a multiple of 32: groups are whole
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float gv = stage[lr * EROW + lc + e], uv = stage[lr * EROW + lc + 16 + e];
+          if (bias) { gv += bias[col + e]; uv += bias[col + 16 + e]; }
+          v[e] = tw_silu(gv) * uv;
+        }
+        OutT* dst = C + (size_t)row * ldc + (n0 + wn0) / 2 + (og >> 1) * 16 + (og & 1) * 8;
+        if (ldc % 8 == 0 && (uintptr_t)C % 16 == 0) {
+          if (sizeof(OutT) == 4) {
+            *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
+          } else {
+            bf16x8 o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
+            *reinterpret_cast<bf16x8*>(dst) = o;
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dst[e] = tw_from_float<OutT>(v[e]);
+        }
+      }
+      continue;
+    }
+#pragma unroll
+    for (int q = lane; q < 32 * CPR; q += 64) {
+      const int lr = q / CPR, lc = (q % CPR) * 8;
+      const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
+      if (row >= M || col >= N) continue;
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = stage[lr * EROW + lc + e];
+      if (bias) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) v[e] += bias[col + e];
+      }
+      if (vec_ok && col + 8 <= N) {
+        if (residual) {
+          const f32x4 r0 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col);
+          const f32x4 r1 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { v[e] += r0[e]; v[4 + e] += r1[e]; }
+        }
+        OutT* dst = C + (size_t)row * ldc + col;
+        if (sizeof(OutT) == 4) {
+          *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+          *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
+        } else {
+          bf16x8 o;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
+          *reinterpret_cast<bf16x8*>(dst) = o;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (col + e < N) {
+            float x = v[e];
+            if (residual) x += residual[(size_t)row * ldr + col + e];
+            C[(size_t)row * ldc + col + e] = tw_from_float<OutT>(x);
+          }
+      }
+    }
+  }
+}
+
 // =====================================================================================
 // Tiled kernel. Workgroup = 4 waves in a 2x2 grid, wave tile (32*WM) x (32*WN).
 // One stage holds 128 bytes of K per row (64 bf16 / 32 f32), rows padded to 144
@@ -215,98 +317,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
     __syncthreads();
   }
 
-  // ---- epilogue: each wave passes its tile through LDS (32 rows at a time) so that a lane
-  // stores 8 consecutive columns of one row: whole cache lines instead of 2- or 4-byte pieces.
-  constexpr int WCOLS = 32 * WN;                             // columns of a wave tile
-  constexpr int EROW = WCOLS + 4;                            // floats per staged row, padded
-  // (the launcher asks for max(pipeline stages, 4 waves x 32 rows x EROW floats) bytes of LDS)
-  float* stage = reinterpret_cast<float*>(lds) + wave * 32 * EROW;
-  constexpr int CPR = WCOLS / 8;                             // 8-column groups per row
-  const bool vec_ok = (ldc % 8 == 0) && (residual == nullptr || ldr % 4 == 0) &&
-                      ((uintptr_t)C % 16 == 0) && ((uintptr_t)residual % 16 == 0);
-#pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    __syncthreads();                                          // the pipeline's (or the last round's) LDS reads are done
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * g + (e % 4)) * EROW + j * 32 + r] = acc[i][j][e];
-    __syncthreads();
-    if (GLU) {
-      // a wave tile's columns are [gate 16 | up 16] pairs; a lane forms 8 outputs of one row
-      constexpr int GPR = WCOLS / 16;                         // 8-output groups per row
-#pragma unroll
-      for (int q = lane; q < 32 * GPR; q += 64) {
-        const int lr = q / GPR, og = q % GPR;
-        const int lc = (og >> 1) * 32 + (og & 1) * 8;         // gate columns lc.., up columns lc + 16..
-        const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
-        if (row >= M || col + 24 > N) continue;               // N is a multiple of 32: groups are whole
-        float v[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float gv = stage[lr * EROW + lc + e], uv = stage[lr * EROW + lc + 16 + e];
-          if (bias) { gv += bias[col + e]; uv += bias[col + 16 + e]; }
-          v[e] = tw_silu(gv) * uv;
-        }
-        OutT* dst = C + (size_t)row * ldc + (n0 + wn0) / 2 + (og >> 1) * 16 + (og & 1) * 8;
-        if (ldc % 8 == 0 && (uintptr_t)C % 16 == 0) {
-          if (sizeof(OutT) == 4) {
-            *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
-          } else {
-            bf16x8 o;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
-            *reinterpret_cast<bf16x8*>(dst) = o;
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) dst[e] = tw_from_float<OutT>(v[e]);
-        }
-      }
-      continue;
-    }
-#pragma unroll
-    for (int q = lane; q < 32 * CPR; q += 64) {
-      const int lr = q / CPR, lc = (q % CPR) * 8;
-      const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
-      if (row >= M || col >= N) continue;
-      float v[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = stage[lr * EROW + lc + e];
-      if (bias) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (col + e < N) v[e] += bias[col + e];
-      }
-      if (vec_ok && col + 8 <= N) {
-        if (residual) {
-          const f32x4 r0 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col);
-          const f32x4 r1 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col + 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { v[e] += r0[e]; v[4 + e] += r1[e]; }
-        }
-        OutT* dst = C + (size_t)row * ldc + col;
-        if (sizeof(OutT) == 4) {
-          *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-          *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
-        } else {
-          bf16x8 o;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
-          *reinterpret_cast<bf16x8*>(dst) = o;
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (col + e < N) {
-            float x = v[e];
-            if (residual) x += residual[(size_t)row * ldr + col + e];
-            C[(size_t)row * ldc + col + e] = tw_from_float<OutT>(x);
-          }
-      }
-    }
-  }
+  tw_tiled_epilogue<OutT, WM, WN, GLU>(acc, lds, bias, residual, ldr, C, ldc, M, N, m0, n0, wm0, wn0, wave, lane);
 }
 
 // =====================================================================================
