@@ -57,6 +57,7 @@ struct AttnArgs {
   float scale;
   int splits;
   int page_shift;         // log2(page_size) if it is a power of two, else -1
+  int n_seqs, max_tiles;  // prefill (bfloat16 kernel): sequences of the launch, 128-row tiles of the longest
 };
 
 // Per-wave online-softmax state for one 16-row tile. Lane (r, g) belongs to row r.
@@ -624,16 +625,38 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int G = a.q_heads / a.kv_heads;
-  const int kvh = blockIdx.y;
-  const int seq = a.seq0 + blockIdx.z;
+  // Which tile this workgroup takes. Tiles are ranked by the keys they see (most first: rank =
+  // tile-from-the-end major, then kv head and sequence). Workgroups are handed to the 8 XCDs in
+  // turn and, within an XCD, to its 32 CUs in turn; while all of them are resident (at most two
+  // per CU), a CU's second workgroup is given the rank that evens out the sum of the two, and the
+  // CUs that get one workgroup the heaviest ranks. With more workgroups than that, heaviest first.
+  int rank;
+  {
+    const int total = gridDim.x, b = blockIdx.x, xcd = b & 7, j = b >> 3;
+    const int n = (total - xcd + 7) >> 3;                       // workgroups of this XCD
+    constexpr int C = 32;
+    int r = j;
+    if (n > C && n <= 2 * C) {
+      const int paired = n - C, single = C - paired;
+      if (j < paired) r = single + j;                           // first of a pair
+      else if (j < C) r = j - paired;                           // alone on its CU: the heaviest
+      else r = n - 1 - (j - C);                                 // second of a pair: mirrors the first
+    }
+    rank = r * 8 + xcd;
+    if (rank >= total) rank = b;                                 // (uneven XCD shares: keep every tile covered)
+  }
+  const int per_tile = a.kv_heads * a.n_seqs;
+  const int tile_from_end = rank / per_tile, sub = rank % per_tile;
+  const int kvh = sub % a.kv_heads;
+  const int seq = a.seq0 + sub / a.kv_heads;
   const int kv_len = a.kv_len[seq];
   const int token0 = a.q_start[seq];
   const int q_len = a.q_start[seq + 1] - token0;
   const int rows = q_len * G;
-  // the tiles that see the most keys start first
   const int n_tiles = (rows + 127) / 128;
-  if ((int)blockIdx.x >= n_tiles) return;
-  const int wg_row0 = (n_tiles - 1 - blockIdx.x) * 128;
+  const int tile_idx = a.max_tiles - 1 - tile_from_end;         // counted from the longest sequence's last tile
+  if (tile_idx < 0 || tile_idx >= n_tiles) return;
+  const int wg_row0 = tile_idx * 128;
   const int* table = a.block_table + (size_t)seq * a.table_stride;
   const int D = a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
   const int pshift = a.page_shift, pmask = P - 1;
@@ -692,8 +715,9 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     const int q = tid + i * 256, key = q / CH, chunk = q % CH;
     k_use[i] = key < 32 && chunk < chunks;
     k_key[i] = key;
-    k_slot[i] = P >= 32 ? 0 : (key >> pshift);             // which of the block's pages
-    k_goff[i] = (P >= 32 ? key : (key & pmask)) * D + chunk * 8;
+    const int key_c = min(key, 31), chunk_c = min(chunk, chunks - 1);   // an unused piece loads a used one's bytes
+    k_slot[i] = P >= 32 ? 0 : (key_c >> pshift);           // which of the block's pages
+    k_goff[i] = (P >= 32 ? key_c : (key_c & pmask)) * D + chunk_c * 8;
     k_loff[i] = key * KROW + chunk * 16;
   }
 #pragma unroll
@@ -702,68 +726,55 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     v_use[i] = d < D;
     v_oct[i] = oct;
     v_slot[i] = P >= 32 ? 0 : ((8 * oct) >> pshift);
-    v_goff[i] = d * P + (P >= 32 ? 8 * oct : ((8 * oct) & pmask));
+    v_goff[i] = min(d, D - 1) * P + (P >= 32 ? 8 * oct : ((8 * oct) & pmask));
     v_loff[i] = d * TW_PF_VROW + oct * 16;
   }
-  auto fetch = [&](int blk_v) {                              // global -> registers
+  // global -> registers. Loads carry no predicate: a page of the block that holds no key of
+  // [lo, kv_len) may not be held at all and is replaced by one of the block that is, so every
+  // address lies inside the pool; what such keys hold never counts (their scores are selected
+  // to -inf) except in the PV product, so their VALUES are made zero here, in the rare block
+  // that crosses the end of the sequence or the start of the window.
+  auto fetch = [&](int blk_v) {
     const int blk = __builtin_amdgcn_readfirstlane(blk_v);
     const int p0 = blk * 32;
     const int first = p0 >> pshift;
     int pg[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pg[i] = (i < ppb && p0 + (i << pshift) < kv_len) ? table[first + i] : -1;
-    const int in_page = P >= 32 ? (p0 & pmask) : 0;          // where the block starts inside its page
-    if (p0 >= lo && p0 + 32 <= kv_len && pg[0] >= 0 && (ppb < 2 || pg[1] >= 0) && (ppb < 4 || (pg[2] >= 0 && pg[3] >= 0))) {
-      // every key of the block is inside the sequence: no predicates, page bases in scalar registers
-      size_t kb[4], vb[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const size_t base = ((size_t)(i < ppb ? pg[i] : pg[0]) * a.kv_heads + kvh) * head_stride;
-        kb[i] = base + (size_t)in_page * D;
-        vb[i] = base + in_page;
-      }
-#pragma unroll
-      for (int i = 0; i < KPIECES; ++i) {
-        const int sl = k_slot[i];
-        const size_t base = sl == 0 ? kb[0] : (sl == 1 ? kb[1] : (sl == 2 ? kb[2] : kb[3]));
-        if (k_use[i]) kreg[i] = tw_load_frag(keys + base + k_goff[i]);
-      }
-#pragma unroll
-      for (int i = 0; i < VPIECES; ++i) {
-        const int sl = v_slot[i];
-        const size_t base = sl == 0 ? vb[0] : (sl == 1 ? vb[1] : (sl == 2 ? vb[2] : vb[3]));
-        if (v_use[i]) vreg[i] = tw_load_frag(values + base + v_goff[i]);
-      }
-      return;
+    for (int i = 0; i < 4; ++i) {
+      const int a0 = P >= 32 ? p0 : p0 + (i << pshift);
+      const int a1 = P >= 32 ? p0 + 31 : a0 + P - 1;
+      pg[i] = (i < ppb && a0 < kv_len && a1 >= lo) ? table[first + i] : -1;
     }
-    // a block at the edge of the sequence: keys outside it are loaded as zeros
-    auto page_of = [&](int ko) {
-      const int i = P >= 32 ? 0 : (ko >> pshift);
-      return i == 0 ? pg[0] : (i == 1 ? pg[1] : (i == 2 ? pg[2] : pg[3]));
-    };
+    int safe = pg[0] >= 0 ? pg[0] : (pg[1] >= 0 ? pg[1] : (pg[2] >= 0 ? pg[2] : pg[3]));
+    if (safe < 0) safe = 0;
+    const int in_page = P >= 32 ? (p0 & pmask) : 0;          // where the block starts inside its page
+    size_t kb[4], vb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const size_t base = ((size_t)(pg[i] >= 0 ? pg[i] : safe) * a.kv_heads + kvh) * head_stride;
+      kb[i] = base + (size_t)in_page * D;
+      vb[i] = base + in_page;
+    }
 #pragma unroll
     for (int i = 0; i < KPIECES; ++i) {
-      const int p = p0 + k_key[i];
-      int page = k_use[i] ? page_of(k_key[i]) : -1;
-      if (p >= kv_len || p < lo) page = -1;
-      const size_t base = ((size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh) * head_stride;
-      kreg[i] = page >= 0 ? tw_load_frag(keys + base + (unsigned)(p & pmask) * D + (k_loff[i] - k_key[i] * KROW) / 2)
-                          : Elem<bf16_t>::zero();
+      const int sl = k_slot[i];
+      const size_t base = sl == 0 ? kb[0] : (sl == 1 ? kb[1] : (sl == 2 ? kb[2] : kb[3]));
+      kreg[i] = tw_load_frag(keys + base + k_goff[i]);
     }
 #pragma unroll
     for (int i = 0; i < VPIECES; ++i) {
-      const int p = p0 + 8 * v_oct[i];
-      int page = v_use[i] ? page_of(8 * v_oct[i]) : -1;
-      if (p >= kv_len || p + 7 < lo) page = -1;
-      const size_t base = ((size_t)(page < 0 ? 0 : page) * a.kv_heads + kvh) * head_stride;
-      const int d = (v_loff[i] - v_oct[i] * 16) / TW_PF_VROW;
-      bf16x8 v = page >= 0 ? tw_load_frag(values + base + (unsigned)d * P + (p & pmask)) : Elem<bf16_t>::zero();
-      if (page >= 0 && (p + 8 > kv_len || p < lo)) {
+      const int sl = v_slot[i];
+      const size_t base = sl == 0 ? vb[0] : (sl == 1 ? vb[1] : (sl == 2 ? vb[2] : vb[3]));
+      vreg[i] = tw_load_frag(values + base + v_goff[i]);
+    }
+    if (p0 + 32 > kv_len || p0 < lo) {
+#pragma unroll
+      for (int i = 0; i < VPIECES; ++i) {
+        const int p = p0 + 8 * v_oct[i];
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          if (p + e >= kv_len || p + e < lo) v[e] = (bf16_t)0.f;
+          if (p + e >= kv_len || p + e < lo) vreg[i][e] = (bf16_t)0.f;
       }
-      vreg[i] = v;
     }
   };
   auto stash = [&](int buf) {                                // registers -> LDS
@@ -782,9 +793,9 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     k_frag[tile] = lds_k + (8 * (r >> 2) + 4 * tile + (r & 3)) * KROW + g * 16;
   const char* v_frag = lds_v + r * TW_PF_VROW + g * 16;
 
-  // EDGE false: every key of the block is visible to every row of the wave (no masks).
-  auto compute = [&](int blk, int buf, auto edge_tag) {
-    constexpr bool EDGE = decltype(edge_tag)::value;
+  // edge: some key of the block is hidden from some row of the wave; only then are scores masked.
+  // The branch covers the masking alone, so the two cases share every register of the rest.
+  auto compute = [&](int blk, int buf, bool edge) {
     const int p0 = blk * 32;
     f32x4 s[2][2];
 #pragma unroll
@@ -803,31 +814,34 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
           tw_mma16(s[1][tile], kf, qf[1][st]);
         }
     }
+    if (edge) {
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) {
+        const int lo_row = a.window > 0 ? t_row[rt] - a.window + 1 : 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int p = p0 + 8 * g + e;
+          if (!(p <= t_row[rt] && p >= lo_row && p < kv_len)) s[rt][e >> 2][e & 3] = -INFINITY;
+        }
+      }
+    }
     bf16x8 pb[2];
     float alpha[2];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
-      float x[8];
       float mx = -INFINITY;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        x[e] = s[rt][e >> 2][e & 3] * c2;
-        if (EDGE) {
-          const int p = p0 + 8 * g + e;
-          const int lo_row = a.window > 0 ? t_row[rt] - a.window + 1 : 0;
-          if (!(p <= t_row[rt] && p >= lo_row && p < kv_len)) x[e] = -INFINITY;
-        }
-        mx = fmaxf(mx, x[e]);
-      }
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[rt][e >> 2][e & 3]);
       mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
-      const float m_new = fmaxf(m[rt], mx);
-      const float m_use = (EDGE && m_new == -INFINITY) ? 0.f : m_new;
+      // m is kept in the scaled log2 domain: m = max(score) * c2 (c2 > 0)
+      const float m_new = fmaxf(m[rt], mx * c2);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
       alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - m_use);
       float sum = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float pe = __builtin_amdgcn_exp2f(x[e] - m_use);
+        const float pe = __builtin_amdgcn_exp2f(fmaf(s[rt][e >> 2][e & 3], c2, -m_use));
         sum += pe;
         pb[rt][e] = (bf16_t)pe;
       }
@@ -838,38 +852,41 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     }
     // rescale the running output only if some row's maximum moved
     const bool moved = __any(alpha[0] != 1.f || alpha[1] != 1.f);
+    if (moved) {
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int dt = 0; dt < DTMAX; ++dt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[rt][dt][j] *= alpha[rt];
+    }
     const char* vbase = v_frag + buf * VSTAGE;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
       if (dt < dts) {
         const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
-#pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-          if (moved) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[rt][dt][j] *= alpha[rt];
-          }
-          tw_mma16(acc[rt][dt], vf, pb[rt]);
-        }
+        tw_mma16(acc[0][dt], vf, pb[0]);
+        tw_mma16(acc[1][dt], vf, pb[1]);
       }
+  };
+  auto compute_if_seen = [&](int blk, int buf) {
+    const int p0 = blk * 32;
+    if (wave_live && p0 <= wave_t_max)
+      compute(blk, buf, !(wave_full && p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len));
   };
 
   fetch(blk_begin);
   stash(0);
   __syncthreads();
-  for (int blk = blk_begin; blk < blk_end; ++blk) {
+  int blk = blk_begin;
+  for (; blk + 1 < blk_end; ++blk) {                        // every fetch unconditional: no register copies
     const int buf = (blk - blk_begin) & 1;
-    if (blk + 1 < blk_end) fetch(blk + 1);
-    if (wave_live && blk * 32 <= wave_t_max) {
-      const int p0 = blk * 32;
-      if (wave_full && p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len)
-        compute(blk, buf, BoolTag<false>());
-      else
-        compute(blk, buf, BoolTag<true>());
-    }
-    if (blk + 1 < blk_end) stash(buf ^ 1);
+    fetch(blk + 1);
+    compute_if_seen(blk, buf);
+    stash(buf ^ 1);
     __syncthreads();
   }
+  compute_if_seen(blk, (blk - blk_begin) & 1);                // the last block (blk_end > blk_begin always)
 
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
@@ -888,7 +905,11 @@ template <int DTMAX>
 static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
   const int G = a.q_heads / a.kv_heads;
   const long rows = (long)max_q_len * G;
-  dim3 grid(tw_div_up(rows, 128), a.kv_heads, n_seqs);
+  a.n_seqs = n_seqs;
+  a.max_tiles = (int)tw_div_up(rows, 128);
+  const long total = (long)a.max_tiles * a.kv_heads * n_seqs;
+  TW_REQUIRE(total < (1L << 30));
+  dim3 grid((unsigned)total);
   const size_t lds_bytes = 2 * 32 * (DTMAX * 32 + 16) + 2 * DTMAX * 16 * TW_PF_VROW;
   auto kernel = attn_prefill_bf16_kernel<DTMAX>;
   static bool attribute_set = false;
