@@ -359,10 +359,22 @@ def sampling_uniform(seed, counter):
     return float(library().tw_sampling_uniform(int(seed) & (2 ** 64 - 1), int(counter)))
 
 
-def sample_rows(logits, out, temperature=None, seeds=None, counters=None):
-    """out[r] = greedy (temperature 0 or None) or sampled token of logits[r]."""
+def sample_workspace_bytes(rows):
+    return int(library().tw_sample_workspace_bytes(int(rows)))
+
+
+def sample_rows(logits, out, temperature=None, seeds=None, counters=None, workspace=None):
+    """out[r] = greedy (temperature 0 or None) or sampled token of logits[r].
+
+    workspace: a device tensor of at least sample_workspace_bytes(rows) bytes (allocated here if None).
+    """
     rows, vocab, ld = _rows(logits, "logits")
     _need(out.numel() == rows, "one output id per row is needed")
+    need = sample_workspace_bytes(rows)
+    if workspace is None:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=logits.device)
+    _need(workspace.is_contiguous() and workspace.numel() * workspace.element_size() >= need,
+          "the sampling workspace is too small")
     if temperature is not None:
         _need(temperature.numel() == rows and seeds.numel() == rows and counters.numel() == rows,
               "one temperature, seed and counter per row are needed")
@@ -371,5 +383,6 @@ def sample_rows(logits, out, temperature=None, seeds=None, counters=None):
                                    _dev(temperature, torch.float32, "temperature") if temperature is not None else None,
                                    _dev(seeds) if temperature is not None else None,
                                    _dev(counters, torch.int32, "counters") if temperature is not None else None,
-                                   _dev(out, torch.int32, "out"), _stream()), "sample_rows")
+                                   _dev(out, torch.int32, "out"), _dev(workspace),
+                                   workspace.numel() * workspace.element_size(), _stream()), "sample_rows")
     return out

@@ -50,6 +50,7 @@ class DeviceSampler:
         self._seeds = torch.zeros(capacity, dtype=torch.int64, device=self.device)
         self._counters = torch.zeros(capacity, dtype=torch.int32, device=self.device)
         self._out = torch.zeros(capacity, dtype=torch.int32, device=self.device)
+        self._scratch = torch.empty(ops.sample_workspace_bytes(capacity), dtype=torch.uint8, device=self.device)
         self._ring = [dict(temps=torch.zeros(capacity, dtype=torch.float32, pin_memory=True),
                            seeds=torch.zeros(capacity, dtype=torch.int64, pin_memory=True),
                            counters=torch.zeros(capacity, dtype=torch.int32, pin_memory=True),
@@ -87,7 +88,7 @@ class DeviceSampler:
             slot["event"].synchronize()
         out = self._out[:rows]
         if all(t == 0 for t in temperatures):
-            ops.sample_rows(logits, out)
+            ops.sample_rows(logits, out, workspace=self._scratch)
         else:
             slot["temps"][:rows] = torch.tensor(temperatures, dtype=torch.float32)
             slot["seeds"][:rows] = torch.tensor([s & (2 ** 63 - 1) for s in seeds], dtype=torch.int64)
@@ -96,7 +97,7 @@ class DeviceSampler:
             self._seeds[:rows].copy_(slot["seeds"][:rows], non_blocking=True)
             self._counters[:rows].copy_(slot["counters"][:rows], non_blocking=True)
             ops.sample_rows(logits, out, temperature=self._temps[:rows], seeds=self._seeds[:rows],
-                            counters=self._counters[:rows])
+                            counters=self._counters[:rows], workspace=self._scratch)
         slot["out"][:rows].copy_(out, non_blocking=True)
         event = torch.cuda.Event()
         event.record(torch.cuda.current_stream(self.device))
