@@ -58,6 +58,8 @@ struct AttnArgs {
   int splits;
   int page_shift;         // log2(page_size) if it is a power of two, else -1
   int n_seqs, max_tiles;  // prefill (bfloat16 kernel): sequences of the launch, 128-row tiles of the longest
+  int kv_chunk, max_chunks;  // prefill (bfloat16 kernel): keys per workgroup (a multiple of 32) and the most
+                             // chunks a tile can have; max_chunks == 1: a tile's keys are never split
 };
 
 // Per-wave online-softmax state for one 16-row tile. Lane (r, g) belongs to row r.
@@ -645,6 +647,8 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     rank = r * 8 + xcd;
     if (rank >= total) rank = b;                                 // (uneven XCD shares: keep every tile covered)
   }
+  const int chunk = rank % a.max_chunks;
+  rank /= a.max_chunks;
   const int per_tile = a.kv_heads * a.n_seqs;
   const int tile_from_end = rank / per_tile, sub = rank % per_tile;
   const int kvh = sub % a.kv_heads;
@@ -697,7 +701,13 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const int t_min = first_pos + wg_row0 / G;
   const int t_max = first_pos + min(rows - 1, wg_row0 + 127) / G;
   const int lo = a.window > 0 ? max(0, t_min - a.window + 1) : 0;       // keys below are never loaded
-  const int blk_begin = lo / 32, blk_end = t_max / 32 + 1;
+  // The tile's key blocks, and the share of them this workgroup takes. A tile split into several
+  // chunks leaves float32 partial results (running maximum, sum, output) that a second kernel merges.
+  const int tile_begin = lo / 32, tile_end = t_max / 32 + 1;
+  const int chunk_blocks = a.max_chunks > 1 ? a.kv_chunk / 32 : tile_end - tile_begin;
+  const int n_chunks = (tile_end - tile_begin + chunk_blocks - 1) / chunk_blocks;
+  if (chunk >= n_chunks) return;
+  const int blk_begin = tile_begin + chunk * chunk_blocks, blk_end = min(tile_end, blk_begin + chunk_blocks);
   const int wave_t_max = first_pos + min(rows - 1, wg_row0 + wave * 32 + 31) / G;
   const int wave_t_min = first_pos + min(rows - 1, wg_row0 + wave * 32) / G;
   const bool wave_live = wg_row0 + wave * 32 < rows;
@@ -888,6 +898,24 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   }
   compute_if_seen(blk, (blk - blk_begin) & 1);                // the last block (blk_end > blk_begin always)
 
+  if (n_chunks > 1) {
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+      if (!row_ok[rt]) continue;
+      const size_t slot = ((size_t)(token0 + tok[rt]) * a.q_heads + head[rt]) * a.max_chunks + chunk;
+      float* dst = a.part_o + slot * D;
+#pragma unroll
+      for (int dt = 0; dt < DTMAX; ++dt)
+        if (dt < dts)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = acc[rt][dt][j];
+      if (g == 0) {
+        a.part_ml[slot * 2] = m[rt];                              // in the scaled log2 domain
+        a.part_ml[slot * 2 + 1] = l[rt];
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
     if (!row_ok[rt]) continue;
@@ -901,13 +929,89 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   }
 }
 
+// Merge of the chunks of split tiles: grid = (8-row slices of the longest sequence's rows, kv_heads,
+// n_seqs); a thread takes 4 output dims of one row, with the prefill kernel's own arithmetic for
+// the key blocks of the row's tile. Chunks are added in index order.
+#define TW_MERGE_ROWS 8          /* rows per workgroup: 32 threads each */
+__global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnArgs a) {
+  const int G = a.q_heads / a.kv_heads;
+  const int kvh = blockIdx.y, seq = a.seq0 + blockIdx.z;
+  const int kv_len = a.kv_len[seq];
+  const int token0 = a.q_start[seq];
+  const int q_len = a.q_start[seq + 1] - token0;
+  const int rows = q_len * G;
+  const int D = a.head_dim, groups = D / 4;                      // groups of 4 output dims per row
+  const int item = threadIdx.x;                                  // 32 threads per row
+  const int row = blockIdx.x * TW_MERGE_ROWS + (item >> 5);
+  if (row >= rows) return;
+  const int wg_row0 = row / 128 * 128;
+  const int first_pos = kv_len - q_len;
+  const int t_min = first_pos + wg_row0 / G;
+  const int t_max = first_pos + min(rows - 1, wg_row0 + 127) / G;
+  const int lo = a.window > 0 ? max(0, t_min - a.window + 1) : 0;
+  const int tile_begin = lo / 32, tile_end = t_max / 32 + 1;
+  const int chunk_blocks = a.kv_chunk / 32;
+  const int n_chunks = (tile_end - tile_begin + chunk_blocks - 1) / chunk_blocks;
+  if (n_chunks <= 1) return;                                     // the prefill kernel wrote the result itself
+  const int tok = row / G, head = kvh * G + row % G;
+  const size_t slot0 = ((size_t)(token0 + tok) * a.q_heads + head) * a.max_chunks;
+  float m_all = -INFINITY;
+  for (int c = 0; c < n_chunks; ++c) m_all = fmaxf(m_all, a.part_ml[(slot0 + c) * 2]);
+  const float m_use = m_all == -INFINITY ? 0.f : m_all;
+  for (int grp = item & 31; grp < groups; grp += 32) {
+    float l_all = 0.f;
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int c = 0; c < n_chunks; ++c) {
+      const float w = __builtin_amdgcn_exp2f(a.part_ml[(slot0 + c) * 2] - m_use);
+      l_all += a.part_ml[(slot0 + c) * 2 + 1] * w;
+      const f32x4 x = *reinterpret_cast<const f32x4*>(a.part_o + (slot0 + c) * D + grp * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] += x[e] * w;
+    }
+    const float inv = l_all > 0.f ? 1.f / l_all : 0.f;
+    bf16_t packed[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) packed[e] = (bf16_t)(o[e] * inv);
+    bf16_t* dst = (bf16_t*)a.out + (size_t)(token0 + tok) * a.ldo + (size_t)head * D + grp * 4;
+    *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(packed);
+  }
+}
+
+// How the keys of a prefill tile are split over workgroups: returns the most chunks a tile can
+// have (1: no splitting) and the keys per chunk. With fewer tiles than the chip has room for,
+// long tiles are cut so that there are about a thousand units of work of similar size.
+static int tw_prefill_split_below = 256;     // one tile per CU or more: tiles are left whole
+extern "C" void tw_attn_prefill_split_below(int tiles) { tw_prefill_split_below = tiles; }   // (for experiments)
+
+extern "C" int tw_attn_prefill_split(int n_seqs, int q_heads, int kv_heads, int max_q_len, int max_kv_len,
+                                     int* kv_chunk) {
+  const int split_below = tw_prefill_split_below;
+  const int G = kv_heads > 0 ? q_heads / kv_heads : 1;
+  const long tiles = (long)tw_div_up((long)max_q_len * G, 128) * kv_heads * n_seqs;
+  *kv_chunk = 0;
+  if (tiles <= 0 || tiles >= split_below || max_kv_len <= 512) return 1;
+  int want = (int)tw_div_up(1024, tiles);
+  if (want > 8) want = 8;
+  int chunk = (int)tw_div_up(tw_div_up(max_kv_len, want), 32) * 32;
+  if (chunk < 256) chunk = 256;
+  const int chunks = (int)tw_div_up(max_kv_len + 31, chunk) + 1;     // a tile's first block may start mid-chunk
+  if (chunks <= 1) return 1;
+  *kv_chunk = chunk;
+  return chunks;
+}
+
+extern "C" long tw_attn_prefill_workspace_floats(int n_tokens, int q_heads, int head_dim, int max_chunks) {
+  return max_chunks > 1 ? (long)n_tokens * q_heads * max_chunks * (head_dim + 2) : 0;
+}
+
 template <int DTMAX>
 static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
   const int G = a.q_heads / a.kv_heads;
   const long rows = (long)max_q_len * G;
   a.n_seqs = n_seqs;
   a.max_tiles = (int)tw_div_up(rows, 128);
-  const long total = (long)a.max_tiles * a.kv_heads * n_seqs;
+  const long total = (long)a.max_tiles * a.kv_heads * n_seqs * a.max_chunks;
   TW_REQUIRE(total < (1L << 30));
   dim3 grid((unsigned)total);
   const size_t lds_bytes = 2 * 32 * (DTMAX * 32 + 16) + 2 * DTMAX * 16 * TW_PF_VROW;
@@ -919,6 +1023,9 @@ static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_
     attribute_set = true;
   }
   kernel<<<grid, 256, lds_bytes, stream>>>(a);
+  int err = TW_LAUNCH_RESULT();
+  if (err || a.max_chunks <= 1) return err;
+  attn_prefill_merge_kernel<<<dim3((unsigned)tw_div_up(rows, TW_MERGE_ROWS), a.kv_heads, n_seqs), 256, 0, stream>>>(a);
   return TW_LAUNCH_RESULT();
 }
 
@@ -1037,7 +1144,8 @@ static int prefill_launch(AttnArgs a, int n_seqs, int max_q_len, int generic, hi
 extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* keys, const void* values,
                                const int* block_table, int table_stride, const int* q_start,
                                const int* kv_len, int seq0, int n_seqs, int max_q_len, void* out,
-                               long ldo, int q_heads, int kv_heads, int head_dim, int page_size,
+                               long ldo, float* workspace, long workspace_floats, int n_tokens, int max_chunks,
+                               int kv_chunk, int q_heads, int kv_heads, int head_dim, int page_size,
                                int window, float scale, int generic, hipStream_t stream) {
   AttnArgs a;
   a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
@@ -1045,6 +1153,7 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = 1;
   a.part_o = nullptr; a.part_ml = nullptr;
+  a.max_chunks = 1; a.kv_chunk = 0;
   a.page_shift = -1;
   for (int sh = 0; sh < 20; ++sh)
     if ((1 << sh) == page_size) a.page_shift = sh;
@@ -1052,6 +1161,16 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
   if (err) return err;
   TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && max_q_len >= 1 && n_seqs <= 65535);
   if (n_seqs == 0) return 0;
+  // Splitting the keys of a tile (bfloat16 kernel only): partial results of token row n, head h, chunk c
+  // at workspace[((n * q_heads + h) * max_chunks + c) * head_dim], their (maximum, sum) pairs behind them.
+  if (max_chunks > 1 && workspace != nullptr) {
+    TW_REQUIRE(kv_chunk >= 32 && kv_chunk % 32 == 0 && n_tokens >= 1);
+    TW_REQUIRE(workspace_floats >= tw_attn_prefill_workspace_floats(n_tokens, q_heads, head_dim, max_chunks));
+    TW_REQUIRE((uintptr_t)workspace % 16 == 0 && (uintptr_t)out % 16 == 0 && ldo % 8 == 0);
+    a.max_chunks = max_chunks; a.kv_chunk = kv_chunk;
+    a.part_o = workspace;
+    a.part_ml = workspace + (size_t)n_tokens * q_heads * max_chunks * head_dim;
+  }
   if (dtype == TW_DTYPE_F32) return prefill_launch<float>(a, n_seqs, max_q_len, generic, stream);
   if (dtype == TW_DTYPE_BF16) return prefill_launch<bf16_t>(a, n_seqs, max_q_len, generic, stream);
   return TW_ERR_BAD_ARGUMENT;

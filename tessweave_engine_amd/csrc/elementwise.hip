@@ -112,8 +112,17 @@ __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restri
   if (mine) {
     const f32x4 wv = *reinterpret_cast<const f32x4*>(w + h);
     T* dst = out + (size_t)o * hidden + h;
+    T packed[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) dst[e] = tw_from_float<T>(v[e] * scale * wv[e]);
+    for (int e = 0; e < 4; ++e) packed[e] = tw_from_float<T>(v[e] * scale * wv[e]);
+    if (sizeof(T) == 2 && ((uintptr_t)out % 8 == 0))
+      *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(packed);      // hidden % 4 == 0: aligned
+    else if (sizeof(T) == 4 && ((uintptr_t)out % 16 == 0))
+      *reinterpret_cast<f32x4*>(dst) = *reinterpret_cast<const f32x4*>(packed);
+    else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[e] = packed[e];
+    }
   }
 }
 
@@ -124,8 +133,8 @@ extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, co
   TW_REQUIRE(add == nullptr || (add_splits > 0 && (rows == nullptr || row_scratch != nullptr)));
   if (n_out == 0) return 0;
   if (out_dtype != TW_DTYPE_F32 && out_dtype != TW_DTYPE_BF16) return TW_ERR_BAD_ARGUMENT;
-  // few rows (decode): one group of 4 elements per thread, everything in registers
-  if (n_out <= 64 && hidden % 4 == 0 && hidden <= 4096 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+  // rows of up to 4096 elements: one group of 4 elements per thread, everything in registers
+  if (hidden % 4 == 0 && hidden <= 4096 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
       (add == nullptr || ((uintptr_t)add % 16 == 0 && add_stride % 4 == 0))) {
     const int threads = (hidden / 4 + 63) / 64 * 64;
     if (out_dtype == TW_DTYPE_F32)

@@ -81,9 +81,16 @@ class GroupedQueryAttention(Mixer):
                             self.q_heads, self.kv_heads, self.head_dim, self.scale, window=window,
                             splits=splits, workspace=ws)
         if ctx.n_seqs > ctx.n_decode:
+            # long key ranges are cut into chunks for separate workgroups when there are few tiles of rows
+            longest = min(ctx.max_kv_len, window + ctx.max_q_len) if window else ctx.max_kv_len
+            split = ops.attn_prefill_split(ctx.n_seqs - ctx.n_decode, self.q_heads, self.kv_heads, ctx.max_q_len, longest)
+            ws = None
+            if split[0] > 1:
+                ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(
+                    n, self.q_heads, self.head_dim, split[0]),), torch.float32)
             ops.attn_prefill(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode,
                              ctx.n_seqs - ctx.n_decode, ctx.max_q_len, out, self.q_heads, self.kv_heads,
-                             self.head_dim, self.scale, window=window)
+                             self.head_dim, self.scale, window=window, split=split, workspace=ws)
         if not self.o.biases and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # the next norm adds them into x
         self.o.forward(ctx, out, x, residual=x)

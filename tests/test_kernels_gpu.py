@@ -350,11 +350,16 @@ def test_attn_prefill_portions(ops, device, dtype, heads, kv_heads, head_dim, pa
     # q lives inside a wider qkv buffer
     buf = torch.zeros(total_q, (heads + 2 * kv_heads) * head_dim, dtype=dtype, device=device)
     buf[:, :heads * head_dim] = q.reshape(total_q, -1).to(device)
-    for generic in (False, True):
+    # also with every tile's keys cut into chunks of 32 or 64 for separate workgroups (fast kernel only)
+    for generic, chunk in ((False, 0), (True, 0), (False, 32), (False, 64)):
         out = torch.full((total_q, heads * head_dim), float("nan"), dtype=dtype, device=device)
+        split = (math.ceil((max(lengths) + 31) / chunk) + 1, chunk) if chunk else None
+        ws = torch.full((ops.attn_prefill_workspace_floats(total_q, heads, head_dim, split[0]),), float("nan"),
+                        device=device) if chunk else None
         ops.attn_prefill(buf, keys, values, table, torch.tensor(q_start, dtype=torch.int32, device=device),
                          torch.tensor(lengths, dtype=torch.int32, device=device), 0, len(cases), max(c[1] for c in cases),
-                         out, heads, kv_heads, head_dim, head_dim ** -0.5, window=window, generic=generic)
+                         out, heads, kv_heads, head_dim, head_dim ** -0.5, window=window, generic=generic,
+                         split=split, workspace=ws)
         torch.testing.assert_close(out.float().cpu().reshape(total_q, heads, head_dim), want, **ATTN_TOL[dtype])
     # the decode kernel on the one-token sequence must agree with the prefill kernel
     s = len(cases) - 1
@@ -424,10 +429,13 @@ def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
     q = q_one[None].expand(q_len, heads, d).contiguous()
     want = plain.attention(q.float(), k, v, torch.arange(n - q_len, n), window=window or None)
     q_start = torch.tensor([0, q_len], dtype=torch.int32, device=device)
-    for generic in (False, True):
+    for generic, chunk in ((False, 0), (True, 0), (False, 32), (False, 96)):
         out = torch.full((q_len, heads * d), float("nan"), dtype=dtype, device=device)
+        split = (math.ceil((n + 31) / chunk) + 1, chunk) if chunk else None
+        ws = torch.full((ops.attn_prefill_workspace_floats(q_len, heads, d, split[0]),), float("nan"),
+                        device=device) if chunk else None
         ops.attn_prefill(q.reshape(q_len, -1).to(device), keys, values, table, q_start, kv_len, 0, 1, q_len, out, heads, 1,
-                         d, d ** -0.5, window=window, generic=generic)
+                         d, d ** -0.5, window=window, generic=generic, split=split, workspace=ws)
         torch.testing.assert_close(out.float().cpu().reshape(q_len, heads, d), want, **ATTN_TOL[dtype])
 
 
