@@ -27,6 +27,7 @@ class EngineConfig:
     adaptive_chunk: bool = False    # flow_engine/engine.py:262-268 feedback controller
     use_graphs: bool = True         # replay decode-only steps from HIP graphs
     lookahead: bool = True          # put a turn on the device before the tokens of the turn before are read
+    tile_rows: int = 128            # rows of a matrix-kernel tile: prompt portions make room for decode tokens (0: never)
 
     def __post_init__(self):
         for key in ("block_size", "kv_blocks", "max_context", "max_active", "max_queue",

@@ -186,6 +186,15 @@ class Engine:
                     break
                 portions.append(Portion(r, count, count == remaining, True))
                 budget -= count
+            # The matrix kernels work on tiles of 128 rows: a step of 256 prompt tokens and 8 decode
+            # tokens would pay for 384. If the decode tokens alone push the step past a multiple of the
+            # tile, the last portion gives up that many tokens (unless it completes its prompt).
+            tile = self.config.tile_rows
+            last = portions[-1]
+            if tile and last.prompt and not last.samples:
+                excess = (len(decode) + sum(p.count for p in portions if p.prompt)) % tile
+                if 0 < excess <= len(decode) and last.count - excess >= self.config.min_prefill_chunk:
+                    last.count -= excess
         return portions
 
     def step(self):

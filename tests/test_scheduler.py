@@ -438,3 +438,35 @@ def test_lookahead_with_cancel_failure_and_prefix_reuse():
     e.cache.check()
     e.close()
     assert len(e.cache.pools[0].free) == 32
+
+
+def test_a_prompt_portion_makes_room_for_decode_tokens_up_to_a_tile_of_rows():
+    global CFG
+    small, CFG = CFG, dict(CFG, max_position_embeddings=1024)
+    try:
+        _portion_and_tile_rows()
+    finally:
+        CFG = small
+
+
+def _portion_and_tile_rows():
+    e, s = make(kv_blocks=256, max_context=1024, prefill_chunk=256, min_prefill_chunk=16, max_active=4)
+    short = [e.submit([1, 2, 3], 40) for _ in range(2)]
+    e.step()                                                            # both short prompts complete, first tokens
+    long = e.submit(list(range(100)) * 7, 4)                            # 700 tokens
+    e.step()
+    assert [(n, w) for _, _, n, w in s.batches[-1]] == [(1, [0]), (1, [0]), (254, [])]      # 2 + 254 = 256 rows, not 258
+    e.step()
+    assert [n for _, _, n, _ in s.batches[-1]] == [1, 1, 254]
+    e.step()                                                            # 192 left: completes the prompt, never shortened
+    assert [(n, w) for _, _, n, w in s.batches[-1]] == [(1, [0]), (1, [0]), (192, [191])]
+    drain(e)
+    assert long.output == expected(long.prompt, 4) and all(r.output == expected([1, 2, 3], 40) for r in short)
+    e.close()
+    e, s = make(kv_blocks=256, max_context=1024, prefill_chunk=256, min_prefill_chunk=16, max_active=4, tile_rows=0)
+    a = e.submit([1, 2, 3], 40)
+    e.step()
+    e.submit(list(range(100)) * 7, 4)
+    e.step()
+    assert [n for _, _, n, _ in s.batches[-1]] == [1, 256]
+    e.close()
