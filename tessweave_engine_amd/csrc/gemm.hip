@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
                                                          const float* __restrict__ bias,
                                                          const float* residual, long ldr, OutT* C,
                                                          long ldc, int M, int N, int K, int tiles_m,
-                                                         int n_blocks) {
+                                                         int n_blocks, int splits, float* __restrict__ partial) {
   typedef typename Elem<T>::Frag Frag;
   constexpr int EPF = Elem<T>::kPerFrag;
   constexpr int KCH = 8;                                    // 16-byte chunks of K per row and stage
@@ -167,7 +167,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
   const int per_xcd = gridDim.x / 8;
   const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
   if (logical >= n_blocks) return;
-  const int tile_m = logical % tiles_m, tile_n = logical / tiles_m;
+  // splits > 1 (few tiles, long K): the k-tiles are dealt to `splits` workgroups per tile, which
+  // leave float32 partial sums partial[split][M][N] for splitk_reduce_kernel.
+  const int n_tiles = n_blocks / splits;
+  const int split = logical / n_tiles, tile = logical % n_tiles;
+  const int tile_m = tile % tiles_m, tile_n = tile / tiles_m;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -225,7 +229,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
   // Two register sets: the global loads of k-tile kt+2 are issued while k-tile kt is multiplied,
   // so two k-tiles per workgroup are on their way from memory at any time.
   Frag a_regs[2][A_LOADS], w_regs[2][W_LOADS];
-  const int k_tiles = (K + BK - 1) / BK;
+  const int k_tiles_all = (K + BK - 1) / BK;
+  const int per_split = (k_tiles_all + splits - 1) / splits;
+  const int kt0 = split * per_split;                          // this workgroup's k-tiles: kt0 .. kt0 + k_tiles - 1
+  const int k_tiles = max(0, min(k_tiles_all, kt0 + per_split) - kt0);
   const int whole_tiles = K / BK;
 
   // whole k-tiles need no predicate at all; the main loop below runs only those
@@ -287,36 +294,44 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
     }
   };
 
-  load_global(0, a_regs[0], w_regs[0]);
-  if (k_tiles > 1) load_global(1, a_regs[1], w_regs[1]);
-  store_lds(0, a_regs[0], w_regs[0]);
+  if (k_tiles > 0) {
+    load_global(kt0, a_regs[0], w_regs[0]);
+    if (k_tiles > 1) load_global(kt0 + 1, a_regs[1], w_regs[1]);
+    store_lds(0, a_regs[0], w_regs[0]);
+  }
   __syncthreads();
-  int kt = 0;
+  int j = 0;                                                  // k-tile kt0 + j is in LDS stage j & 1
   // Main loop: two k-tiles per round, every load whole and unconditional, so that the register
   // sets are plain loop-carried values (conditional loads cost a register copy per loaded dword).
-  for (; kt + 3 < whole_tiles; kt += 2) {
-    load_whole(kt + 2, a_regs[0], w_regs[0]);               // LDS stage 0, register set 0 is free
+  const int whole_here = min(k_tiles, whole_tiles - kt0);
+  for (; j + 3 < whole_here; j += 2) {
+    load_whole(kt0 + j + 2, a_regs[0], w_regs[0]);           // LDS stage 0, register set 0 is free
     multiply(0);
     store_lds(1, a_regs[1], w_regs[1]);
     __syncthreads();
-    load_whole(kt + 3, a_regs[1], w_regs[1]);               // LDS stage 1, register set 1 is free
+    load_whole(kt0 + j + 3, a_regs[1], w_regs[1]);           // LDS stage 1, register set 1 is free
     multiply(1);
     store_lds(0, a_regs[0], w_regs[0]);
     __syncthreads();
   }
-  // The last few k-tiles (kt is even here): the same rounds with every step conditional.
-  for (; kt < k_tiles; kt += 2) {
-    if (kt + 2 < k_tiles) load_global(kt + 2, a_regs[0], w_regs[0]);
+  // The last few k-tiles (j is even here): the same rounds with every step conditional.
+  for (; j < k_tiles; j += 2) {
+    if (j + 2 < k_tiles) load_global(kt0 + j + 2, a_regs[0], w_regs[0]);
     multiply(0);
-    if (kt + 1 < k_tiles) store_lds(1, a_regs[1], w_regs[1]);
+    if (j + 1 < k_tiles) store_lds(1, a_regs[1], w_regs[1]);
     __syncthreads();
-    if (kt + 1 >= k_tiles) break;
-    if (kt + 3 < k_tiles) load_global(kt + 3, a_regs[1], w_regs[1]);
+    if (j + 1 >= k_tiles) break;
+    if (j + 3 < k_tiles) load_global(kt0 + j + 3, a_regs[1], w_regs[1]);
     multiply(1);
-    if (kt + 2 < k_tiles) store_lds(0, a_regs[0], w_regs[0]);
+    if (j + 2 < k_tiles) store_lds(0, a_regs[0], w_regs[0]);
     __syncthreads();
   }
 
+  if (splits > 1) {
+    tw_tiled_epilogue<float, WM, WN, false>(acc, lds, nullptr, nullptr, 0, partial + (size_t)split * M * N, (long)N,
+                                            M, N, m0, n0, wm0, wn0, wave, lane);
+    return;
+  }
   tw_tiled_epilogue<OutT, WM, WN, GLU>(acc, lds, bias, residual, ldr, C, ldc, M, N, m0, n0, wm0, wn0, wave, lane);
 }
 
@@ -554,14 +569,29 @@ __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* 
 // =====================================================================================
 // Host side
 // =====================================================================================
+// How many K ranges the tiled kernel uses: with fewer tiles than the chip has room for (a prompt
+// portion of a few hundred rows against a square or tall matrix) the k-tiles of a tile are dealt
+// to several workgroups. Depends on the shape only.
+static int tiled_splits(int M, int N, int K, int epf, int bm, int bn) {
+  const long tiles = (long)tw_div_up(M, bm) * tw_div_up(N, bn);
+  if (tiles >= 192) return 1;
+  const int k_tiles = tw_div_up(K, 8 * epf);
+  long splits = tw_div_up(384, tiles);
+  if (splits > k_tiles / 8) splits = k_tiles / 8;
+  if (splits > 8) splits = 8;
+  return splits < 1 ? 1 : (int)splits;
+}
+
 template <typename T, typename OutT, int WM, int WN, bool SHUF, bool GLU>
 static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
-                        const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
-                        hipStream_t stream) {
+                        const float* residual, long ldr, OutT* C, long ldc, float* partial,
+                        long partial_bytes, int M, int N, int K, hipStream_t stream) {
   constexpr int BM = 64 * WM, BN = 64 * WN, KCH = 8;
   constexpr int EPF = Elem<T>::kPerFrag;
   const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
-  const long n_blocks = (long)tiles_m * tiles_n;
+  int splits = GLU ? 1 : tiled_splits(M, N, K, EPF, BM, BN);
+  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4 || (uintptr_t)partial % 16 != 0)) splits = 1;
+  const long n_blocks = (long)tiles_m * tiles_n * splits;
   TW_REQUIRE(n_blocks < (1L << 30));
   // per-tile offsets are 32-bit
   TW_REQUIRE((long)BM * lda < (1L << 31));
@@ -579,7 +609,11 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
     attribute_set = true;
   }
   kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m,
-                                           (int)n_blocks);
+                                           (int)n_blocks, splits, partial);
+  int err = TW_LAUNCH_RESULT();
+  if (err || splits == 1) return err;
+  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
+                                                                             ldr, C, ldc, M, N);
   return TW_LAUNCH_RESULT();
 }
 
@@ -596,12 +630,19 @@ static int skinny_lds_splits(int N, int K, int epf) {
   return splits < 1 ? 1 : splits;
 }
 
+// Bytes of split-K scratch tw_linear can use for up to max_rows rows (0: none needed).
 extern "C" long tw_linear_workspace_bytes(int dtype, int max_rows, int N, int K) {
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
   if (K % epf) return 0;
   const int rows = max_rows < 64 ? max_rows : 64;
-  const int splits = skinny_lds_splits(N, K, epf);
-  return splits > 1 ? (long)splits * rows * N * 4 : 0;
+  int splits = skinny_lds_splits(N, K, epf);
+  long bytes = splits > 1 ? (long)splits * rows * N * 4 : 0;
+  if (max_rows > 64) {
+    splits = tiled_splits(max_rows, N, K, epf, 128, 128);
+    const long tiled = splits > 1 ? (long)splits * max_rows * N * 4 : 0;
+    if (tiled > bytes) bytes = tiled;
+  }
+  return bytes;
 }
 
 template <typename T, typename OutT, int MT, bool PARTIAL, bool SHUF, bool GLU>
@@ -659,8 +700,8 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
     return launch_skinny_lds_m<T, OutT, false, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
   if (force == 4)
-    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
-  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
+    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
 }
 
 template <typename T, typename OutT>

@@ -140,6 +140,7 @@ def test_silu_mul(ops, device, dtype):
 LINEAR_SHAPES = [  # m, n, k
     (1, 16, 64), (3, 389, 320), (8, 1000, 1032), (16, 48, 4096), (17, 130, 192), (33, 64, 8200),
     (64, 256, 512), (65, 200, 136), (130, 389, 64), (300, 520, 776),
+    (130, 96, 4096), (257, 260, 2056),      # few tiles, long K: the tiled kernel splits K as well
 ]
 
 
