@@ -981,12 +981,9 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnArgs a) {
 // How the keys of a prefill tile are split over workgroups: returns the most chunks a tile can
 // have (1: no splitting) and the keys per chunk. With fewer tiles than the chip has room for,
 // long tiles are cut so that there are about a thousand units of work of similar size.
-static int tw_prefill_split_below = 256;     // one tile per CU or more: tiles are left whole
-extern "C" void tw_attn_prefill_split_below(int tiles) { tw_prefill_split_below = tiles; }   // (for experiments)
-
 extern "C" int tw_attn_prefill_split(int n_seqs, int q_heads, int kv_heads, int max_q_len, int max_kv_len,
                                      int* kv_chunk) {
-  const int split_below = tw_prefill_split_below;
+  const int split_below = 256;                     // one tile per CU or more: tiles are left whole (measured)
   const int G = kv_heads > 0 ? q_heads / kv_heads : 1;
   const long tiles = (long)tw_div_up((long)max_q_len * G, 128) * kv_heads * n_seqs;
   *kv_chunk = 0;

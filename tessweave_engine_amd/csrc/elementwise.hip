@@ -182,29 +182,16 @@ extern "C" int tw_rope_table(const int* positions, const float* inv_freq, float*
 //   keys  [page][kv_head][offset][d]      and raw v to
 //   values[page][kv_head][d][offset]      (transposed inside the page),
 // slot = page * page_size + offset; a negative slot writes nothing.
-// If `partial` is given, the row's values are first formed as
-// round_T(sum_s partial[s][n][col] + bias[col]) (the split-K sums of the q/k/v
-// projection) and q, k, v are all written to qkv before anything else happens.
+// (With `partial`, the split-K sums of the q/k/v projection, qkv_finish_kernel below does the
+// same from round_T(sum_s partial[s][n][col] + bias[col]), one workgroup per (token, head).)
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* __restrict__ cos_t,
                                      const float* __restrict__ sin_t, const int* __restrict__ slots,
                                      T* __restrict__ keys, T* __restrict__ values, int q_heads,
-                                     int kv_heads, int head_dim, int rot, int page_size, int write_cache,
-                                     const float* __restrict__ partial, int splits, size_t split_stride,
-                                     const float* __restrict__ bias) {
+                                     int kv_heads, int head_dim, int rot, int page_size, int write_cache) {
   const int n = blockIdx.x;
   const int half = rot / 2;
   T* row = qkv + (size_t)n * ld;
-  if (partial) {
-    const int width = (q_heads + 2 * kv_heads) * head_dim;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) {
-      float v = 0.f;
-      for (int s = 0; s < splits; ++s) v += partial[s * split_stride + (size_t)n * width + c];
-      if (bias) v += bias[c];
-      row[c] = tw_from_float<T>(v);
-    }
-    __syncthreads();
-  }
   const float* c = cos_t + (size_t)n * half;
   const float* s = sin_t + (size_t)n * half;
   const int slot = write_cache ? slots[n] : -1;
@@ -300,7 +287,8 @@ extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_
   TW_REQUIRE(ld >= (long)(q_heads + 2 * kv_heads) * head_dim);
   TW_REQUIRE(!write_cache || (slots && keys && values));
   if (n == 0) return 0;
-  if (partial && n <= 65535) {
+  if (partial) {
+    TW_REQUIRE(n <= 65535);
     dim3 grid(q_heads + 2 * kv_heads, n);
     const int threads = head_dim / 2 <= 64 ? 64 : 128;
     if (dtype == TW_DTYPE_F32)
@@ -318,12 +306,11 @@ extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_
   if (dtype == TW_DTYPE_F32)
     rope_kv_write_kernel<float><<<n, 256, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
                                                        (float*)values, q_heads, kv_heads, head_dim, rot,
-                                                       page_size, write_cache, partial, splits, split_stride, bias);
+                                                       page_size, write_cache);
   else if (dtype == TW_DTYPE_BF16)
     rope_kv_write_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots,
                                                         (bf16_t*)keys, (bf16_t*)values, q_heads, kv_heads,
-                                                        head_dim, rot, page_size, write_cache, partial, splits,
-                                                        split_stride, bias);
+                                                        head_dim, rot, page_size, write_cache);
   else
     return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
