@@ -13,7 +13,7 @@ from tiny_configs import TINY, make_folder
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "C"])
 def tiny(request, tmp_path_factory, device):
     name = request.param
     folder = tmp_path_factory.mktemp(f"eng{name}")

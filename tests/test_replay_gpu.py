@@ -24,14 +24,14 @@ from tiny_configs import TINY, make_folder
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
 
-LENGTHS = {"A": [37, 49, 70, 33, 64, 40], "B": [33, 41, 64, 100, 124, 35, 50]}
+LENGTHS = {"A": [37, 49, 70, 33, 64, 40], "B": [33, 41, 64, 100, 124, 35, 50], "C": [36, 65, 97, 130, 34, 48]}
 
 
 def round64(n):
     return (n + 63) // 64 * 64
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "C"])
 def tiny(request, tmp_path_factory, device):
     name = request.param
     folder = tmp_path_factory.mktemp(f"tiny{name}")

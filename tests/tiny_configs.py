@@ -1,4 +1,6 @@
-"""Two tiny configurations of the architecture that differ in every size and option."""
+"""Tiny configurations of the architecture that differ in every size and option. A and B have small
+heads (16, 32); C has the head size of the real checkpoints (128), whose kernels are separate
+instantiations, two query heads per kv head, and pages of 32."""
 
 TINY_A = dict(
     architectures=["Qwen2ForCausalLM"], model_type="qwen2",
@@ -14,7 +16,15 @@ TINY_B = dict(
     tie_word_embeddings=False, use_sliding_window=False, max_position_embeddings=1024, hidden_act="silu")
 TINY_B_PAGE, TINY_B_SEED = 8, 1
 
-TINY = {"A": (TINY_A, TINY_A_PAGE, TINY_A_SEED), "B": (TINY_B, TINY_B_PAGE, TINY_B_SEED)}
+TINY_C = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2",
+    num_hidden_layers=2, hidden_size=256, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+    intermediate_size=336, vocab_size=300, rope_theta=5e5, rms_norm_eps=1e-6,
+    tie_word_embeddings=False, use_sliding_window=False, max_position_embeddings=1024, hidden_act="silu")
+TINY_C_PAGE, TINY_C_SEED = 32, 2
+
+TINY = {"A": (TINY_A, TINY_A_PAGE, TINY_A_SEED), "B": (TINY_B, TINY_B_PAGE, TINY_B_SEED),
+        "C": (TINY_C, TINY_C_PAGE, TINY_C_SEED)}
 
 
 def make_folder(path, name):
