@@ -612,7 +612,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 #define TW_PF_VROW 80                       /* LDS bytes per value row (32 keys = 64 B, padded) */
 
 
-template <int DTMAX>
+// EXACT: head_dim == 16 * DTMAX, so every loop over the head has compile-time bounds (with run-time
+// bounds the compiler indexes the accumulators dynamically, several instructions per MFMA).
+template <int DTMAX, bool EXACT>
 __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
   constexpr int KROW = DTMAX * 32 + 16;                 // LDS bytes per key row, padded
@@ -662,14 +664,14 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   if (tile_idx < 0 || tile_idx >= n_tiles) return;
   const int wg_row0 = tile_idx * 128;
   const int* table = a.block_table + (size_t)seq * a.table_stride;
-  const int D = a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
+  const int D = EXACT ? DTMAX * 16 : a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
   const int pshift = a.page_shift, pmask = P - 1;
   const int ppb = P >= 32 ? 1 : (32 >> pshift);
   const unsigned head_stride = (unsigned)P * D;
   const bf16_t* keys = (const bf16_t*)a.keys;
   const bf16_t* values = (const bf16_t*)a.values;
   const int first_pos = kv_len - q_len;
-  const bool whole_chunks = (chunks & 3) == 0;           // head_dim a multiple of 32: no partial MFMA step
+  const bool whole_chunks = EXACT || (chunks & 3) == 0;  // head_dim a multiple of 32: no partial MFMA step
   const float c2 = a.scale * 1.44269504088896340736f;    // scores are kept in the log2 domain
 
   // ---- this wave's two row tiles -----------------------------------------------
@@ -687,7 +689,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
 #pragma unroll
     for (int st = 0; st < NSMAX; ++st) {
       const int chunk = st * 4 + g;
-      qf[rt][st] = (row_ok[rt] && chunk < chunks) ? tw_load_frag(q_row + chunk * 8) : Elem<bf16_t>::zero();
+      qf[rt][st] = (row_ok[rt] && (EXACT || chunk < chunks)) ? tw_load_frag(q_row + chunk * 8) : Elem<bf16_t>::zero();
     }
   }
   f32x4 acc[2][DTMAX];
@@ -817,7 +819,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       const char* base = k_frag[tile] + buf * KSTAGE;
 #pragma unroll
       for (int st = 0; st < NSMAX; ++st)
-        if (st * 4 < chunks) {
+        if (EXACT || st * 4 < chunks) {
           bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + st * 64);
           if (!whole_chunks && st * 4 + g >= chunks) kf = Elem<bf16_t>::zero();
           tw_mma16(s[0][tile], kf, qf[0][st]);
@@ -873,7 +875,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     const char* vbase = v_frag + buf * VSTAGE;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts) {
+      if (EXACT || dt < dts) {
         const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
         tw_mma16(acc[0][dt], vf, pb[0]);
         tw_mma16(acc[1][dt], vf, pb[1]);
@@ -906,7 +908,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       float* dst = a.part_o + slot * D;
 #pragma unroll
       for (int dt = 0; dt < DTMAX; ++dt)
-        if (dt < dts)
+        if (EXACT || dt < dts)
 #pragma unroll
           for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = acc[rt][dt][j];
       if (g == 0) {
@@ -923,7 +925,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     bf16_t* dst = (bf16_t*)a.out + (size_t)(token0 + tok[rt]) * a.ldo + (size_t)head[rt] * D;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (dt < dts)
+      if (EXACT || dt < dts)
 #pragma unroll
         for (int j = 0; j < 4; ++j) dst[dt * 16 + 4 * g + j] = (bf16_t)(acc[rt][dt][j] * inv);
   }
@@ -1002,7 +1004,7 @@ extern "C" long tw_attn_prefill_workspace_floats(int n_tokens, int q_heads, int 
   return max_chunks > 1 ? (long)n_tokens * q_heads * max_chunks * (head_dim + 2) : 0;
 }
 
-template <int DTMAX>
+template <int DTMAX, bool EXACT>
 static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_t stream) {
   const int G = a.q_heads / a.kv_heads;
   const long rows = (long)max_q_len * G;
@@ -1012,7 +1014,7 @@ static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_
   TW_REQUIRE(total < (1L << 30));
   dim3 grid((unsigned)total);
   const size_t lds_bytes = 2 * 32 * (DTMAX * 32 + 16) + 2 * DTMAX * 16 * TW_PF_VROW;
-  auto kernel = attn_prefill_bf16_kernel<DTMAX>;
+  auto kernel = attn_prefill_bf16_kernel<DTMAX, EXACT>;
   static bool attribute_set = false;
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
@@ -1121,9 +1123,11 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
 template <typename T>
 static int prefill_launch(AttnArgs a, int n_seqs, int max_q_len, int generic, hipStream_t stream) {
   if (IsBf16<T>::value && a.page_shift >= 3 && !generic) {
-    if (a.head_dim <= 64) return prefill_bf16_launch<4>(a, n_seqs, max_q_len, stream);
-    if (a.head_dim <= 128) return prefill_bf16_launch<8>(a, n_seqs, max_q_len, stream);
-    return prefill_bf16_launch<16>(a, n_seqs, max_q_len, stream);
+    if (a.head_dim == 64) return prefill_bf16_launch<4, true>(a, n_seqs, max_q_len, stream);
+    if (a.head_dim < 64) return prefill_bf16_launch<4, false>(a, n_seqs, max_q_len, stream);
+    if (a.head_dim == 128) return prefill_bf16_launch<8, true>(a, n_seqs, max_q_len, stream);
+    if (a.head_dim < 128) return prefill_bf16_launch<8, false>(a, n_seqs, max_q_len, stream);
+    return prefill_bf16_launch<16, false>(a, n_seqs, max_q_len, stream);
   }
   const int G = a.q_heads / a.kv_heads;
   const long rows = (long)max_q_len * G;
