@@ -470,3 +470,47 @@ def _portion_and_tile_rows():
     e.step()
     assert [n for _, _, n, _ in s.batches[-1]] == [1, 256]
     e.close()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_arrivals_cancellations_and_both_ways_of_reading(seed):
+    """Random prompts, budgets, arrival times and cancellations: with and without lookahead every request that
+    is not cancelled gets the toy model's tokens, and no page is lost, held twice or left behind."""
+    import random
+    rng = random.Random(seed)
+    plans = []
+    for i in range(14):
+        prompt = [rng.randrange(VOCAB) for _ in range(rng.choice([1, 2, 3, 5, 8, 13, 21, 30]))]
+        plans.append(dict(prompt=prompt, max_tokens=rng.choice([1, 2, 3, 6, 11]), at=rng.randrange(0, 25),
+                          cancel_at=rng.randrange(3, 40) if rng.random() < 0.25 else None,
+                          temperature=rng.choice([0.0, 0.0, 0.7])))
+    results = []
+    for look in (True, False):
+        make_engine = make_lookahead if look else make
+        e, s = make_engine(kv_blocks=24, max_active=3, prefill_chunk=rng.choice([2, 4, 7]), prefix_cache=bool(seed % 2),
+                           max_queue=32)
+        assert e.lookahead == look
+        live = {}
+        for turn in range(400):
+            for i, p in enumerate(plans):
+                if p["at"] == turn:
+                    live[i] = e.submit(p["prompt"], p["max_tokens"], temperature=p["temperature"], seed=i)
+                if p["cancel_at"] == turn and i in live:
+                    e.cancel(live[i].id)
+            busy = e.step()
+            e.cache.check()
+            if not busy and turn > 45:
+                break
+        assert not e.requests and e._inflight is None
+        out = {}
+        for i, r in live.items():
+            if r.status == "cancelled":
+                assert r.output == expected(plans[i]["prompt"], len(r.output))       # a prefix of the right tokens
+            else:
+                assert r.status == "length" and r.output == expected(plans[i]["prompt"], plans[i]["max_tokens"])
+            out[i] = (r.status, r.output if r.status != "cancelled" else None)
+        e.close()
+        assert len(e.cache.pools[0].free) == 24
+        results.append(out)
+    assert {i: v for i, v in results[0].items() if v[1] is not None and results[1][i][1] is not None} == \
+           {i: v for i, v in results[1].items() if v[1] is not None and results[0][i][1] is not None}
