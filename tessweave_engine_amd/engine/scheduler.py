@@ -211,6 +211,7 @@ class Engine:
             if self.lookahead:
                 feed = self.sampler.out_buffer
                 if getattr(self.stepper, "token_feed", None) is not feed:
+                    self.stepper.segment_graphs = False      # launches are hidden behind the step before
                     self.stepper.set_token_feed(feed)
             entries = []
             for p in portions:
@@ -229,7 +230,10 @@ class Engine:
             if not sampled:
                 self._inflight = None
             elif self.lookahead:
-                self._inflight = (self.sampler.sample_async(*arguments), [(p.request, i) for i, p in enumerate(sampled)])
+                # on the step's own stream: the sampling kernels follow the step without a wait between streams
+                with self._sampling_stream():
+                    pending = self.sampler.sample_async(*arguments)
+                self._inflight = (pending, [(p.request, i) for i, p in enumerate(sampled)])
             else:
                 ids = self.sampler.sample(*arguments)
                 self._inflight = (ids, [(p.request, i) for i, p in enumerate(sampled)])
@@ -252,6 +256,14 @@ class Engine:
             if self.config.adaptive_chunk and n_prompt:
                 self._adapt_chunk(elapsed, n_prompt)
             return True
+
+    def _sampling_stream(self):
+        stream = getattr(self.stepper, "stream", None)
+        if stream is None:
+            import contextlib
+            return contextlib.nullcontext()
+        import torch
+        return torch.cuda.stream(stream)
 
     def flush(self):
         """Read and commit the tokens of the last turn, if they are still unread (lookahead)."""

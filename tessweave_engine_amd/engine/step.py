@@ -62,6 +62,7 @@ class Stepper:
         self._graphs = {}
         self._warm = set()
         self.token_feed = None
+        self.segment_graphs = True
         self._staging = []
         self._staging_events = []
         self._staging_next = 0
@@ -283,10 +284,12 @@ class Stepper:
     def _capture(self, ctx):
         """Capture model.forward(ctx) as a chain of graphs.
 
-        Launching a graph costs host time per node before its first kernel starts. The step is
-        therefore cut after the first layer run and then every GRAPH_SEGMENT_RUNS runs: the
-        first graph is short and starts at once, and every later one is launched while its
-        predecessor still runs.
+        Launching a graph costs host time per node before its first kernel starts. With
+        `segment_graphs` the step is therefore cut after the first layer run and then every
+        GRAPH_SEGMENT_RUNS runs: the first graph is short and starts at once, and every later one
+        is launched while its predecessor still runs. A caller that launches a step while the step
+        before still runs (the scheduler's lookahead) turns it off: the launch is hidden anyway, and
+        every cut costs about 8 us between two graphs.
         """
         lib = library()
         stream = self.stream.cuda_stream
@@ -302,7 +305,7 @@ class Stepper:
             return code
 
         def segment_end(i):
-            if i + 1 < n_runs and (i == 0 or (i + 1) % GRAPH_SEGMENT_RUNS == 0):
+            if self.segment_graphs and i + 1 < n_runs and (i == 0 or (i + 1) % GRAPH_SEGMENT_RUNS == 0):
                 check(end_segment(), "graph capture end")
                 check(lib.tw_graph_begin(stream), "graph capture begin")
 
