@@ -140,6 +140,47 @@ def test_lookahead_and_reading_every_turn_give_the_same_tokens(tiny):
     assert outs[0][2] == (plain.greedy(tiny["config"], tiny["weights"], prompts[2], 5), "length")
 
 
+def test_many_requests_with_few_pages_give_the_same_tokens_with_and_without_lookahead(tiny):
+    """A few hundred turns of serving in 32-bit, where rounding cannot flip a choice: random prompt lengths,
+    temperatures, arrivals, cancellations and two EOS ids, with so few pages that requests wait for them and
+    prefix pages are evicted. The tokens of every request are the same in both modes, and no page is lost."""
+    import random
+    rng = random.Random(7)
+    vocab = tiny["cfg"]["vocab_size"]
+    plans = [dict(prompt=[rng.randrange(vocab) for _ in range(rng.choice([1, 3, 9, 31, 64, 100]))],
+                  max_tokens=rng.choice([1, 2, 7, 20, 40]), temperature=rng.choice([0.0, 0.0, 0.8, 1.5]),
+                  gap=rng.choice([0, 0, 1, 3]), cancel_after=rng.randrange(2, 30) if rng.random() < 0.1 else None)
+             for _ in range(150)]
+    pages = 2 * -(-(100 + 40 + 48) // tiny["page"]) + 3
+    outs = []
+    for look in (True, False):
+        e = engine(tiny, no_lookahead=not look, kv_blocks=pages, max_context=256, prefill_chunk=48, max_active=6,
+                   no_prefix_cache=False)
+        e.model_config = dataclasses.replace(e.model_config, eos_token_ids=(17, vocab - 2))
+        live, cancel, nxt, wait, turn = {}, {}, 0, 0, 0
+        while nxt < len(plans) or e.requests:
+            while nxt < len(plans) and wait <= 0 and len(e.waiting) < 8:
+                p = plans[nxt]
+                live[nxt] = e.submit(p["prompt"], p["max_tokens"], temperature=p["temperature"], seed=nxt)
+                if p["cancel_after"]:
+                    cancel[turn + p["cancel_after"]] = live[nxt].id
+                wait, nxt = p["gap"], nxt + 1
+            if turn in cancel:
+                e.cancel(cancel[turn])
+            e.step()
+            wait, turn = wait - 1, turn + 1
+            if turn % 64 == 0:
+                e.cache.check()
+            assert turn < 20000
+        e.flush()
+        e.cache.check()
+        outs.append({i: (r.status, tuple(r.output)) for i, r in live.items()})
+        e.close()
+    differ = [i for i in outs[0] if outs[0][i] != outs[1][i] and "cancelled" not in (outs[0][i][0], outs[1][i][0])]
+    assert not differ, [(outs[0][i], outs[1][i]) for i in differ[:3]]
+    assert sum(v[0] == "stop" for v in outs[0].values()) >= 1
+
+
 def test_prefix_pages_are_reused_on_the_gpu(tiny):
     page = tiny["page"]
     shared = prompts_for(tiny, [32], seed=4)[0]
