@@ -527,6 +527,17 @@ __global__ __launch_bounds__(TW_REDUCE_THREADS) void attn_decode_reduce_kernel(
   __shared__ float s_l;
   const int head = blockIdx.x, local = blockIdx.y, tid = threadIdx.x;
   const size_t slot0 = ((size_t)local * q_heads + head) * splits;
+  const int cols = TW_REDUCE_THREADS / head_dim > 0 ? TW_REDUCE_THREADS / head_dim : 1;   // head_dim <= 256
+  const int d = tid % head_dim, c = tid / head_dim;
+  // The first 8 partial outputs of this thread are on their way while the weights are formed
+  // (the kernel's time is a chain of memory latencies).
+  const int token = q_start[seq0 + local];
+  float po[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int sp = c + i * cols;
+    po[i] = (c < cols && sp < splits) ? part_o[(slot0 + sp) * head_dim + d] : 0.f;
+  }
   if (tid < 64) {
     const float mine = tid < splits ? part_ml[(slot0 + tid) * 2] : -INFINITY;
     const float m = tw_wave_max(mine);
@@ -540,18 +551,21 @@ __global__ __launch_bounds__(TW_REDUCE_THREADS) void attn_decode_reduce_kernel(
     if (tid == 0) s_l = l;
   }
   __syncthreads();
-  const int cols = TW_REDUCE_THREADS / head_dim > 0 ? TW_REDUCE_THREADS / head_dim : 1;   // head_dim <= 256
-  const int d = tid % head_dim, c = tid / head_dim;
   float o = 0.f;
-  if (c < cols)
-    for (int sp = c; sp < splits; sp += cols) o += part_o[(slot0 + sp) * head_dim + d] * s_w[sp];
+  if (c < cols) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int sp = c + i * cols;
+      if (sp < splits) o += po[i] * s_w[sp];
+    }
+    for (int sp = c + 8 * cols; sp < splits; sp += cols) o += part_o[(slot0 + sp) * head_dim + d] * s_w[sp];
+  }
   s_acc[tid] = o;
   __syncthreads();
   if (tid < head_dim) {
     float total = 0.f;
     for (int i = 0; i < cols; ++i) total += s_acc[i * head_dim + tid];
     const float l = s_l;
-    const int token = q_start[seq0 + local];
     out[(size_t)token * ldo + (size_t)head * head_dim + tid] = tw_from_float<T>(l > 0.f ? total / l : 0.f);
   }
 }

@@ -88,29 +88,35 @@ __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restri
   const bool mine = h < hidden;
   float* src = x + (size_t)r * hidden;
   f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  f32x4 wv = {0.f, 0.f, 0.f, 0.f};
   if (mine) {
+    // Every load of the row is issued before the first one is waited for (the kernel's time is a
+    // chain of memory latencies): the row itself, the weight, and the partial sums 8 at a time.
+    // The partial sums are still added one after the other in index order, then the row.
+    const f32x4 xv = *reinterpret_cast<const f32x4*>(src + h);
+    wv = *reinterpret_cast<const f32x4*>(w + h);
     if (add) {
       const float* p = add + (size_t)r * hidden + h;
-      int s = 0;
-      for (; s + 4 <= add_splits; s += 4) {
-        const f32x4 a0 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 0) * add_stride);
-        const f32x4 a1 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 1) * add_stride);
-        const f32x4 a2 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 2) * add_stride);
-        const f32x4 a3 = *reinterpret_cast<const f32x4*>(p + (size_t)(s + 3) * add_stride);
-        v = (((v + a0) + a1) + a2) + a3;
+      for (int s0 = 0; s0 < add_splits; s0 += 8) {
+        f32x4 a[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          a[i] = s0 + i < add_splits ? *reinterpret_cast<const f32x4*>(p + (size_t)(s0 + i) * add_stride)
+                                     : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (s0 + i < add_splits) v = v + a[i];
       }
-      for (; s < add_splits; ++s) v = v + *reinterpret_cast<const f32x4*>(p + (size_t)s * add_stride);
-      v = v + *reinterpret_cast<const f32x4*>(src + h);
+      v = v + xv;
       if (!rows) *reinterpret_cast<f32x4*>(src + h) = v;
     } else {
-      v = *reinterpret_cast<const f32x4*>(src + h);
+      v = xv;
     }
   }
   float ss = mine ? ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3] : 0.f;
   ss = tw_block_sum(ss, lds);
   const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
   if (mine) {
-    const f32x4 wv = *reinterpret_cast<const f32x4*>(w + h);
     T* dst = out + (size_t)o * hidden + h;
     T packed[4];
 #pragma unroll
@@ -184,6 +190,13 @@ extern "C" int tw_rope_table(const int* positions, const float* inv_freq, float*
 // slot = page * page_size + offset; a negative slot writes nothing.
 // (With `partial`, the split-K sums of the q/k/v projection, qkv_finish_kernel below does the
 // same from round_T(sum_s partial[s][n][col] + bias[col]), one workgroup per (token, head).)
+// One rotated pair, with the products and sums spelled out so that both kernels below round alike
+// (left to the compiler, a*b - c*d is contracted to one fused multiply-add or the other).
+__device__ __forceinline__ void tw_rotate_pair(float lo, float hi, float c, float s, float& out_lo, float& out_hi) {
+  out_lo = __fmaf_rn(lo, c, -__fmul_rn(hi, s));
+  out_hi = __fmaf_rn(hi, c, __fmul_rn(lo, s));
+}
+
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* __restrict__ cos_t,
                                      const float* __restrict__ sin_t, const int* __restrict__ slots,
@@ -203,9 +216,9 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* 
     const int head = i / half, j = i % half;
     T* x = row + (size_t)head * head_dim;
     const float lo = tw_to_float(x[j]), hi = tw_to_float(x[j + half]);
-    const float cj = c[j], sj = s[j];
-    const T out_lo = tw_from_float<T>(lo * cj - hi * sj);
-    const T out_hi = tw_from_float<T>(hi * cj + lo * sj);
+    float r_lo, r_hi;
+    tw_rotate_pair(lo, hi, c[j], s[j], r_lo, r_hi);
+    const T out_lo = tw_from_float<T>(r_lo), out_hi = tw_from_float<T>(r_hi);
     if (head < q_heads) {
       x[j] = out_lo;
       x[j + half] = out_hi;
@@ -247,11 +260,32 @@ __global__ void qkv_finish_kernel(T* __restrict__ qkv, long ld, const float* __r
   const int half = rot / 2;
   const int col0 = head * head_dim;
   const float* src = partial + (size_t)n * width + col0;
-  auto value = [&](int d) {
-    float v = 0.f;
-    for (int s = 0; s < splits; ++s) v += src[s * split_stride + d];
-    if (bias) v += bias[col0 + d];
-    return tw_to_float(tw_from_float<T>(v));          // what the projection would have stored
+  // The sums of two columns at once, every load issued before the first is waited for (the
+  // kernel's time is a chain of memory latencies); added in split order, then the bias.
+  auto values2 = [&](int d0, int d1, float& v0, float& v1) {
+    v0 = 0.f;
+    v1 = 0.f;
+    const float b0 = bias ? bias[col0 + d0] : 0.f, b1 = bias ? bias[col0 + d1] : 0.f;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+      float a0[8], a1[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        a0[i] = s0 + i < splits ? src[(s0 + i) * split_stride + d0] : 0.f;
+        a1[i] = s0 + i < splits ? src[(s0 + i) * split_stride + d1] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (s0 + i < splits) {
+          v0 += a0[i];
+          v1 += a1[i];
+        }
+    }
+    if (bias) {
+      v0 += b0;
+      v1 += b1;
+    }
+    v0 = tw_to_float(tw_from_float<T>(v0));           // what the projection would have stored
+    v1 = tw_to_float(tw_from_float<T>(v1));
   };
   const int slot = write_cache ? slots[n] : -1;
   const int page = slot >= 0 ? slot / page_size : 0;
@@ -262,17 +296,32 @@ __global__ void qkv_finish_kernel(T* __restrict__ qkv, long ld, const float* __r
     if (!is_q && slot < 0) return;
     T* dst = is_q ? row : keys + (((size_t)page * kv_heads + (head - q_heads)) * page_size + off) * head_dim;
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
-      const float lo = value(j), hi = value(j + half);
       const float cj = cos_t[(size_t)n * half + j], sj = sin_t[(size_t)n * half + j];
-      dst[j] = tw_from_float<T>(lo * cj - hi * sj);
-      dst[j + half] = tw_from_float<T>(hi * cj + lo * sj);
+      float lo, hi;
+      values2(j, j + half, lo, hi);
+      float r_lo, r_hi;
+      tw_rotate_pair(lo, hi, cj, sj, r_lo, r_hi);
+      dst[j] = tw_from_float<T>(r_lo);
+      dst[j + half] = tw_from_float<T>(r_hi);
     }
-    for (int d = rot + threadIdx.x; d < head_dim; d += blockDim.x) dst[d] = tw_from_float<T>(value(d));
+    for (int d = rot + threadIdx.x; d < head_dim; d += 2 * blockDim.x) {      // the part that is not rotated
+      const int d1 = d + blockDim.x < head_dim ? d + blockDim.x : d;
+      float v0, v1;
+      values2(d, d1, v0, v1);
+      dst[d] = tw_from_float<T>(v0);
+      if (d1 != d) dst[d1] = tw_from_float<T>(v1);
+    }
   } else {
     if (slot < 0) return;
     const int kh = head - q_heads - kv_heads;
     T* dst = values + ((size_t)page * kv_heads + kh) * head_dim * page_size + off;
-    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) dst[(size_t)d * page_size] = tw_from_float<T>(value(d));
+    for (int d = threadIdx.x; d < head_dim; d += 2 * blockDim.x) {
+      const int d1 = d + blockDim.x < head_dim ? d + blockDim.x : d;
+      float v0, v1;
+      values2(d, d1, v0, v1);
+      dst[(size_t)d * page_size] = tw_from_float<T>(v0);
+      if (d1 != d) dst[(size_t)d1 * page_size] = tw_from_float<T>(v1);
+    }
   }
 }
 
