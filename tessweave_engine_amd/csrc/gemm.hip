@@ -19,6 +19,7 @@
 // C[M, N/2][.., 16j + i] = silu(gate_j[i]) * up_j[i] in their epilogues, in float32 from the
 // accumulators, so the [M, N] intermediate never reaches memory.
 #include "tw_common.h"
+#include "gemm_shared.h"
 
 // element offset of (row n, 16-byte chunk c) in the shuffled layout
 __device__ __forceinline__ size_t tw_shuffled_chunk(int n, int c, int k_steps, int epf) {
@@ -29,310 +30,6 @@ template <typename T>
 __device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p) {
   // weights are read once per step: do not keep them in the caches
   return __builtin_nontemporal_load(reinterpret_cast<const typename Elem<T>::Frag*>(p));
-}
-
-__device__ __forceinline__ float tw_silu(float g) { return g / (1.0f + expf(-g)); }
-
-// Epilogue of the tiled kernels: each wave passes its tile through LDS (32 rows at a time) so
-// that a lane stores 8 consecutive columns of one row, whole cache lines instead of 2- or 4-byte
-// pieces; bias, residual, the output type and the SiLU-multiply of GLU pairs are applied here.
-// `lds` must hold 4 waves x 32 rows x (32 * WN + 4) floats and no wave may still read its old contents
-// (the first __syncthreads below sees to that).
-template <typename OutT, int WM, int WN, bool GLU>
-__device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* lds, const float* __restrict__ bias,
-                                                  const float* residual, long ldr, OutT* C, long ldc, int M, int N,
-                                                  int m0, int n0, int wm0, int wn0, int wave, int lane) {
-  const int r = lane & 31, g = lane >> 5;
-  constexpr int WCOLS = 32 * WN;                             // columns of a wave tile
-  constexpr int EROW = WCOLS + 4;                            // floats per staged row, padded
-  // (the launcher asks for max(pipeline stages, 4 waves x 32 rows x EROW floats) bytes of LDS)
-  float* stage = reinterpret_cast<float*>(lds) + wave * 32 * EROW;
-  constexpr int CPR = WCOLS / 8;                             // 8-column groups per row
-  const bool vec_ok = (ldc % 8 == 0) && (residual == nullptr || ldr % 4 == 0) &&
-                      ((uintptr_t)C % 16 == 0) && ((uintptr_t)residual % 16 == 0);
-#pragma unroll
-  for (int i = 0; i < WM; ++i) {
-    __syncthreads();                                          // the pipeline's (or the last round's) LDS reads are done
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * g + (e % 4)) * EROW + j * 32 + r] = acc[i][j][e];
-    __syncthreads();
-    if (GLU) {
-      // a wave tile's columns are [gate 16 | up 16] pairs; a lane forms 8 outputs of one row
-      constexpr int GPR = WCOLS / 16;                         // 8-output groups per row
-#pragma unroll
-      for (int q = lane; q < 32 * GPR; q += 64) {
-        const int lr = q / GPR, og = q % GPR;
-        const int lc = (og >> 1) * 32 + (og & 1) * 8;         // gate columns lc.., up columns lc + 16..
-        const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
-        if (row >= M || col + 24 > N) continue;               // N is a multiple of 32: groups are whole
-        float v[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          float gv = stage[lr * EROW + lc + e], uv = stage[lr * EROW + lc + 16 + e];
-          if (bias) { gv += bias[col + e]; uv += bias[col + 16 + e]; }
-          v[e] = tw_silu(gv) * uv;
-        }
-        OutT* dst = C + (size_t)row * ldc + (n0 + wn0) / 2 + (og >> 1) * 16 + (og & 1) * 8;
-        if (ldc % 8 == 0 && (uintptr_t)C % 16 == 0) {
-          if (sizeof(OutT) == 4) {
-            *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
-          } else {
-            bf16x8 o;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
-            *reinterpret_cast<bf16x8*>(dst) = o;
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) dst[e] = tw_from_float<OutT>(v[e]);
-        }
-      }
-      continue;
-    }
-#pragma unroll
-    for (int q = lane; q < 32 * CPR; q += 64) {
-      const int lr = q / CPR, lc = (q % CPR) * 8;
-      const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
-      if (row >= M || col >= N) continue;
-      float v[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = stage[lr * EROW + lc + e];
-      if (bias) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (col + e < N) v[e] += bias[col + e];
-      }
-      if (vec_ok && col + 8 <= N) {
-        if (residual) {
-          const f32x4 r0 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col);
-          const f32x4 r1 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col + 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { v[e] += r0[e]; v[4 + e] += r1[e]; }
-        }
-        OutT* dst = C + (size_t)row * ldc + col;
-        if (sizeof(OutT) == 4) {
-          *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-          *reinterpret_cast<f32x4*>(dst + 4) = f32x4{v[4], v[5], v[6], v[7]};
-        } else {
-          bf16x8 o;
-#pragma unroll
-          for (int e = 0; e < 8; ++e) o[e] = (bf16_t)v[e];
-          *reinterpret_cast<bf16x8*>(dst) = o;
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (col + e < N) {
-            float x = v[e];
-            if (residual) x += residual[(size_t)row * ldr + col + e];
-            C[(size_t)row * ldc + col + e] = tw_from_float<OutT>(x);
-          }
-      }
-    }
-  }
-}
-
-// =====================================================================================
-// Tiled kernel. Workgroup = 4 waves in a 2x2 grid, wave tile (32*WM) x (32*WN).
-// One stage holds 128 bytes of K per row (64 bf16 / 32 f32), rows padded to 144
-// bytes in LDS so that 16-byte fragment reads of 8 consecutive lanes hit
-// distinct banks. Two stages: the next stage's global loads are in flight
-// while the current one is multiplied.
-// =====================================================================================
-#define TW_LDS_ROW 144
-
-// SHUF: W is in the shuffled layout and ldw is its k_steps. GLU: see the top of the file.
-template <typename T, typename OutT, int WM, int WN, bool SHUF, bool GLU>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A, long lda,
-                                                         const T* __restrict__ W, long ldw,
-                                                         const float* __restrict__ bias,
-                                                         const float* residual, long ldr, OutT* C,
-                                                         long ldc, int M, int N, int K, int tiles_m,
-                                                         int n_blocks, int splits, float* __restrict__ partial) {
-  typedef typename Elem<T>::Frag Frag;
-  constexpr int EPF = Elem<T>::kPerFrag;
-  constexpr int KCH = 8;                                    // 16-byte chunks of K per row and stage
-  constexpr int BK = KCH * EPF;
-  constexpr int BM = 64 * WM, BN = 64 * WN;
-  constexpr int LROW = KCH * 16 + 16;                       // LDS bytes per row of a stage, padded
-  constexpr int A_LOADS = BM * KCH / 256, W_LOADS = BN * KCH / 256;
-  constexpr int STAGE = (BM + BN) * LROW;                   // bytes of one stage: A rows then W rows
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-
-  // Blocks are dealt to the 8 XCDs round-robin; give each XCD a contiguous run
-  // of tiles so that neighbours sharing a weight tile share an L2.
-  const int per_xcd = gridDim.x / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (logical >= n_blocks) return;
-  // splits > 1 (few tiles, long K): the k-tiles are dealt to `splits` workgroups per tile, which
-  // leave float32 partial sums partial[split][M][N] for splitk_reduce_kernel.
-  const int n_tiles = n_blocks / splits;
-  const int split = logical / n_tiles, tile = logical % n_tiles;
-  const int tile_m = tile % tiles_m, tile_n = tile / tiles_m;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm0 = (wave >> 1) * 32 * WM, wn0 = (wave & 1) * 32 * WN;
-  const int r = lane & 31, g = lane >> 5;
-
-  f32x16 acc[WM][WN];
-#pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-  // Global addressing: a tile base that is the same for every lane, plus per-thread element
-  // offsets fixed for the whole K loop. Rows past the end are clamped to the last valid row
-  // (what they produce is never stored), so whole k-tiles need no predicate.
-  const T* a_tile = A + (size_t)m0 * lda;
-  const T* w_tile = SHUF ? W + (size_t)(n0 / 16) * ldw * 64 * EPF : W + (size_t)n0 * ldw;
-  const int k_steps_w = SHUF ? (int)ldw : 0;
-  unsigned a_off[A_LOADS], w_off[W_LOADS];
-  int st_off[A_LOADS];
-#pragma unroll
-  for (int i = 0; i < A_LOADS; ++i) {
-    const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
-    a_off[i] = (unsigned)(min(m0 + row, M - 1) - m0) * (unsigned)lda + kc * EPF;
-  }
-  constexpr int SPT = KCH / 4;                             // shuffled k-steps per k-tile
-  int w_st_off[W_LOADS], w_ks[W_LOADS];
-  const int n_blocks_w = (N + 15) / 16;
-#pragma unroll
-  for (int i = 0; i < W_LOADS; ++i) {
-    const int c = tid + i * 256;
-    if (SHUF) {
-      // piece c of the tile: block (16 rows x 4 chunks) c / 64, lane c % 64 of that block
-      const int blk = c >> 6, ln = c & 63, nblk = blk / SPT, ks = blk % SPT;
-      const int gblk = min(n0 / 16 + nblk, n_blocks_w - 1);
-      w_off[i] = (unsigned)(gblk - n0 / 16) * (unsigned)ldw * 64 * EPF + (ks * 64 + ln) * EPF;
-      w_ks[i] = ks;
-      w_st_off[i] = (nblk * 16 + (ln & 15)) * LROW + (ks * 4 + (ln >> 4)) * 16;
-    } else {
-      const int row = c / KCH, kc = c % KCH;
-      w_off[i] = (unsigned)(min(n0 + row, N - 1) - n0) * (unsigned)ldw + kc * EPF;
-      w_ks[i] = 0;
-      w_st_off[i] = row * LROW + kc * 16;
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < A_LOADS; ++i) {
-    const int c = tid + i * 256, row = c / KCH, kc = c % KCH;
-    st_off[i] = row * LROW + kc * 16;
-  }
-  const int kc_mine = tid % KCH;
-
-  // Two register sets: the global loads of k-tile kt+2 are issued while k-tile kt is multiplied,
-  // so two k-tiles per workgroup are on their way from memory at any time.
-  Frag a_regs[2][A_LOADS], w_regs[2][W_LOADS];
-  const int k_tiles_all = (K + BK - 1) / BK;
-  const int per_split = (k_tiles_all + splits - 1) / splits;
-  const int kt0 = split * per_split;                          // this workgroup's k-tiles: kt0 .. kt0 + k_tiles - 1
-  const int k_tiles = max(0, min(k_tiles_all, kt0 + per_split) - kt0);
-  const int whole_tiles = K / BK;
-
-  // whole k-tiles need no predicate at all; the main loop below runs only those
-  auto load_whole = [&](int kt, Frag* a_reg, Frag* w_reg) {
-    const T* ab = a_tile + (size_t)kt * BK;
-    const T* wb = SHUF ? w_tile + (size_t)kt * SPT * 64 * EPF : w_tile + (size_t)kt * BK;
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) a_reg[i] = tw_load_frag(ab + a_off[i]);
-#pragma unroll
-    for (int i = 0; i < W_LOADS; ++i) w_reg[i] = tw_load_frag(wb + w_off[i]);
-  };
-  auto load_global = [&](int kt, Frag* a_reg, Frag* w_reg) {
-    if (kt < whole_tiles) {
-      load_whole(kt, a_reg, w_reg);
-    } else {                                                // the last, partial k-tile: chunks past K are zeros
-      const T* ab = a_tile + (size_t)kt * BK;
-      const T* wb = SHUF ? w_tile + (size_t)kt * SPT * 64 * EPF : w_tile + (size_t)kt * BK;
-      const bool ok = kt * BK + kc_mine * EPF < K;
-#pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) a_reg[i] = ok ? tw_load_frag(ab + a_off[i]) : Elem<T>::zero();
-#pragma unroll
-      for (int i = 0; i < W_LOADS; ++i) {
-        const bool w_ok = SHUF ? kt * SPT + w_ks[i] < k_steps_w : ok;     // the shuffled layout is zero padded
-        w_reg[i] = w_ok ? tw_load_frag(wb + w_off[i]) : Elem<T>::zero();
-      }
-    }
-  };
-  auto store_lds = [&](int buf, const Frag* a_reg, const Frag* w_reg) {
-    char* base = lds + buf * STAGE;
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<Frag*>(base + st_off[i]) = a_reg[i];
-#pragma unroll
-    for (int i = 0; i < W_LOADS; ++i) *reinterpret_cast<Frag*>(base + BM * LROW + w_st_off[i]) = w_reg[i];
-  };
-
-  // this lane's fragment addresses in stage 0 (k-chunk pair cc adds 32 bytes)
-  const char* a_frag = lds + (wm0 + r) * LROW + g * 16;
-  const char* w_frag = lds + (BM + wn0 + r) * LROW + g * 16;
-  auto read_frags = [&](int buf, int cc, Frag* af, Frag* wf) {
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-      af[i] = *reinterpret_cast<const Frag*>(a_frag + buf * STAGE + i * 32 * LROW + cc * 32);
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-      wf[j] = *reinterpret_cast<const Frag*>(w_frag + buf * STAGE + j * 32 * LROW + cc * 32);
-  };
-
-  auto multiply = [&](int buf) {
-    // the fragments of the next k-chunk pair are read from LDS while this one is multiplied
-    Frag af[2][WM], wf[2][WN];
-    read_frags(buf, 0, af[0], wf[0]);
-#pragma unroll
-    for (int cc = 0; cc < KCH / 2; ++cc) {
-      if (cc + 1 < KCH / 2) read_frags(buf, cc + 1, af[(cc + 1) & 1], wf[(cc + 1) & 1]);
-#pragma unroll
-      for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[cc & 1][i], wf[cc & 1][j]);
-    }
-  };
-
-  if (k_tiles > 0) {
-    load_global(kt0, a_regs[0], w_regs[0]);
-    if (k_tiles > 1) load_global(kt0 + 1, a_regs[1], w_regs[1]);
-    store_lds(0, a_regs[0], w_regs[0]);
-  }
-  __syncthreads();
-  int j = 0;                                                  // k-tile kt0 + j is in LDS stage j & 1
-  // Main loop: two k-tiles per round, every load whole and unconditional, so that the register
-  // sets are plain loop-carried values (conditional loads cost a register copy per loaded dword).
-  const int whole_here = min(k_tiles, whole_tiles - kt0);
-  for (; j + 3 < whole_here; j += 2) {
-    load_whole(kt0 + j + 2, a_regs[0], w_regs[0]);           // LDS stage 0, register set 0 is free
-    multiply(0);
-    store_lds(1, a_regs[1], w_regs[1]);
-    __syncthreads();
-    load_whole(kt0 + j + 3, a_regs[1], w_regs[1]);           // LDS stage 1, register set 1 is free
-    multiply(1);
-    store_lds(0, a_regs[0], w_regs[0]);
-    __syncthreads();
-  }
-  // The last few k-tiles (j is even here): the same rounds with every step conditional.
-  for (; j < k_tiles; j += 2) {
-    if (j + 2 < k_tiles) load_global(kt0 + j + 2, a_regs[0], w_regs[0]);
-    multiply(0);
-    if (j + 1 < k_tiles) store_lds(1, a_regs[1], w_regs[1]);
-    __syncthreads();
-    if (j + 1 >= k_tiles) break;
-    if (j + 3 < k_tiles) load_global(kt0 + j + 3, a_regs[1], w_regs[1]);
-    multiply(1);
-    if (j + 2 < k_tiles) store_lds(0, a_regs[0], w_regs[0]);
-    __syncthreads();
-  }
-
-  if (splits > 1) {
-    tw_tiled_epilogue<float, WM, WN, false>(acc, lds, nullptr, nullptr, 0, partial + (size_t)split * M * N, (long)N,
-                                            M, N, m0, n0, wm0, wn0, wave, lane);
-    return;
-  }
-  tw_tiled_epilogue<OutT, WM, WN, GLU>(acc, lds, bias, residual, ldr, C, ldc, M, N, m0, n0, wm0, wn0, wave, lane);
 }
 
 // =====================================================================================
@@ -512,20 +209,6 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
   }
 }
 
-template <typename OutT>
-__global__ void splitk_reduce_kernel(const float* __restrict__ partial, int splits,
-                                     const float* __restrict__ bias, const float* residual, long ldr,
-                                     OutT* C, long ldc, int M, int N) {
-  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= (long)M * N) return;
-  const int row = (int)(i / N), col = (int)(i % N);
-  float v = 0.f;
-  for (int s = 0; s < splits; ++s) v += partial[(size_t)s * M * N + i];
-  if (bias) v += bias[col];
-  if (residual) v += residual[(size_t)row * ldr + col];
-  C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
-}
-
 // =====================================================================================
 // Generic kernel: any K. One thread per output element, float32 accumulation.
 // =====================================================================================
@@ -569,54 +252,6 @@ __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* 
 // =====================================================================================
 // Host side
 // =====================================================================================
-// How many K ranges the tiled kernel uses: with fewer tiles than the chip has room for (a prompt
-// portion of a few hundred rows against a square or tall matrix) the k-tiles of a tile are dealt
-// to several workgroups. Depends on the shape only.
-static int tiled_splits(int M, int N, int K, int epf, int bm, int bn) {
-  const long tiles = (long)tw_div_up(M, bm) * tw_div_up(N, bn);
-  if (tiles >= 192) return 1;
-  const int k_tiles = tw_div_up(K, 8 * epf);
-  long splits = tw_div_up(384, tiles);
-  if (splits > k_tiles / 8) splits = k_tiles / 8;
-  if (splits > 8) splits = 8;
-  return splits < 1 ? 1 : (int)splits;
-}
-
-template <typename T, typename OutT, int WM, int WN, bool SHUF, bool GLU>
-static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
-                        const float* residual, long ldr, OutT* C, long ldc, float* partial,
-                        long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  constexpr int BM = 64 * WM, BN = 64 * WN, KCH = 8;
-  constexpr int EPF = Elem<T>::kPerFrag;
-  const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
-  int splits = GLU ? 1 : tiled_splits(M, N, K, EPF, BM, BN);
-  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4 || (uintptr_t)partial % 16 != 0)) splits = 1;
-  const long n_blocks = (long)tiles_m * tiles_n * splits;
-  TW_REQUIRE(n_blocks < (1L << 30));
-  // per-tile offsets are 32-bit
-  TW_REQUIRE((long)BM * lda < (1L << 31));
-  TW_REQUIRE(SHUF ? (long)(BN / 16) * ldw * 64 * EPF < (1L << 31) : (long)BN * ldw < (1L << 31));
-  const int grid = (int)((n_blocks + 7) / 8 * 8);
-  const size_t pipeline_bytes = 2 * (size_t)(BM + BN) * (KCH * 16 + 16);
-  const size_t epilogue_bytes = 4 * 32 * (size_t)(32 * WN + 4) * 4;
-  const size_t lds_bytes = pipeline_bytes > epilogue_bytes ? pipeline_bytes : epilogue_bytes;
-  auto kernel = gemm_tiled_kernel<T, OutT, WM, WN, SHUF, GLU>;
-  static bool attribute_set = false;   // per instantiation
-  if (!attribute_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes);
-    if (e != hipSuccess) return (int)e;
-    attribute_set = true;
-  }
-  kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m,
-                                           (int)n_blocks, splits, partial);
-  int err = TW_LAUNCH_RESULT();
-  if (err || splits == 1) return err;
-  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
-                                                                             ldr, C, ldc, M, N);
-  return TW_LAUNCH_RESULT();
-}
-
 // How many K ranges the skinny kernel uses for an [N, K] weight: enough workgroups to fill 256
 // CUs twice, each range at least 16 MFMA steps long. The choice depends on N and K only, never
 // on the rows of a batch.
@@ -638,8 +273,7 @@ extern "C" long tw_linear_workspace_bytes(int dtype, int max_rows, int N, int K)
   int splits = skinny_lds_splits(N, K, epf);
   long bytes = splits > 1 ? (long)splits * rows * N * 4 : 0;
   if (max_rows > 64) {
-    splits = tiled_splits(max_rows, N, K, epf, 128, 128);
-    const long tiled = splits > 1 ? (long)splits * max_rows * N * 4 : 0;
+    const long tiled = tw_tiled_workspace_bytes(dtype, max_rows, N, K);
     if (tiled > bytes) bytes = tiled;
   }
   return bytes;
@@ -677,13 +311,13 @@ static int launch_skinny_lds_m(const T* A, long lda, const T* W, long ldw, const
   return launch_skinny_lds<T, OutT, 4, PARTIAL, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
 }
 
-// force: 0 = choose, 1 = generic, 3 = tiled 128x128, 4 = tiled 128x256, 5 = skinny
+// force: 0 = choose, 1 = generic, 3 = tiled 128x128, 4 = tiled 128x256, 5 = skinny, 6 = tiled 256x256
 template <typename T, typename OutT, bool SHUF, bool GLU>
 static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const float* bias,
                            const float* residual, long ldr, OutT* C, long ldc, float* partial,
                            long partial_bytes, int M, int N, int K, int force, hipStream_t stream) {
   constexpr int EPF = Elem<T>::kPerFrag;
-  TW_REQUIRE(force == 0 || force == 1 || force == 3 || force == 4 || force == 5);
+  TW_REQUIRE(force == 0 || force == 1 || force == 3 || force == 4 || force == 5 || force == 6);
   // the shuffled layout exists only for K that is a multiple of 16 bytes and is always aligned
   const bool aligned = K % EPF == 0 && lda % EPF == 0 && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) &&
                        (SHUF || ldw % EPF == 0);
@@ -699,9 +333,10 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
     TW_REQUIRE(M <= 64);
     return launch_skinny_lds_m<T, OutT, false, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
-  if (force == 4)
-    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  const int shape = force == 3 ? 1 : (force == 4 ? 2 : (force == 6 ? 3 : 0));
+  return tw_tiled_linear(sizeof(T) == 4 ? TW_DTYPE_F32 : TW_DTYPE_BF16, sizeof(OutT) == 4 ? 1 : 0, SHUF ? 1 : 0,
+                         GLU ? 1 : 0, shape, A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes,
+                         M, N, K, stream);
 }
 
 template <typename T, typename OutT>

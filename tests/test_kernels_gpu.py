@@ -161,8 +161,12 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
     t = dict(atol=2e-5 * scale, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2 * scale, rtol=2e-2)
     shuffled = ops.shuffle_weight(w)
     torch.testing.assert_close(shuffled.to_rows(), w, atol=0, rtol=0)          # an exact permutation
+    big = (ops.GEMM_TILED_256,) if dtype == torch.bfloat16 else ()     # 256x256 tiles: bfloat16, shuffled weights
+    if not big:                                                        # ... and refused otherwise
+        with pytest.raises(Exception, match="refused its arguments"):
+            ops.linear(x, shuffled, torch.empty((m, n), dtype=dtype, device=device), force=ops.GEMM_TILED_256)
     for force in forces + [("shuffled", f) for f in (ops.GEMM_AUTO, ops.GEMM_GENERIC, ops.GEMM_TILED, ops.GEMM_TILED_WIDE)
-                           + ((ops.GEMM_SKINNY,) if m <= 64 else ())]:
+                           + big + ((ops.GEMM_SKINNY,) if m <= 64 else ())]:
         wt = w
         if isinstance(force, tuple):
             wt, force = shuffled, force[1]
@@ -204,7 +208,7 @@ def test_linear_partials(ops, device, dtype, m, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 64), (8, 208, 320), (17, 48, 1032), (64, 1040, 256), (65, 80, 64),
-                                       (200, 400, 320), (130, 16, 101)])
+                                       (200, 400, 320), (130, 16, 101), (520, 272, 200)])
 def test_linear_glu(ops, device, dtype, m, inter, k):
     """silu(x gate^T + b) * (x up^T + b) from interleaved rows, every kernel and both layouts."""
     x = rand((m, k), dtype, device, 1.0, seed=1)
@@ -226,7 +230,8 @@ def test_linear_glu(ops, device, dtype, m, inter, k):
         u = xd @ up.double().cpu().T + (bu.double().cpu() if b is not None else 0)
         want = torch.nn.functional.silu(g) * u
         for weight in layouts:
-            for force in forces:
+            big = [ops.GEMM_TILED_256] if (dtype == torch.bfloat16 and weight is not w) else []
+            for force in forces + big:
                 out = torch.full((m, inter), float("nan"), dtype=dtype, device=device)
                 ops.linear_glu(x, weight, out, bias=b, force=force)
                 torch.testing.assert_close(out.double().cpu(), want, **t)
