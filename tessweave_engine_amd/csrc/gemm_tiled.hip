@@ -141,7 +141,14 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
   // leave float32 partial sums partial[split][M][N] for splitk_reduce_kernel.
   const int n_tiles = n_blocks / splits;
   const int split = logical / n_tiles, tile = logical % n_tiles;
-  const int tile_m = tile % tiles_m, tile_n = tile / tiles_m;
+  // Tiles in bands of 2,048 rows, so that the workgroups an XCD runs at a time share column tiles as
+  // well as row tiles (all the row tiles of a tall matrix in one column would share one weight tile
+  // and fetch an activation tile each).
+  constexpr int BAND = 2048 / BM;
+  const int tiles_n = n_tiles / tiles_m;
+  const int band = tile / (BAND * tiles_n), in_band = tile - band * BAND * tiles_n;
+  const int band_rows = min(BAND, tiles_m - band * BAND);
+  const int tile_m = band * BAND + in_band % band_rows, tile_n = in_band / band_rows;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -324,6 +331,145 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 }
 
 // =====================================================================================
+// 256x256 tiles, bfloat16, shuffled weights, K a multiple of 32, with global memory copied
+// straight into LDS (`global_load_lds_dwordx4`: lane l's 16 bytes land at the wave's LDS base +
+// 16 l, from any address the lane names). No staging registers and no LDS write instructions.
+//
+// A k-tile is 32 elements of K (64 bytes a row, one k-step of the shuffled layout). A stage of
+// LDS holds 16 blocks of A and 16 of W; a block is 16 rows x 4 chunks of 16 bytes in the order
+// [chunk][row], 1 KB, which is how W lies in memory (a fragment read takes 256 consecutive bytes
+// per 16 lanes); an A block is [row][chunk] with the chunks of a row swizzled (see a_src below).
+// Four stages: the copy of k-tile t+4 is started when k-tile t has been read into registers.
+//
+// Per k-tile and wave: 2 k-chunk pairs of 16 MFMAs (wave tile 128x128, accumulators in AGPRs).
+// The fragments of a pair are read while the pair before is multiplied, so the barrier that
+// publishes the next k-tile lies between the two pairs of this one and the matrix unit has
+// work on both sides of it.
+// =====================================================================================
+typedef __attribute__((address_space(3))) void* tw_lds_ptr;
+#define TW_DMA_STAGE 32768
+#ifndef TW_DMA_STAGES
+#define TW_DMA_STAGES 4
+#endif
+
+template <typename OutT, bool GLU>
+__global__ __launch_bounds__(256) void gemm_dma256_kernel(const bf16_t* __restrict__ A, long lda,
+                                                          const bf16_t* __restrict__ W, long k_steps,
+                                                          const float* __restrict__ bias, const float* residual,
+                                                          long ldr, OutT* C, long ldc, int M, int N, int K,
+                                                          int tiles_m, int n_blocks) {
+  constexpr int WM = 4, WN = 4, BM = 256, BN = 256;
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  const int per_xcd = gridDim.x / 8;
+  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;   // neighbours in an XCD share weight tiles
+  if (logical >= n_blocks) return;
+  // Tiles in bands of 8 row tiles: the 32 workgroups an XCD runs at a time then cover 8 row tiles x 4
+  // column tiles and fetch 12 operand tiles between them (with all the row tiles of a tall matrix in
+  // one column they would fetch one per workgroup).
+  const int tiles_n = n_blocks / tiles_m;
+  const int band = logical / (8 * tiles_n), in_band = logical - band * 8 * tiles_n;
+  const int band_rows = min(8, tiles_m - band * 8);
+  const int tile_m = band * 8 + in_band % band_rows, tile_n = in_band / band_rows;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+  const int r = lane & 31, g = lane >> 5;
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // what this lane copies per k-tile: its slot of A blocks 4 wave .. 4 wave + 3 and of W blocks likewise.
+  // Rows past M and blocks past N are clamped to the last valid one (their products are never stored).
+  const int k_tiles = K / 32;
+  const int n_blocks_w = (N + 15) / 16;
+  const bf16_t* a_src[4];
+  const bf16_t* w_src[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    // slot l of an A block holds row l / 4, chunk (l % 4) ^ (row / 4 % 4): four neighbouring lanes fetch
+    // 64 consecutive bytes, and 16 rows of one chunk lie in 16 different 16-byte columns of LDS
+    const int row16 = lane >> 2, chunk = (lane & 3) ^ ((row16 >> 2) & 3);
+    const int row = min(m0 + (4 * wave + b) * 16 + row16, M - 1);
+    a_src[b] = A + (size_t)row * lda + chunk * 8;
+    const int blk = min(n0 / 16 + 4 * wave + b, n_blocks_w - 1);
+    w_src[b] = W + (size_t)blk * k_steps * 512 + lane * 8;
+  }
+  auto copy_tile = [&](int kt_v) {
+    const int kt = min(kt_v, k_tiles - 1);               // past the end: a copy nobody reads
+    char* stage = lds + (kt_v % TW_DMA_STAGES) * TW_DMA_STAGE + wave * 4096;
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      __builtin_amdgcn_global_load_lds(a_src[b] + (size_t)kt * 32, (tw_lds_ptr)(stage + b * 1024), 16, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      __builtin_amdgcn_global_load_lds(w_src[b] + (size_t)kt * 512, (tw_lds_ptr)(stage + 16384 + b * 1024), 16, 0, 0);
+  };
+  // this lane's fragment addresses in stage 0: row block, then chunk 2 cc + g, then row
+  const int a_row16 = r & 15, a_swz = (a_row16 >> 2) & 3;
+  const char* a_block = lds + (wm0 / 16 + (r >> 4)) * 1024 + a_row16 * 64;
+  const char* a_frag_cc[2] = {a_block + ((g ^ a_swz) * 16), a_block + (((2 + g) ^ a_swz) * 16)};
+  const char* w_frag = lds + 16384 + (wn0 / 16 + (r >> 4)) * 1024 + g * 256 + (r & 15) * 16;
+  auto read_frags = [&](int kt, int cc, bf16x8* af, bf16x8* wf) {
+    const int st = (kt % TW_DMA_STAGES) * TW_DMA_STAGE;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(a_frag_cc[cc] + st + i * 2048);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(w_frag + st + cc * 512 + j * 2048);
+  };
+  auto multiply = [&](const bf16x8* af, const bf16x8* wf) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[i], wf[j]);
+  };
+  // wait until at most `n` of this wave's copies are in flight (they finish in order), then meet the others
+#define TW_DMA_PUBLISH(n)                                                     \
+  do {                                                                        \
+    asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)" ::: "memory");          \
+    __builtin_amdgcn_s_barrier();                                             \
+    asm volatile("" ::: "memory");                                            \
+  } while (0)
+#define TW_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+
+  bf16x8 af[2][WM], wf[2][WN];
+#if TW_DMA_STAGES == 4
+#define TW_DMA_PUBLISH_FIRST() TW_DMA_PUBLISH(24)
+#define TW_DMA_PUBLISH_REST() TW_DMA_PUBLISH(16)
+#else
+#define TW_DMA_PUBLISH_FIRST() TW_DMA_PUBLISH(32)
+#define TW_DMA_PUBLISH_REST() TW_DMA_PUBLISH(24)
+#endif
+#pragma unroll
+  for (int t = 0; t < TW_DMA_STAGES; ++t) copy_tile(t);
+  TW_DMA_PUBLISH_FIRST();                                  // k-tile 0 has landed, for every wave
+  read_frags(0, 0, af[0], wf[0]);
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    read_frags(kt, 1, af[1], wf[1]);
+    multiply(af[0], wf[0]);
+    TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+    TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+    // every fragment of k-tile kt is in registers now; k-tile kt + 1 (copies of kt + 2 and kt + 3
+    // may still be in flight) becomes visible, and kt's stage is free for kt + 4
+    TW_DMA_PUBLISH_REST();
+    copy_tile(kt + TW_DMA_STAGES);
+    read_frags(kt + 1, 0, af[0], wf[0]);                   // (after the last k-tile: read, never used)
+    multiply(af[1], wf[1]);
+    TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+    TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // no copy may land in the epilogue's staging area
+#undef TW_SGB
+#undef TW_DMA_PUBLISH
+  tw_tiled_epilogue<OutT, WM, WN, GLU>(acc, lds, bias, residual, ldr, C, ldc, M, N, m0, n0, wm0, wn0, wave, lane);
+}
+
+// =====================================================================================
 // Host side
 // =====================================================================================
 // How many K ranges the tiled kernel uses: with fewer tiles than the chip has room for (a prompt
@@ -375,12 +521,34 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
 }
 
 
-// Which tile: 256x256 when there are at least two rounds of them for 256 CUs (per MFMA it moves half
+template <typename OutT, bool GLU>
+static int launch_dma256(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias,
+                         const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
+                         hipStream_t stream) {
+  TW_REQUIRE(K % 32 == 0 && K >= 32 && lda % 8 == 0);
+  const int tiles_m = tw_div_up(M, 256), tiles_n = tw_div_up(N, 256);
+  const long n_blocks = (long)tiles_m * tiles_n;
+  TW_REQUIRE(n_blocks < (1L << 30));
+  const int grid = (int)((n_blocks + 7) / 8 * 8);
+  const size_t lds_bytes = TW_DMA_STAGES * TW_DMA_STAGE;          // also covers the epilogue's staging area
+  auto kernel = gemm_dma256_kernel<OutT, GLU>;
+  static bool attribute_set = false;   // per instantiation
+  if (!attribute_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    attribute_set = true;
+  }
+  kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m, (int)n_blocks);
+  return TW_LAUNCH_RESULT();
+}
+
+// Which tile: 256x256 when there are at least one and a half rounds of them for 256 CUs (per MFMA it moves half
 // the bytes through the 64 B/clk vector-memory path and the LDS that 128x128 does); 128x256 when that
 // makes one round that fills most of the chip; else 128x128, two workgroups per CU.
 static int choose_shape(bool big_ok, int M, int N) {
   if (big_ok) {
-    if ((long)tw_div_up(M, 256) * tw_div_up(N, 256) >= 512) return 3;
+    if ((long)tw_div_up(M, 256) * tw_div_up(N, 256) >= 384) return 3;
     const long wide = (long)tw_div_up(M, 128) * tw_div_up(N, 256);
     if (wide >= 192 && wide <= 256) return 2;
   }
@@ -394,8 +562,11 @@ static int tiled_by_shape(int shape, const T* A, long lda, const T* W, long ldw,
   constexpr bool BIG = sizeof(T) == 2 && SHUF;
   if (shape == 0) shape = choose_shape(BIG, M, N);
   if (shape == 3) {
-    if constexpr (BIG)
+    if constexpr (BIG) {
+      if (K % 32 == 0)
+        return launch_dma256<OutT, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
       return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    }
     return TW_ERR_BAD_ARGUMENT;
   }
   if (shape == 2)
