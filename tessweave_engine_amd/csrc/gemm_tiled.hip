@@ -348,17 +348,20 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 // =====================================================================================
 typedef __attribute__((address_space(3))) void* tw_lds_ptr;
 #define TW_DMA_STAGE 32768
-#ifndef TW_DMA_STAGES
 #define TW_DMA_STAGES 4
+#ifndef TW_DMA_WAVES
+#define TW_DMA_WAVES 4          /* 8 (two waves to a SIMD, 128x64 each) measured 2-5 % slower */
 #endif
 
-template <typename OutT, bool GLU>
-__global__ __launch_bounds__(256) void gemm_dma256_kernel(const bf16_t* __restrict__ A, long lda,
+// NW waves in 2 rows: 4 waves with tiles of 128x128 each, or 8 with 128x64 (two to a SIMD).
+// WCOLS: waves side by side; CB: blocks of A, and of W, a wave copies per k-tile.
+template <typename OutT, bool GLU, int NW, int WCOLS = NW / 2, int CB = 16 / NW>
+__global__ __launch_bounds__(64 * NW) void gemm_dma256_kernel(const bf16_t* __restrict__ A, long lda,
                                                           const bf16_t* __restrict__ W, long k_steps,
                                                           const float* __restrict__ bias, const float* residual,
                                                           long ldr, OutT* C, long ldc, int M, int N, int K,
                                                           int tiles_m, int n_blocks) {
-  constexpr int WM = 4, WN = 4, BM = 256, BN = 256;
+  constexpr int WM = 4, WN = NW == 4 ? 4 : 2, BM = 256, BN = 256;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int per_xcd = gridDim.x / 8;
   const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;   // neighbours in an XCD share weight tiles
@@ -373,7 +376,7 @@ __global__ __launch_bounds__(256) void gemm_dma256_kernel(const bf16_t* __restri
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
+  const int wm0 = (wave / WCOLS) * 128, wn0 = (wave % WCOLS) * 32 * WN;
   const int r = lane & 31, g = lane >> 5;
 
   f32x16 acc[WM][WN];
@@ -384,30 +387,30 @@ __global__ __launch_bounds__(256) void gemm_dma256_kernel(const bf16_t* __restri
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // what this lane copies per k-tile: its slot of A blocks 4 wave .. 4 wave + 3 and of W blocks likewise.
+  // what this lane copies per k-tile: its slot of A blocks CB wave .. CB wave + CB - 1 and of W blocks likewise.
   // Rows past M and blocks past N are clamped to the last valid one (their products are never stored).
   const int k_tiles = K / 32;
   const int n_blocks_w = (N + 15) / 16;
-  const bf16_t* a_src[4];
+  const bf16_t* a_src[4];                                  // (CB of them are used)
   const bf16_t* w_src[4];
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
+  for (int b = 0; b < CB; ++b) {
     // slot l of an A block holds row l / 4, chunk (l % 4) ^ (row / 4 % 4): four neighbouring lanes fetch
     // 64 consecutive bytes, and 16 rows of one chunk lie in 16 different 16-byte columns of LDS
     const int row16 = lane >> 2, chunk = (lane & 3) ^ ((row16 >> 2) & 3);
-    const int row = min(m0 + (4 * wave + b) * 16 + row16, M - 1);
+    const int row = min(m0 + (CB * wave + b) * 16 + row16, M - 1);
     a_src[b] = A + (size_t)row * lda + chunk * 8;
-    const int blk = min(n0 / 16 + 4 * wave + b, n_blocks_w - 1);
+    const int blk = min(n0 / 16 + CB * wave + b, n_blocks_w - 1);
     w_src[b] = W + (size_t)blk * k_steps * 512 + lane * 8;
   }
   auto copy_tile = [&](int kt_v) {
     const int kt = min(kt_v, k_tiles - 1);               // past the end: a copy nobody reads
-    char* stage = lds + (kt_v % TW_DMA_STAGES) * TW_DMA_STAGE + wave * 4096;
+    char* stage = lds + (kt_v % TW_DMA_STAGES) * TW_DMA_STAGE + wave * CB * 1024;
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
+    for (int b = 0; b < CB; ++b)
       __builtin_amdgcn_global_load_lds(a_src[b] + (size_t)kt * 32, (tw_lds_ptr)(stage + b * 1024), 16, 0, 0);
 #pragma unroll
-    for (int b = 0; b < 4; ++b)
+    for (int b = 0; b < CB; ++b)
       __builtin_amdgcn_global_load_lds(w_src[b] + (size_t)kt * 512, (tw_lds_ptr)(stage + 16384 + b * 1024), 16, 0, 0);
   };
   // this lane's fragment addresses in stage 0: row block, then chunk 2 cc + g, then row
@@ -429,22 +432,19 @@ __global__ __launch_bounds__(256) void gemm_dma256_kernel(const bf16_t* __restri
       for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[i], wf[j]);
   };
   // wait until at most `n` of this wave's copies are in flight (they finish in order), then meet the others
-#define TW_DMA_PUBLISH(n)                                                     \
+  // (a wave has 2 CB copies per k-tile: n4 is the count for 4 waves, n8 for 8)
+#define TW_DMA_PUBLISH(n4, n8)                                                \
   do {                                                                        \
-    asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)" ::: "memory");          \
+    if constexpr (NW == 4) asm volatile("s_waitcnt vmcnt(" #n4 ") lgkmcnt(0)" ::: "memory"); \
+    else asm volatile("s_waitcnt vmcnt(" #n8 ") lgkmcnt(0)" ::: "memory");    \
     __builtin_amdgcn_s_barrier();                                             \
     asm volatile("" ::: "memory");                                            \
   } while (0)
 #define TW_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 
   bf16x8 af[2][WM], wf[2][WN];
-#if TW_DMA_STAGES == 4
-#define TW_DMA_PUBLISH_FIRST() TW_DMA_PUBLISH(24)
-#define TW_DMA_PUBLISH_REST() TW_DMA_PUBLISH(16)
-#else
-#define TW_DMA_PUBLISH_FIRST() TW_DMA_PUBLISH(32)
-#define TW_DMA_PUBLISH_REST() TW_DMA_PUBLISH(24)
-#endif
+#define TW_DMA_PUBLISH_FIRST() TW_DMA_PUBLISH(24, 12)     /* three k-tiles of copies may be in flight */
+#define TW_DMA_PUBLISH_REST() TW_DMA_PUBLISH(16, 8)       /* two */
 #pragma unroll
   for (int t = 0; t < TW_DMA_STAGES; ++t) copy_tile(t);
   TW_DMA_PUBLISH_FIRST();                                  // k-tile 0 has landed, for every wave
@@ -452,20 +452,30 @@ __global__ __launch_bounds__(256) void gemm_dma256_kernel(const bf16_t* __restri
   for (int kt = 0; kt < k_tiles; ++kt) {
     read_frags(kt, 1, af[1], wf[1]);
     multiply(af[0], wf[0]);
-    TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
-    TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+    if constexpr (NW == 4) {
+      TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+      TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+    } else {
+      TW_SGB(0x100, 3); TW_SGB(0x008, 4); TW_SGB(0x100, 3); TW_SGB(0x008, 4);
+    }
     // every fragment of k-tile kt is in registers now; k-tile kt + 1 (copies of kt + 2 and kt + 3
     // may still be in flight) becomes visible, and kt's stage is free for kt + 4
     TW_DMA_PUBLISH_REST();
     copy_tile(kt + TW_DMA_STAGES);
     read_frags(kt + 1, 0, af[0], wf[0]);                   // (after the last k-tile: read, never used)
     multiply(af[1], wf[1]);
-    TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
-    TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+    if constexpr (NW == 4) {
+      TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+      TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
+    } else {
+      TW_SGB(0x020, 2); TW_SGB(0x100, 3); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 3); TW_SGB(0x008, 4);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // no copy may land in the epilogue's staging area
 #undef TW_SGB
 #undef TW_DMA_PUBLISH
+#undef TW_DMA_PUBLISH_FIRST
+#undef TW_DMA_PUBLISH_REST
   tw_tiled_epilogue<OutT, WM, WN, GLU>(acc, lds, bias, residual, ldr, C, ldc, M, N, m0, n0, wm0, wn0, wave, lane);
 }
 
@@ -531,7 +541,7 @@ static int launch_dma256(const bf16_t* A, long lda, const bf16_t* W, long ldw, c
   TW_REQUIRE(n_blocks < (1L << 30));
   const int grid = (int)((n_blocks + 7) / 8 * 8);
   const size_t lds_bytes = TW_DMA_STAGES * TW_DMA_STAGE;          // also covers the epilogue's staging area
-  auto kernel = gemm_dma256_kernel<OutT, GLU>;
+  auto kernel = gemm_dma256_kernel<OutT, GLU, TW_DMA_WAVES>;
   static bool attribute_set = false;   // per instantiation
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -539,7 +549,7 @@ static int launch_dma256(const bf16_t* A, long lda, const bf16_t* W, long ldw, c
     if (e != hipSuccess) return (int)e;
     attribute_set = true;
   }
-  kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m, (int)n_blocks);
+  kernel<<<grid, 64 * TW_DMA_WAVES, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m, (int)n_blocks);
   return TW_LAUNCH_RESULT();
 }
 
