@@ -331,52 +331,53 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 }
 
 // =====================================================================================
-// 256x256 tiles, bfloat16, shuffled weights, K a multiple of 32, with global memory copied
-// straight into LDS (`global_load_lds_dwordx4`: lane l's 16 bytes land at the wave's LDS base +
-// 16 l, from any address the lane names). No staging registers and no LDS write instructions.
+// bfloat16, shuffled weights, K a multiple of 32: tiles whose operands are copied from global
+// memory straight into LDS (`global_load_lds_dwordx4`: lane l's 16 bytes land at the wave's LDS
+// base + 16 l, from any address the lane names). No staging registers, no LDS write instructions.
+// Workgroup = 4 waves in a 2x2 grid, wave tile (32*WM) x (32*WN): 128x128 (two workgroups a CU),
+// 128x256, 256x256 (one a CU, the accumulators in AGPRs).
 //
 // A k-tile is 32 elements of K (64 bytes a row, one k-step of the shuffled layout). A stage of
-// LDS holds 16 blocks of A and 16 of W; a block is 16 rows x 4 chunks of 16 bytes in the order
-// [chunk][row], 1 KB, which is how W lies in memory (a fragment read takes 256 consecutive bytes
-// per 16 lanes); an A block is [row][chunk] with the chunks of a row swizzled (see a_src below).
-// Four stages: the copy of k-tile t+4 is started when k-tile t has been read into registers.
+// LDS holds the tile's blocks of A, then those of W; a block is 16 rows x 4 chunks of 16 bytes,
+// 1 KB. A W block is [chunk][row], which is how W lies in memory (a fragment read takes 256
+// consecutive bytes per 16 lanes); an A block is [row][chunk] with the chunks of a row swizzled
+// (see a_src below). Four stages: the copy of k-tile t+4 starts when k-tile t is in registers.
 //
-// Per k-tile and wave: 2 k-chunk pairs of 16 MFMAs (wave tile 128x128, accumulators in AGPRs).
-// The fragments of a pair are read while the pair before is multiplied, so the barrier that
-// publishes the next k-tile lies between the two pairs of this one and the matrix unit has
-// work on both sides of it.
+// Per k-tile and wave: 2 k-chunk pairs of WM*WN MFMAs. The fragments of a pair are read while the
+// pair before is multiplied, so the barrier that publishes the next k-tile lies between the two
+// pairs of this one and the matrix unit has work queued on both sides of it.
+// splits > 1: as in gemm_tiled_kernel.
 // =====================================================================================
 typedef __attribute__((address_space(3))) void* tw_lds_ptr;
-#define TW_DMA_STAGE 32768
 #define TW_DMA_STAGES 4
-#ifndef TW_DMA_WAVES
-#define TW_DMA_WAVES 4          /* 8 (two waves to a SIMD, 128x64 each) measured 2-5 % slower */
-#endif
 
-// NW waves in 2 rows: 4 waves with tiles of 128x128 each, or 8 with 128x64 (two to a SIMD).
-// WCOLS: waves side by side; CB: blocks of A, and of W, a wave copies per k-tile.
-template <typename OutT, bool GLU, int NW, int WCOLS = NW / 2, int CB = 16 / NW>
-__global__ __launch_bounds__(64 * NW) void gemm_dma256_kernel(const bf16_t* __restrict__ A, long lda,
-                                                          const bf16_t* __restrict__ W, long k_steps,
-                                                          const float* __restrict__ bias, const float* residual,
-                                                          long ldr, OutT* C, long ldc, int M, int N, int K,
-                                                          int tiles_m, int n_blocks) {
-  constexpr int WM = 4, WN = NW == 4 ? 4 : 2, BM = 256, BN = 256;
+template <typename OutT, int WM, int WN, bool GLU>
+__global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict__ A, long lda,
+                                                       const bf16_t* __restrict__ W, long k_steps,
+                                                       const float* __restrict__ bias, const float* residual,
+                                                       long ldr, OutT* C, long ldc, int M, int N, int K,
+                                                       int tiles_m, int n_blocks, int splits,
+                                                       float* __restrict__ partial) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int STAGE = (BM + BN) * 64;                 // bytes: A blocks, then W blocks
+  constexpr int COPIES = WM + WN;                       // 1 KB copies per wave and k-tile
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int per_xcd = gridDim.x / 8;
-  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;   // neighbours in an XCD share weight tiles
+  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;   // neighbours in an XCD share operand tiles
   if (logical >= n_blocks) return;
-  // Tiles in bands of 8 row tiles: the 32 workgroups an XCD runs at a time then cover 8 row tiles x 4
-  // column tiles and fetch 12 operand tiles between them (with all the row tiles of a tall matrix in
-  // one column they would fetch one per workgroup).
-  const int tiles_n = n_blocks / tiles_m;
-  const int band = logical / (8 * tiles_n), in_band = logical - band * 8 * tiles_n;
-  const int band_rows = min(8, tiles_m - band * 8);
-  const int tile_m = band * 8 + in_band % band_rows, tile_n = in_band / band_rows;
+  const int n_tiles = n_blocks / splits;
+  const int split = logical / n_tiles, tile = logical % n_tiles;
+  // Tiles in bands of 2,048 rows: the workgroups an XCD runs at a time then share column tiles as well
+  // as row tiles (all the row tiles of a tall matrix in one column would fetch an activation tile each).
+  constexpr int BAND = 2048 / BM;
+  const int tiles_n = n_tiles / tiles_m;
+  const int band = tile / (BAND * tiles_n), in_band = tile - band * BAND * tiles_n;
+  const int band_rows = min(BAND, tiles_m - band * BAND);
+  const int tile_m = band * BAND + in_band % band_rows, tile_n = in_band / band_rows;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave / WCOLS) * 128, wn0 = (wave % WCOLS) * 32 * WN;
+  const int wm0 = (wave >> 1) * 32 * WM, wn0 = (wave & 1) * 32 * WN;
   const int r = lane & 31, g = lane >> 5;
 
   f32x16 acc[WM][WN];
@@ -387,39 +388,50 @@ __global__ __launch_bounds__(64 * NW) void gemm_dma256_kernel(const bf16_t* __re
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // what this lane copies per k-tile: its slot of A blocks CB wave .. CB wave + CB - 1 and of W blocks likewise.
-  // Rows past M and blocks past N are clamped to the last valid one (their products are never stored).
-  const int k_tiles = K / 32;
+  // this workgroup's k-tiles: kt0 .. kt0 + k_tiles - 1
+  const int k_tiles_all = K / 32;
+  const int per_split = (k_tiles_all + splits - 1) / splits;
+  const int kt0 = split * per_split;
+  const int k_tiles = max(0, min(k_tiles_all, kt0 + per_split) - kt0);
+
+  // What this lane copies per k-tile: its slot of A blocks WM wave .. WM wave + WM - 1 and of W blocks
+  // WN wave .. WN wave + WN - 1. Rows past M and blocks past N are clamped to the last valid one (their
+  // products are never stored).
   const int n_blocks_w = (N + 15) / 16;
-  const bf16_t* a_src[4];                                  // (CB of them are used)
-  const bf16_t* w_src[4];
-#pragma unroll
-  for (int b = 0; b < CB; ++b) {
+  const bf16_t* a_src[4];                                  // (WM of them are used)
+  const bf16_t* w_src[4];                                  // (WN)
+  {
     // slot l of an A block holds row l / 4, chunk (l % 4) ^ (row / 4 % 4): four neighbouring lanes fetch
     // 64 consecutive bytes, and 16 rows of one chunk lie in 16 different 16-byte columns of LDS
     const int row16 = lane >> 2, chunk = (lane & 3) ^ ((row16 >> 2) & 3);
-    const int row = min(m0 + (CB * wave + b) * 16 + row16, M - 1);
-    a_src[b] = A + (size_t)row * lda + chunk * 8;
-    const int blk = min(n0 / 16 + CB * wave + b, n_blocks_w - 1);
-    w_src[b] = W + (size_t)blk * k_steps * 512 + lane * 8;
+#pragma unroll
+    for (int b = 0; b < WM; ++b) {
+      const int row = min(m0 + (WM * wave + b) * 16 + row16, M - 1);
+      a_src[b] = A + (size_t)row * lda + (size_t)kt0 * 32 + chunk * 8;
+    }
+#pragma unroll
+    for (int b = 0; b < WN; ++b) {
+      const int blk = min(n0 / 16 + WN * wave + b, n_blocks_w - 1);
+      w_src[b] = W + ((size_t)blk * k_steps + kt0) * 512 + lane * 8;
+    }
   }
-  auto copy_tile = [&](int kt_v) {
-    const int kt = min(kt_v, k_tiles - 1);               // past the end: a copy nobody reads
-    char* stage = lds + (kt_v % TW_DMA_STAGES) * TW_DMA_STAGE + wave * CB * 1024;
+  auto copy_tile = [&](int t_v) {                          // k-tile kt0 + t_v into stage t_v % 4
+    const int t = min(t_v, k_tiles - 1);                   // past the end: a copy nobody reads
+    char* stage = lds + (t_v % TW_DMA_STAGES) * STAGE;
 #pragma unroll
-    for (int b = 0; b < CB; ++b)
-      __builtin_amdgcn_global_load_lds(a_src[b] + (size_t)kt * 32, (tw_lds_ptr)(stage + b * 1024), 16, 0, 0);
+    for (int b = 0; b < WM; ++b)
+      __builtin_amdgcn_global_load_lds(a_src[b] + (size_t)t * 32, (tw_lds_ptr)(stage + (WM * wave + b) * 1024), 16, 0, 0);
 #pragma unroll
-    for (int b = 0; b < CB; ++b)
-      __builtin_amdgcn_global_load_lds(w_src[b] + (size_t)kt * 512, (tw_lds_ptr)(stage + 16384 + b * 1024), 16, 0, 0);
+    for (int b = 0; b < WN; ++b)
+      __builtin_amdgcn_global_load_lds(w_src[b] + (size_t)t * 512, (tw_lds_ptr)(stage + BM * 64 + (WN * wave + b) * 1024), 16, 0, 0);
   };
-  // this lane's fragment addresses in stage 0: row block, then chunk 2 cc + g, then row
+  // this lane's fragment addresses in stage 0
   const int a_row16 = r & 15, a_swz = (a_row16 >> 2) & 3;
   const char* a_block = lds + (wm0 / 16 + (r >> 4)) * 1024 + a_row16 * 64;
   const char* a_frag_cc[2] = {a_block + ((g ^ a_swz) * 16), a_block + (((2 + g) ^ a_swz) * 16)};
-  const char* w_frag = lds + 16384 + (wn0 / 16 + (r >> 4)) * 1024 + g * 256 + (r & 15) * 16;
-  auto read_frags = [&](int kt, int cc, bf16x8* af, bf16x8* wf) {
-    const int st = (kt % TW_DMA_STAGES) * TW_DMA_STAGE;
+  const char* w_frag = lds + BM * 64 + (wn0 / 16 + (r >> 4)) * 1024 + g * 256 + (r & 15) * 16;
+  auto read_frags = [&](int t, int cc, bf16x8* af, bf16x8* wf) {
+    const int st = (t % TW_DMA_STAGES) * STAGE;
 #pragma unroll
     for (int i = 0; i < WM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(a_frag_cc[cc] + st + i * 2048);
 #pragma unroll
@@ -431,51 +443,54 @@ __global__ __launch_bounds__(64 * NW) void gemm_dma256_kernel(const bf16_t* __re
 #pragma unroll
       for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[i], wf[j]);
   };
-  // wait until at most `n` of this wave's copies are in flight (they finish in order), then meet the others
-  // (a wave has 2 CB copies per k-tile: n4 is the count for 4 waves, n8 for 8)
-#define TW_DMA_PUBLISH(n4, n8)                                                \
+  // Wait until at most `tiles` k-tiles of this wave's copies are in flight (copies finish in order), then
+  // meet the other waves. The count is an immediate of the instruction, hence the cases.
+#define TW_DMA_WAIT(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)" ::: "memory")
+#define TW_DMA_PUBLISH(tiles)                                                 \
   do {                                                                        \
-    if constexpr (NW == 4) asm volatile("s_waitcnt vmcnt(" #n4 ") lgkmcnt(0)" ::: "memory"); \
-    else asm volatile("s_waitcnt vmcnt(" #n8 ") lgkmcnt(0)" ::: "memory");    \
+    if constexpr (COPIES * (tiles) == 8) TW_DMA_WAIT(8);                      \
+    else if constexpr (COPIES * (tiles) == 12) TW_DMA_WAIT(12);               \
+    else if constexpr (COPIES * (tiles) == 16) TW_DMA_WAIT(16);               \
+    else if constexpr (COPIES * (tiles) == 18) TW_DMA_WAIT(18);               \
+    else if constexpr (COPIES * (tiles) == 24) TW_DMA_WAIT(24);               \
+    else TW_DMA_WAIT(0);                                                      \
     __builtin_amdgcn_s_barrier();                                             \
     asm volatile("" ::: "memory");                                            \
   } while (0)
 #define TW_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+  // the order asked of the scheduler: G groups of (copies, fragment reads, MFMAs) per k-chunk pair
+  constexpr int G = WM * WN >= 16 ? 4 : 2;
 
   bf16x8 af[2][WM], wf[2][WN];
-#define TW_DMA_PUBLISH_FIRST() TW_DMA_PUBLISH(24, 12)     /* three k-tiles of copies may be in flight */
-#define TW_DMA_PUBLISH_REST() TW_DMA_PUBLISH(16, 8)       /* two */
+  if (k_tiles > 0) {
 #pragma unroll
-  for (int t = 0; t < TW_DMA_STAGES; ++t) copy_tile(t);
-  TW_DMA_PUBLISH_FIRST();                                  // k-tile 0 has landed, for every wave
-  read_frags(0, 0, af[0], wf[0]);
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    read_frags(kt, 1, af[1], wf[1]);
-    multiply(af[0], wf[0]);
-    if constexpr (NW == 4) {
-      TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
-      TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
-    } else {
-      TW_SGB(0x100, 3); TW_SGB(0x008, 4); TW_SGB(0x100, 3); TW_SGB(0x008, 4);
-    }
-    // every fragment of k-tile kt is in registers now; k-tile kt + 1 (copies of kt + 2 and kt + 3
-    // may still be in flight) becomes visible, and kt's stage is free for kt + 4
-    TW_DMA_PUBLISH_REST();
-    copy_tile(kt + TW_DMA_STAGES);
-    read_frags(kt + 1, 0, af[0], wf[0]);                   // (after the last k-tile: read, never used)
-    multiply(af[1], wf[1]);
-    if constexpr (NW == 4) {
-      TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
-      TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 2); TW_SGB(0x008, 4);
-    } else {
-      TW_SGB(0x020, 2); TW_SGB(0x100, 3); TW_SGB(0x008, 4); TW_SGB(0x020, 2); TW_SGB(0x100, 3); TW_SGB(0x008, 4);
+    for (int t = 0; t < TW_DMA_STAGES; ++t) copy_tile(t);
+    TW_DMA_PUBLISH(3);                                     // k-tile 0 has landed, for every wave
+    read_frags(0, 0, af[0], wf[0]);
+    for (int t = 0; t < k_tiles; ++t) {
+      read_frags(t, 1, af[1], wf[1]);
+      multiply(af[0], wf[0]);
+#pragma unroll
+      for (int q = 0; q < G; ++q) { TW_SGB(0x100, (WM + WN) / G); TW_SGB(0x008, WM * WN / G); }
+      // every fragment of k-tile t is in registers now; k-tile t + 1 (copies of t + 2 and t + 3 may
+      // still be in flight) becomes visible, and t's stage is free for t + 4
+      TW_DMA_PUBLISH(2);
+      copy_tile(t + TW_DMA_STAGES);
+      read_frags(t + 1, 0, af[0], wf[0]);                  // (after the last k-tile: read, never used)
+      multiply(af[1], wf[1]);
+#pragma unroll
+      for (int q = 0; q < G; ++q) { TW_SGB(0x020, COPIES / G); TW_SGB(0x100, (WM + WN) / G); TW_SGB(0x008, WM * WN / G); }
     }
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // no copy may land in the epilogue's staging area
 #undef TW_SGB
 #undef TW_DMA_PUBLISH
-#undef TW_DMA_PUBLISH_FIRST
-#undef TW_DMA_PUBLISH_REST
+#undef TW_DMA_WAIT
+  if (splits > 1) {
+    tw_tiled_epilogue<float, WM, WN, false>(acc, lds, nullptr, nullptr, 0, partial + (size_t)split * M * N, (long)N,
+                                            M, N, m0, n0, wm0, wn0, wave, lane);
+    return;
+  }
   tw_tiled_epilogue<OutT, WM, WN, GLU>(acc, lds, bias, residual, ldr, C, ldc, M, N, m0, n0, wm0, wn0, wave, lane);
 }
 
@@ -531,17 +546,22 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
 }
 
 
-template <typename OutT, bool GLU>
-static int launch_dma256(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias,
-                         const float* residual, long ldr, OutT* C, long ldc, int M, int N, int K,
-                         hipStream_t stream) {
+template <typename OutT, int WM, int WN, bool GLU>
+static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias,
+                      const float* residual, long ldr, OutT* C, long ldc, float* partial, long partial_bytes,
+                      int M, int N, int K, hipStream_t stream) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
   TW_REQUIRE(K % 32 == 0 && K >= 32 && lda % 8 == 0);
-  const int tiles_m = tw_div_up(M, 256), tiles_n = tw_div_up(N, 256);
-  const long n_blocks = (long)tiles_m * tiles_n;
+  const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
+  int splits = GLU ? 1 : tiled_splits(M, N, K, 8, BM, BN);
+  if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4 || (uintptr_t)partial % 16 != 0)) splits = 1;
+  const long n_blocks = (long)tiles_m * tiles_n * splits;
   TW_REQUIRE(n_blocks < (1L << 30));
   const int grid = (int)((n_blocks + 7) / 8 * 8);
-  const size_t lds_bytes = TW_DMA_STAGES * TW_DMA_STAGE;          // also covers the epilogue's staging area
-  auto kernel = gemm_dma256_kernel<OutT, GLU, TW_DMA_WAVES>;
+  const size_t pipeline_bytes = TW_DMA_STAGES * (size_t)(BM + BN) * 64;
+  const size_t epilogue_bytes = 4 * 32 * (size_t)(32 * WN + 4) * 4;
+  const size_t lds_bytes = pipeline_bytes > epilogue_bytes ? pipeline_bytes : epilogue_bytes;
+  auto kernel = gemm_dma_kernel<OutT, WM, WN, GLU>;
   static bool attribute_set = false;   // per instantiation
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -549,13 +569,21 @@ static int launch_dma256(const bf16_t* A, long lda, const bf16_t* W, long ldw, c
     if (e != hipSuccess) return (int)e;
     attribute_set = true;
   }
-  kernel<<<grid, 64 * TW_DMA_WAVES, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m, (int)n_blocks);
+  kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m,
+                                           (int)n_blocks, splits, partial);
+  int err = TW_LAUNCH_RESULT();
+  if (err || splits == 1) return err;
+  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
+                                                                             ldr, C, ldc, M, N);
   return TW_LAUNCH_RESULT();
 }
 
 // Which tile: 256x256 when there are at least one and a half rounds of them for 256 CUs (per MFMA it moves half
 // the bytes through the 64 B/clk vector-memory path and the LDS that 128x128 does); 128x256 when that
 // makes one round that fills most of the chip; else 128x128, two workgroups per CU.
+#ifndef TW_DMA_SHAPES
+#define TW_DMA_SHAPES 0xC      /* bit s: shape s uses the direct-to-LDS kernel (at 128x128 it gains nothing) */
+#endif
 static int choose_shape(bool big_ok, int M, int N) {
   if (big_ok) {
     if ((long)tw_div_up(M, 256) * tw_div_up(N, 256) >= 384) return 3;
@@ -571,14 +599,20 @@ static int tiled_by_shape(int shape, const T* A, long lda, const T* W, long ldw,
                           long partial_bytes, int M, int N, int K, hipStream_t stream) {
   constexpr bool BIG = sizeof(T) == 2 && SHUF;
   if (shape == 0) shape = choose_shape(BIG, M, N);
-  if (shape == 3) {
-    if constexpr (BIG) {
-      if (K % 32 == 0)
-        return launch_dma256<OutT, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, stream);
-      return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+  if constexpr (BIG) {
+    // bfloat16 and shuffled weights: the kernels that copy straight into LDS, if K allows
+    if (K % 32 == 0 && K >= 32 && lda % 8 == 0) {
+      if constexpr ((TW_DMA_SHAPES & 8) != 0)
+        if (shape == 3) return launch_dma<OutT, 4, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+      if constexpr ((TW_DMA_SHAPES & 4) != 0)
+        if (shape == 2) return launch_dma<OutT, 2, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+      if constexpr ((TW_DMA_SHAPES & 2) != 0)
+        if (shape == 1) return launch_dma<OutT, 2, 2, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
     }
-    return TW_ERR_BAD_ARGUMENT;
+    if (shape == 3)
+      return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
+  if (shape == 3) return TW_ERR_BAD_ARGUMENT;
   if (shape == 2)
     return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
