@@ -94,7 +94,7 @@ __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restri
     // chain of memory latencies): the row itself, the weight, and the partial sums 8 at a time.
     // The partial sums are still added one after the other in index order, then the row.
     const f32x4 xv = *reinterpret_cast<const f32x4*>(src + h);
-    wv = *reinterpret_cast<const f32x4*>(w + h);
+    if (add) wv = *reinterpret_cast<const f32x4*>(w + h);      // (few rows; with many, the weight is read below)
     if (add) {
       const float* p = add + (size_t)r * hidden + h;
       for (int s0 = 0; s0 < add_splits; s0 += 8) {
@@ -117,6 +117,7 @@ __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restri
   ss = tw_block_sum(ss, lds);
   const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
   if (mine) {
+    if (!add) wv = *reinterpret_cast<const f32x4*>(w + h);
     T* dst = out + (size_t)o * hidden + h;
     T packed[4];
 #pragma unroll
