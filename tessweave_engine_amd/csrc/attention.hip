@@ -57,7 +57,8 @@ struct AttnArgs {
   float scale;
   int splits;
   int page_shift;         // log2(page_size) if it is a power of two, else -1
-  int n_seqs, max_tiles;  // prefill (bfloat16 kernel): sequences of the launch, 128-row tiles of the longest
+  int n_seqs, max_tiles;  // prefill (bfloat16 kernel): sequences of the launch, row tiles of the longest
+  int tile_rows;          // rows of such a tile: 128, or 64 when there would be too few workgroups
   int kv_chunk, max_chunks;  // prefill (bfloat16 kernel): keys per workgroup (a multiple of 32) and the most
                              // chunks a tile can have; max_chunks == 1: a tile's keys are never split
 };
@@ -617,7 +618,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 
 // =====================================================================================
 // Prefill, bfloat16, pages of 8 keys or a power of two above: a workgroup of 4
-// waves owns 128 consecutive (token, head) rows of one kv head, 32 per wave. The
+// waves owns 128 (or 64) consecutive (token, head) rows of one kv head, 32 (16) per wave. The
 // keys and values of each 32-key block are copied ONCE per workgroup into LDS
 // (keys outside the sequence as zeros) while the block before is computed; every
 // K or V fragment a wave reads from LDS serves both of its 16-row tiles.
@@ -628,8 +629,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 
 // EXACT: head_dim == 16 * DTMAX, so every loop over the head has compile-time bounds (with run-time
 // bounds the compiler indexes the accumulators dynamically, several instructions per MFMA).
-template <int DTMAX, bool EXACT>
+template <int DTMAX, bool EXACT, int RT>
 __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
+  constexpr int TR = 64 * RT;                           // rows of a workgroup's tile: RT tiles of 16 per wave
   constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
   constexpr int KROW = DTMAX * 32 + 16;                 // LDS bytes per key row, padded
   constexpr int KSTAGE = 32 * KROW, VSTAGE = DTMAX * 16 * TW_PF_VROW;
@@ -673,10 +675,10 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const int token0 = a.q_start[seq];
   const int q_len = a.q_start[seq + 1] - token0;
   const int rows = q_len * G;
-  const int n_tiles = (rows + 127) / 128;
+  const int n_tiles = (rows + TR - 1) / TR;
   const int tile_idx = a.max_tiles - 1 - tile_from_end;         // counted from the longest sequence's last tile
   if (tile_idx < 0 || tile_idx >= n_tiles) return;
-  const int wg_row0 = tile_idx * 128;
+  const int wg_row0 = tile_idx * TR;
   const int* table = a.block_table + (size_t)seq * a.table_stride;
   const int D = EXACT ? DTMAX * 16 : a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
   const int pshift = a.page_shift, pmask = P - 1;
@@ -689,12 +691,12 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const float c2 = a.scale * 1.44269504088896340736f;    // scores are kept in the log2 domain
 
   // ---- this wave's two row tiles -----------------------------------------------
-  bf16x8 qf[2][NSMAX];
-  int t_row[2], tok[2], head[2];
-  bool row_ok[2];
+  bf16x8 qf[RT][NSMAX];
+  int t_row[RT], tok[RT], head[RT];
+  bool row_ok[RT];
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
-    const int row = wg_row0 + wave * 32 + rt * 16 + r;
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = wg_row0 + wave * 16 * RT + rt * 16 + r;
     row_ok[rt] = row < rows;
     tok[rt] = row / G;
     head[rt] = kvh * G + row % G;
@@ -706,16 +708,19 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       qf[rt][st] = (row_ok[rt] && (EXACT || chunk < chunks)) ? tw_load_frag(q_row + chunk * 8) : Elem<bf16_t>::zero();
     }
   }
-  f32x4 acc[2][DTMAX];
-  float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+  f32x4 acc[RT][DTMAX];
+  float m[RT], l[RT];
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt)
+  for (int rt = 0; rt < RT; ++rt) {
+    m[rt] = -INFINITY;
+    l[rt] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt) acc[rt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   // ---- the workgroup's key range ------------------------------------------------
   const int t_min = first_pos + wg_row0 / G;
-  const int t_max = first_pos + min(rows - 1, wg_row0 + 127) / G;
+  const int t_max = first_pos + min(rows - 1, wg_row0 + TR - 1) / G;
   const int lo = a.window > 0 ? max(0, t_min - a.window + 1) : 0;       // keys below are never loaded
   // The tile's key blocks, and the share of them this workgroup takes. A tile split into several
   // chunks leaves float32 partial results (running maximum, sum, output) that a second kernel merges.
@@ -724,10 +729,10 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const int n_chunks = (tile_end - tile_begin + chunk_blocks - 1) / chunk_blocks;
   if (chunk >= n_chunks) return;
   const int blk_begin = tile_begin + chunk * chunk_blocks, blk_end = min(tile_end, blk_begin + chunk_blocks);
-  const int wave_t_max = first_pos + min(rows - 1, wg_row0 + wave * 32 + 31) / G;
-  const int wave_t_min = first_pos + min(rows - 1, wg_row0 + wave * 32) / G;
-  const bool wave_live = wg_row0 + wave * 32 < rows;
-  const bool wave_full = wg_row0 + wave * 32 + 32 <= rows;
+  const int wave_t_max = first_pos + min(rows - 1, wg_row0 + wave * 16 * RT + 16 * RT - 1) / G;
+  const int wave_t_min = first_pos + min(rows - 1, wg_row0 + wave * 16 * RT) / G;
+  const bool wave_live = wg_row0 + wave * 16 * RT < rows;
+  const bool wave_full = wg_row0 + wave * 16 * RT + 16 * RT <= rows;
   const int wave_lo_max = a.window > 0 ? wave_t_max - a.window + 1 : 0;  // largest lower bound among the wave's rows
 
   // This thread's share of a block, fixed for the whole loop: K piece i is 16 bytes
@@ -823,9 +828,9 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   // The branch covers the masking alone, so the two cases share every register of the rest.
   auto compute = [&](int blk, int buf, bool edge) {
     const int p0 = blk * 32;
-    f32x4 s[2][2];
+    f32x4 s[RT][2];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int tile = 0; tile < 2; ++tile) s[rt][tile] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -836,13 +841,13 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         if (EXACT || st * 4 < chunks) {
           bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + st * 64);
           if (!whole_chunks && st * 4 + g >= chunks) kf = Elem<bf16_t>::zero();
-          tw_mma16(s[0][tile], kf, qf[0][st]);
-          tw_mma16(s[1][tile], kf, qf[1][st]);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) tw_mma16(s[rt][tile], kf, qf[rt][st]);
         }
     }
     if (edge) {
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt) {
+      for (int rt = 0; rt < RT; ++rt) {
         const int lo_row = a.window > 0 ? t_row[rt] - a.window + 1 : 0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -851,10 +856,10 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         }
       }
     }
-    bf16x8 pb[2];
-    float alpha[2];
+    bf16x8 pb[RT];
+    float alpha[RT];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < RT; ++rt) {
       float mx = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[rt][e >> 2][e & 3]);
@@ -877,10 +882,13 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       m[rt] = m_new;
     }
     // rescale the running output only if some row's maximum moved
-    const bool moved = __any(alpha[0] != 1.f || alpha[1] != 1.f);
+    bool changed = false;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) changed = changed || alpha[rt] != 1.f;
+    const bool moved = __any(changed);
     if (moved) {
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
+      for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int dt = 0; dt < DTMAX; ++dt)
 #pragma unroll
@@ -891,8 +899,8 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     for (int dt = 0; dt < DTMAX; ++dt)
       if (EXACT || dt < dts) {
         const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
-        tw_mma16(acc[0][dt], vf, pb[0]);
-        tw_mma16(acc[1][dt], vf, pb[1]);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) tw_mma16(acc[rt][dt], vf, pb[rt]);
       }
   };
   auto compute_if_seen = [&](int blk, int buf) {
@@ -916,7 +924,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
 
   if (n_chunks > 1) {
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < RT; ++rt) {
       if (!row_ok[rt]) continue;
       const size_t slot = ((size_t)(token0 + tok[rt]) * a.q_heads + head[rt]) * a.max_chunks + chunk;
       float* dst = a.part_o + slot * D;
@@ -933,7 +941,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     return;
   }
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
+  for (int rt = 0; rt < RT; ++rt) {
     if (!row_ok[rt]) continue;
     const float inv = l[rt] > 0.f ? 1.f / l[rt] : 0.f;
     bf16_t* dst = (bf16_t*)a.out + (size_t)(token0 + tok[rt]) * a.ldo + (size_t)head[rt] * D;
@@ -960,10 +968,10 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnArgs a) {
   const int item = threadIdx.x;                                  // 32 threads per row
   const int row = blockIdx.x * TW_MERGE_ROWS + (item >> 5);
   if (row >= rows) return;
-  const int wg_row0 = row / 128 * 128;
+  const int wg_row0 = row / a.tile_rows * a.tile_rows;
   const int first_pos = kv_len - q_len;
   const int t_min = first_pos + wg_row0 / G;
-  const int t_max = first_pos + min(rows - 1, wg_row0 + 127) / G;
+  const int t_max = first_pos + min(rows - 1, wg_row0 + a.tile_rows - 1) / G;
   const int lo = a.window > 0 ? max(0, t_min - a.window + 1) : 0;
   const int tile_begin = lo / 32, tile_end = t_max / 32 + 1;
   const int chunk_blocks = a.kv_chunk / 32;
@@ -997,11 +1005,24 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnArgs a) {
 // How the keys of a prefill tile are split over workgroups: returns the most chunks a tile can
 // have (1: no splitting) and the keys per chunk. With fewer tiles than the chip has room for,
 // long tiles are cut so that there are about a thousand units of work of similar size.
-extern "C" int tw_attn_prefill_split(int n_seqs, int q_heads, int kv_heads, int max_q_len, int max_kv_len,
-                                     int* kv_chunk) {
-  const int split_below = 256;                     // one tile per CU or more: tiles are left whole (measured)
+// Rows of a workgroup's tile in the bfloat16 prefill kernel: 128 (32 per wave), or 64 (16 per wave)
+// when 128 would leave the chip with few workgroups: the kernel's time is a chain of latencies
+// (fragment reads, MFMAs, the softmax's dependent steps), and more waves hide more of it.
+static int prefill_tile_rows(int n_seqs, int q_heads, int kv_heads, int max_q_len, int asked) {
+  if (asked == 64 || asked == 128) return asked;
   const int G = kv_heads > 0 ? q_heads / kv_heads : 1;
   const long tiles = (long)tw_div_up((long)max_q_len * G, 128) * kv_heads * n_seqs;
+  return tiles < 640 ? 64 : 128;                    // (2,048 tokens of 28 heads: 64 is 16 % faster; 4,096: 10 % slower)
+}
+
+// tile_rows: 0 (choose), 64 or 128; *tile_rows_out is the choice, to be given to tw_attn_prefill.
+extern "C" int tw_attn_prefill_split(int n_seqs, int q_heads, int kv_heads, int max_q_len, int max_kv_len,
+                                     int tile_rows_in, int* kv_chunk, int* tile_rows_out) {
+  const int split_below = 256;                     // one tile per CU or more: tiles are left whole (measured)
+  const int G = kv_heads > 0 ? q_heads / kv_heads : 1;
+  const int tile_rows = prefill_tile_rows(n_seqs, q_heads, kv_heads, max_q_len, tile_rows_in);
+  *tile_rows_out = tile_rows;
+  const long tiles = (long)tw_div_up((long)max_q_len * G, tile_rows) * kv_heads * n_seqs;
   *kv_chunk = 0;
   if (tiles <= 0 || tiles >= split_below || max_kv_len <= 512) return 1;
   int want = (int)tw_div_up(1024, tiles);
@@ -1023,19 +1044,26 @@ static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_
   const int G = a.q_heads / a.kv_heads;
   const long rows = (long)max_q_len * G;
   a.n_seqs = n_seqs;
-  a.max_tiles = (int)tw_div_up(rows, 128);
+  a.tile_rows = prefill_tile_rows(n_seqs, a.q_heads, a.kv_heads, max_q_len, a.tile_rows);
+  a.max_tiles = (int)tw_div_up(rows, a.tile_rows);
   const long total = (long)a.max_tiles * a.kv_heads * n_seqs * a.max_chunks;
   TW_REQUIRE(total < (1L << 30));
   dim3 grid((unsigned)total);
   const size_t lds_bytes = 2 * 32 * (DTMAX * 32 + 16) + 2 * DTMAX * 16 * TW_PF_VROW;
-  auto kernel = attn_prefill_bf16_kernel<DTMAX, EXACT>;
   static bool attribute_set = false;
   if (!attribute_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<DTMAX, EXACT, 1>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<DTMAX, EXACT, 2>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (e != hipSuccess) return (int)e;
     attribute_set = true;
   }
-  kernel<<<grid, 256, lds_bytes, stream>>>(a);
+  if (a.tile_rows == 64)
+    attn_prefill_bf16_kernel<DTMAX, EXACT, 1><<<grid, 256, lds_bytes, stream>>>(a);
+  else
+    attn_prefill_bf16_kernel<DTMAX, EXACT, 2><<<grid, 256, lds_bytes, stream>>>(a);
   int err = TW_LAUNCH_RESULT();
   if (err || a.max_chunks <= 1) return err;
   attn_prefill_merge_kernel<<<dim3((unsigned)tw_div_up(rows, TW_MERGE_ROWS), a.kv_heads, n_seqs), 256, 0, stream>>>(a);
@@ -1160,9 +1188,11 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
                                const int* block_table, int table_stride, const int* q_start,
                                const int* kv_len, int seq0, int n_seqs, int max_q_len, void* out,
                                long ldo, float* workspace, long workspace_floats, int n_tokens, int max_chunks,
-                               int kv_chunk, int q_heads, int kv_heads, int head_dim, int page_size,
+                               int kv_chunk, int tile_rows, int q_heads, int kv_heads, int head_dim, int page_size,
                                int window, float scale, int generic, hipStream_t stream) {
   AttnArgs a;
+  TW_REQUIRE(tile_rows == 0 || tile_rows == 64 || tile_rows == 128);
+  a.tile_rows = tile_rows;
   a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
   a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;

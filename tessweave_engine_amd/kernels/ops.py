@@ -340,14 +340,15 @@ def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out
     return out
 
 
-def attn_prefill_split(n_seqs, q_heads, kv_heads, max_q_len, max_kv_len):
-    """(max_chunks, kv_chunk): how the fast prefill kernel would cut the keys of a tile into chunks that
-    separate workgroups take (max_chunks == 1: not at all) for a launch of this shape."""
+def attn_prefill_split(n_seqs, q_heads, kv_heads, max_q_len, max_kv_len, tile_rows=0):
+    """(max_chunks, kv_chunk, tile_rows): how the fast prefill kernel would cut the keys of a tile into
+    chunks that separate workgroups take (max_chunks == 1: not at all) for a launch of this shape, and the
+    rows of a workgroup's tile it would use (tile_rows 64 or 128 asks for that size)."""
     import ctypes
-    chunk = ctypes.c_int(0)
+    chunk, rows = ctypes.c_int(0), ctypes.c_int(0)
     chunks = int(library().tw_attn_prefill_split(int(n_seqs), q_heads, kv_heads, int(max_q_len), int(max_kv_len),
-                                                 ctypes.byref(chunk)))
-    return chunks, int(chunk.value)
+                                                 int(tile_rows), ctypes.byref(chunk), ctypes.byref(rows)))
+    return chunks, int(chunk.value), int(rows.value)
 
 
 def attn_prefill_workspace_floats(n_tokens, q_heads, head_dim, max_chunks):
@@ -358,13 +359,14 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
                  kv_heads, head_dim, scale, window=0, generic=False, split=None, workspace=None):
     """Attention of sequences seq0..seq0+n_seqs-1 with up to max_q_len query tokens each.
 
-    split = (max_chunks, kv_chunk) from attn_prefill_split with a float32 workspace of
+    split = (max_chunks, kv_chunk[, tile_rows]) from attn_prefill_split with a float32 workspace of
     attn_prefill_workspace_floats(rows of q, ...) lets the fast bfloat16 kernel cut long key ranges
     into chunks for separate workgroups (a second kernel merges them in a fixed order).
     """
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
     max_chunks, kv_chunk, ws_ptr, ws_floats = 1, 0, None, 0
+    tile_rows = int(split[2]) if split is not None and len(split) > 2 else 0
     if split is not None and split[0] > 1:
         max_chunks, kv_chunk = int(split[0]), int(split[1])
         _need(workspace is not None and workspace.dtype == torch.float32, "split prefill attention needs a float32 workspace")
@@ -373,7 +375,7 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
                                     _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
                                     _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
                                     seq0, n_seqs, int(max_q_len), _dev(out), ldo, ws_ptr, ws_floats, q.shape[0],
-                                    max_chunks, kv_chunk, q_heads, kv_heads, head_dim,
+                                    max_chunks, kv_chunk, tile_rows, q_heads, kv_heads, head_dim,
                                     keys.shape[2], int(window or 0), float(scale), 1 if generic else 0,
                                     _stream()), "attn_prefill")
     return out

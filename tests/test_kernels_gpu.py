@@ -357,10 +357,12 @@ def test_attn_prefill_portions(ops, device, dtype, heads, kv_heads, head_dim, pa
     # q lives inside a wider qkv buffer
     buf = torch.zeros(total_q, (heads + 2 * kv_heads) * head_dim, dtype=dtype, device=device)
     buf[:, :heads * head_dim] = q.reshape(total_q, -1).to(device)
-    # also with every tile's keys cut into chunks of 32 or 64 for separate workgroups (fast kernel only)
-    for generic, chunk in ((False, 0), (True, 0), (False, 32), (False, 64)):
+    # also with every tile's keys cut into chunks of 32 or 64 for separate workgroups, and with tiles of 64
+    # and of 128 rows (fast kernel only)
+    for generic, chunk, tile_rows in ((False, 0, 0), (True, 0, 0), (False, 32, 64), (False, 64, 128), (False, 0, 64),
+                                      (False, 0, 128)):
         out = torch.full((total_q, heads * head_dim), float("nan"), dtype=dtype, device=device)
-        split = (math.ceil((max(lengths) + 31) / chunk) + 1, chunk) if chunk else None
+        split = (math.ceil((max(lengths) + 31) / chunk) + 1 if chunk else 1, chunk, tile_rows)
         ws = torch.full((ops.attn_prefill_workspace_floats(total_q, heads, head_dim, split[0]),), float("nan"),
                         device=device) if chunk else None
         ops.attn_prefill(buf, keys, values, table, torch.tensor(q_start, dtype=torch.int32, device=device),
@@ -436,9 +438,9 @@ def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
     q = q_one[None].expand(q_len, heads, d).contiguous()
     want = plain.attention(q.float(), k, v, torch.arange(n - q_len, n), window=window or None)
     q_start = torch.tensor([0, q_len], dtype=torch.int32, device=device)
-    for generic, chunk in ((False, 0), (True, 0), (False, 32), (False, 96)):
+    for generic, chunk, tile_rows in ((False, 0, 64), (False, 0, 128), (True, 0, 0), (False, 32, 128), (False, 96, 64)):
         out = torch.full((q_len, heads * d), float("nan"), dtype=dtype, device=device)
-        split = (math.ceil((n + 31) / chunk) + 1, chunk) if chunk else None
+        split = (math.ceil((n + 31) / chunk) + 1 if chunk else 1, chunk, tile_rows)
         ws = torch.full((ops.attn_prefill_workspace_floats(q_len, heads, d, split[0]),), float("nan"),
                         device=device) if chunk else None
         ops.attn_prefill(q.reshape(q_len, -1).to(device), keys, values, table, q_start, kv_len, 0, 1, q_len, out, heads, 1,
