@@ -665,12 +665,14 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     rank = r * 8 + xcd;
     if (rank >= total) rank = b;                                 // (uneven XCD shares: keep every tile covered)
   }
-  const int chunk = rank % a.max_chunks;
+  // (the divisions run on the vector unit; what they give is the same for every lane, and saying so
+  // keeps the block-table lookups and page addresses of the loop below on the scalar unit)
+  const int chunk = __builtin_amdgcn_readfirstlane(rank % a.max_chunks);
   rank /= a.max_chunks;
   const int per_tile = a.kv_heads * a.n_seqs;
-  const int tile_from_end = rank / per_tile, sub = rank % per_tile;
-  const int kvh = sub % a.kv_heads;
-  const int seq = a.seq0 + sub / a.kv_heads;
+  const int tile_from_end = __builtin_amdgcn_readfirstlane(rank / per_tile), sub = rank % per_tile;
+  const int kvh = __builtin_amdgcn_readfirstlane(sub % a.kv_heads);
+  const int seq = __builtin_amdgcn_readfirstlane(a.seq0 + sub / a.kv_heads);
   const int kv_len = a.kv_len[seq];
   const int token0 = a.q_start[seq];
   const int q_len = a.q_start[seq + 1] - token0;
@@ -682,7 +684,6 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const int* table = a.block_table + (size_t)seq * a.table_stride;
   const int D = EXACT ? DTMAX * 16 : a.head_dim, dts = D / 16, chunks = D / 8, P = a.page_size;
   const int pshift = a.page_shift, pmask = P - 1;
-  const int ppb = P >= 32 ? 1 : (32 >> pshift);
   const unsigned head_stride = (unsigned)P * D;
   const bf16_t* keys = (const bf16_t*)a.keys;
   const bf16_t* values = (const bf16_t*)a.values;
@@ -765,39 +766,45 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   // address lies inside the pool; what such keys hold never counts (their scores are selected
   // to -inf) except in the PV product, so their VALUES are made zero here, in the rare block
   // that crosses the end of the sequence or the start of the window.
-  auto fetch = [&](int blk_v) {
+  // Each lane looks up the pages of its own pieces in the block table, one block ahead of the
+  // fetch (all four waves doing the same table arithmetic on the CU's one scalar unit was what
+  // bounded this kernel).
+  int k_pg[KPIECES], v_pg[VPIECES];
+  auto lookup = [&](int blk_v) {
+    const int blk = __builtin_amdgcn_readfirstlane(min(blk_v, blk_end - 1));
+    const int p0 = blk * 32;
+    const int* entry = table + (p0 >> pshift);
+    if (p0 >= lo && p0 + 32 <= kv_len) {                     // every key of the block counts: the common case
+#pragma unroll
+      for (int i = 0; i < KPIECES; ++i) k_pg[i] = entry[k_slot[i]];
+#pragma unroll
+      for (int i = 0; i < VPIECES; ++i) v_pg[i] = entry[v_slot[i]];
+    } else {
+      const int safe = P >= 32 ? 0 : ((max(lo, p0) - p0) >> pshift);   // a page of the block that is held
+      auto held = [&](int slot) {
+        const int a0 = P >= 32 ? p0 : p0 + (slot << pshift);
+        const int a1 = P >= 32 ? p0 + 31 : a0 + P - 1;
+        return (a0 < kv_len && a1 >= lo) ? slot : safe;
+      };
+#pragma unroll
+      for (int i = 0; i < KPIECES; ++i) k_pg[i] = entry[held(k_slot[i])];
+#pragma unroll
+      for (int i = 0; i < VPIECES; ++i) v_pg[i] = entry[held(v_slot[i])];
+    }
+  };
+  const size_t head_off = (size_t)kvh * head_stride;
+  const size_t page_stride = (size_t)a.kv_heads * head_stride;
+  auto fetch = [&](int blk_v) {                              // (after lookup of the same block)
     const int blk = __builtin_amdgcn_readfirstlane(blk_v);
     const int p0 = blk * 32;
-    const int first = p0 >> pshift;
-    int pg[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int a0 = P >= 32 ? p0 : p0 + (i << pshift);
-      const int a1 = P >= 32 ? p0 + 31 : a0 + P - 1;
-      pg[i] = (i < ppb && a0 < kv_len && a1 >= lo) ? table[first + i] : -1;
-    }
-    int safe = pg[0] >= 0 ? pg[0] : (pg[1] >= 0 ? pg[1] : (pg[2] >= 0 ? pg[2] : pg[3]));
-    if (safe < 0) safe = 0;
     const int in_page = P >= 32 ? (p0 & pmask) : 0;          // where the block starts inside its page
-    size_t kb[4], vb[4];
+    const size_t k_in = head_off + (size_t)in_page * D, v_in = head_off + in_page;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const size_t base = ((size_t)(pg[i] >= 0 ? pg[i] : safe) * a.kv_heads + kvh) * head_stride;
-      kb[i] = base + (size_t)in_page * D;
-      vb[i] = base + in_page;
-    }
+    for (int i = 0; i < KPIECES; ++i)
+      kreg[i] = tw_load_frag(keys + ((size_t)k_pg[i] * page_stride + k_in + k_goff[i]));
 #pragma unroll
-    for (int i = 0; i < KPIECES; ++i) {
-      const int sl = k_slot[i];
-      const size_t base = sl == 0 ? kb[0] : (sl == 1 ? kb[1] : (sl == 2 ? kb[2] : kb[3]));
-      kreg[i] = tw_load_frag(keys + base + k_goff[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < VPIECES; ++i) {
-      const int sl = v_slot[i];
-      const size_t base = sl == 0 ? vb[0] : (sl == 1 ? vb[1] : (sl == 2 ? vb[2] : vb[3]));
-      vreg[i] = tw_load_frag(values + base + v_goff[i]);
-    }
+    for (int i = 0; i < VPIECES; ++i)
+      vreg[i] = tw_load_frag(values + ((size_t)v_pg[i] * page_stride + v_in + v_goff[i]));
     if (p0 + 32 > kv_len || p0 < lo) {
 #pragma unroll
       for (int i = 0; i < VPIECES; ++i) {
@@ -833,18 +840,31 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int tile = 0; tile < 2; ++tile) s[rt][tile] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // every key fragment of the block is asked for before the first is multiplied, and the value
+    // fragments before the softmax, so that LDS latency passes behind other work
+    bf16x8 kf[2][NSMAX];
 #pragma unroll
     for (int tile = 0; tile < 2; ++tile) {
       const char* base = k_frag[tile] + buf * KSTAGE;
 #pragma unroll
       for (int st = 0; st < NSMAX; ++st)
         if (EXACT || st * 4 < chunks) {
-          bf16x8 kf = *reinterpret_cast<const bf16x8*>(base + st * 64);
-          if (!whole_chunks && st * 4 + g >= chunks) kf = Elem<bf16_t>::zero();
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) tw_mma16(s[rt][tile], kf, qf[rt][st]);
+          kf[tile][st] = *reinterpret_cast<const bf16x8*>(base + st * 64);
+          if (!whole_chunks && st * 4 + g >= chunks) kf[tile][st] = Elem<bf16_t>::zero();
         }
     }
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int st = 0; st < NSMAX; ++st)
+        if (EXACT || st * 4 < chunks)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) tw_mma16(s[rt][tile], kf[tile][st], qf[rt][st]);
+    const char* vbase = v_frag + buf * VSTAGE;
+    bf16x8 vf[DTMAX];
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (EXACT || dt < dts) vf[dt] = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
     if (edge) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
@@ -894,14 +914,11 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) acc[rt][dt][j] *= alpha[rt];
     }
-    const char* vbase = v_frag + buf * VSTAGE;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (EXACT || dt < dts) {
-        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
+      if (EXACT || dt < dts)
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) tw_mma16(acc[rt][dt], vf, pb[rt]);
-      }
+        for (int rt = 0; rt < RT; ++rt) tw_mma16(acc[rt][dt], vf[dt], pb[rt]);
   };
   auto compute_if_seen = [&](int blk, int buf) {
     const int p0 = blk * 32;
@@ -909,13 +926,16 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       compute(blk, buf, !(wave_full && p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len));
   };
 
+  lookup(blk_begin);
   fetch(blk_begin);
+  lookup(blk_begin + 1);
   stash(0);
   __syncthreads();
   int blk = blk_begin;
   for (; blk + 1 < blk_end; ++blk) {                        // every fetch unconditional: no register copies
     const int buf = (blk - blk_begin) & 1;
     fetch(blk + 1);
+    lookup(blk + 2);                                         // (its page numbers replace those just used)
     compute_if_seen(blk, buf);
     stash(buf ^ 1);
     __syncthreads();
