@@ -122,8 +122,7 @@ struct RowTile {
       s[j] = ok ? s[j] * a.scale : -INFINITY;
       mx = fmaxf(mx, s[j]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
+    mx = tw_rows_max(mx);
     const float m_new = fmaxf(m, mx);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = tw_exp<T>(m - m_use);
@@ -134,8 +133,7 @@ struct RowTile {
       pr[j] = tw_exp<T>(s[j] - m_use);
       sum += pr[j];
     }
-    sum += __shfl_xor(sum, 16, TW_WAVE);
-    sum += __shfl_xor(sum, 32, TW_WAVE);
+    sum = tw_rows_sum(sum);
     l = l * alpha + sum;
     m = m_new;
     // ---- O^T += V^T P^T (this lane loads d = 16 dt + r, keys p0 + 4g .. + 3) ----
@@ -391,8 +389,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
       pr[e] = (!EDGE || (p < kv_len && p >= lo)) ? s[e >> 2][e & 3] * a.scale : -INFINITY;
       mx = fmaxf(mx, pr[e]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
+    mx = tw_rows_max(mx);
     const float m_new = fmaxf(m, mx);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
     float sum = 0.f;
@@ -403,8 +400,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
       sum += pe;
       pb[e] = (bf16_t)pe;
     }
-    sum += __shfl_xor(sum, 16, TW_WAVE);
-    sum += __shfl_xor(sum, 32, TW_WAVE);
+    sum = tw_rows_sum(sum);
     // the running maximum of a row rarely moves after the first blocks: rescale only then
     if (__any(m_new > m)) {
       const float alpha = __expf(m - m_use);
@@ -883,8 +879,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       float mx = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[rt][e >> 2][e & 3]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, TW_WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, TW_WAVE));
+      mx = tw_rows_max(mx);
       // m is kept in the scaled log2 domain: m = max(score) * c2 (c2 > 0)
       const float m_new = fmaxf(m[rt], mx * c2);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -896,8 +891,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         sum += pe;
         pb[rt][e] = (bf16_t)pe;
       }
-      sum += __shfl_xor(sum, 16, TW_WAVE);
-      sum += __shfl_xor(sum, 32, TW_WAVE);
+      sum = tw_rows_sum(sum);
       l[rt] = l[rt] * alpha[rt] + sum;
       m[rt] = m_new;
     }

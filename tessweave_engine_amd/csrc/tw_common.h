@@ -119,6 +119,22 @@ __device__ __forceinline__ float tw_wave_max(float v) {
   return v;
 }
 
+// A value combined over lanes l, l ^ 16, l ^ 32, l ^ 48 (the four 16-lane rows of a wave) with gfx950's
+// lane-swap instructions: two vector instructions per step instead of a round trip through the LDS
+// crossbar (ds_bpermute), which sat in the dependent chain of every softmax block.
+__device__ __forceinline__ float tw_rows_max(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float tw_rows_sum(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result. The
 // order of additions is fixed by the block size alone.
 __device__ __forceinline__ float tw_block_sum(float v, float* lds /* >= 16 floats */) {
