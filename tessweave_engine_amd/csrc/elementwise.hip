@@ -133,6 +133,43 @@ __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restri
   }
 }
 
+// Many rows, nothing to add: one WAVE per row (4 rows per workgroup), a row of up to 4096 elements
+// in registers as up to 16 groups of 4, every load issued at once, and no barrier: the sum of squares
+// is a wave reduction. (With one workgroup of 896 threads per row, 2,048 rows of 3,584 took 15 us.)
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                           T* __restrict__ out, int n_rows, int hidden, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  const float* src = x + (size_t)row * hidden;
+  f32x4 v[16];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int h = (i * 64 + lane) * 4;
+    v[i] = h < hidden ? *reinterpret_cast<const f32x4*>(src + h) : f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) ss += ((v[i][0] * v[i][0] + v[i][1] * v[i][1]) + v[i][2] * v[i][2]) + v[i][3] * v[i][3];
+  ss = tw_wave_sum(ss);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+  T* dst = out + (size_t)row * hidden;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int h = (i * 64 + lane) * 4;
+    if (h >= hidden) continue;
+    const f32x4 wv = *reinterpret_cast<const f32x4*>(w + h);
+    T packed[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) packed[e] = tw_from_float<T>(v[i][e] * scale * wv[e]);
+    if (sizeof(T) == 2)
+      *reinterpret_cast<uint64_t*>(dst + h) = *reinterpret_cast<const uint64_t*>(packed);
+    else
+      *reinterpret_cast<f32x4*>(dst + h) = *reinterpret_cast<const f32x4*>(packed);
+  }
+}
+
 extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, const int* rows,
                           int n_out, int hidden, float eps, const float* add, int add_splits,
                           long add_stride, float* row_scratch, hipStream_t stream) {
@@ -140,6 +177,14 @@ extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, co
   TW_REQUIRE(add == nullptr || (add_splits > 0 && (rows == nullptr || row_scratch != nullptr)));
   if (n_out == 0) return 0;
   if (out_dtype != TW_DTYPE_F32 && out_dtype != TW_DTYPE_BF16) return TW_ERR_BAD_ARGUMENT;
+  if (add == nullptr && rows == nullptr && n_out >= 256 && hidden % 4 == 0 && hidden <= 4096 &&
+      (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    if (out_dtype == TW_DTYPE_F32)
+      rmsnorm_wave_kernel<float><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, (float*)out, n_out, hidden, eps);
+    else
+      rmsnorm_wave_kernel<bf16_t><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, (bf16_t*)out, n_out, hidden, eps);
+    return TW_LAUNCH_RESULT();
+  }
   // rows of up to 4096 elements: one group of 4 elements per thread, everything in registers
   if (hidden % 4 == 0 && hidden <= 4096 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
       (add == nullptr || ((uintptr_t)add % 16 == 0 && add_stride % 4 == 0))) {

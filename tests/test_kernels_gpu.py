@@ -45,6 +45,12 @@ def test_rmsnorm(ops, device, dtype, hidden, eps):
     ops.rmsnorm(x, w, eps, out)
     want = plain.rms_norm(x.cpu().double(), w.cpu().double(), eps).float()
     torch.testing.assert_close(out.float().cpu(), want, **tol(dtype, (3e-6, 3e-6), (1e-2, 1e-2)))
+    # many rows (another kernel: one wave per row)
+    xm = rand((261, hidden), torch.float32, device, 3.0, seed=5)
+    outm = torch.full((261, hidden), float("nan"), dtype=dtype, device=device)
+    ops.rmsnorm(xm, w, eps, outm)
+    wantm = plain.rms_norm(xm.cpu().double(), w.cpu().double(), eps).float()
+    torch.testing.assert_close(outm.float().cpu(), wantm, **tol(dtype, (3e-6, 3e-6), (1e-2, 1e-2)))
     # gathered rows
     rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=device)
     out2 = torch.empty(3, hidden, dtype=dtype, device=device)
