@@ -317,7 +317,7 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
                            const float* residual, long ldr, OutT* C, long ldc, float* partial,
                            long partial_bytes, int M, int N, int K, int force, hipStream_t stream) {
   constexpr int EPF = Elem<T>::kPerFrag;
-  TW_REQUIRE(force == 0 || force == 1 || force == 3 || force == 4 || force == 5 || force == 6);
+  TW_REQUIRE(force == 0 || force == 1 || (force >= 3 && force <= 7));
   // the shuffled layout exists only for K that is a multiple of 16 bytes and is always aligned
   const bool aligned = K % EPF == 0 && lda % EPF == 0 && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) &&
                        (SHUF || ldw % EPF == 0);
@@ -333,7 +333,7 @@ static int linear_dispatch(const T* A, long lda, const T* W, long ldw, const flo
     TW_REQUIRE(M <= 64);
     return launch_skinny_lds_m<T, OutT, false, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
-  const int shape = force == 3 ? 1 : (force == 4 ? 2 : (force == 6 ? 3 : 0));
+  const int shape = force == 3 ? 1 : (force == 4 ? 2 : (force == 6 ? 3 : (force == 7 ? 4 : 0)));
   return tw_tiled_linear(sizeof(T) == 4 ? TW_DTYPE_F32 : TW_DTYPE_BF16, sizeof(OutT) == 4 ? 1 : 0, SHUF ? 1 : 0,
                          GLU ? 1 : 0, shape, A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes,
                          M, N, K, stream);

@@ -450,6 +450,8 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
   do {                                                                        \
     if constexpr (COPIES * (tiles) == 8) TW_DMA_WAIT(8);                      \
     else if constexpr (COPIES * (tiles) == 12) TW_DMA_WAIT(12);               \
+    else if constexpr (COPIES * (tiles) == 14) TW_DMA_WAIT(14);               \
+    else if constexpr (COPIES * (tiles) == 21) TW_DMA_WAIT(21);               \
     else if constexpr (COPIES * (tiles) == 16) TW_DMA_WAIT(16);               \
     else if constexpr (COPIES * (tiles) == 18) TW_DMA_WAIT(18);               \
     else if constexpr (COPIES * (tiles) == 24) TW_DMA_WAIT(24);               \
@@ -459,7 +461,7 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
   } while (0)
 #define TW_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
   // the order asked of the scheduler: G groups of (copies, fragment reads, MFMAs) per k-chunk pair
-  constexpr int G = WM * WN >= 16 ? 4 : 2;
+  constexpr int G = (WM + WN) % 2 ? 1 : (WM * WN >= 16 ? 4 : 2);
 
   bf16x8 af[2][WM], wf[2][WN];
   if (k_tiles > 0) {
@@ -578,19 +580,30 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
   return TW_LAUNCH_RESULT();
 }
 
-// Which tile: 256x256 when there are at least one and a half rounds of them for 256 CUs (per MFMA it moves half
-// the bytes through the 64 B/clk vector-memory path and the LDS that 128x128 does); 128x256 when that
-// makes one round that fills most of the chip; else 128x128, two workgroups per CU.
+// Which tile (1: 128x128, 2: 128x256, 3: 256x256, 4: 256x192): the one with the least estimated time,
+// rounds of tiles over 256 CUs (128x128: two to a CU, so half rounds) x tile area / the rate a tile of
+// that shape reaches when the chip is full (measured, relative). The estimate ranks the shapes as
+// measured on the projections of 7B-class models from 256 to 16,384 rows. Larger tiles move fewer
+// bytes per MFMA through the 64 B/clk vector-memory path and LDS; smaller ones waste less in the
+// last round.
 #ifndef TW_DMA_SHAPES
 #define TW_DMA_SHAPES 0xC      /* bit s: shape s uses the direct-to-LDS kernel (at 128x128 it gains nothing) */
 #endif
 static int choose_shape(bool big_ok, int M, int N) {
-  if (big_ok) {
-    if ((long)tw_div_up(M, 256) * tw_div_up(N, 256) >= 384) return 3;
-    const long wide = (long)tw_div_up(M, 128) * tw_div_up(N, 256);
-    if (wide >= 192 && wide <= 256) return 2;
+  if (!big_ok) return 1;
+  const int bm[5] = {0, 128, 128, 256, 256}, bn[5] = {0, 128, 256, 256, 192};
+  const double rate[5] = {0, 0.80, 0.93, 1.15, 1.00};
+  int best = 1;
+  double best_cost = 0;
+  for (int shape = 1; shape <= 4; ++shape) {
+    const long tiles = (long)tw_div_up(M, bm[shape]) * tw_div_up(N, bn[shape]);
+    const double cost = (double)tw_div_up(tiles, 256) * bm[shape] * bn[shape] / rate[shape];
+    if (shape == 1 || cost < best_cost) {
+      best = shape;
+      best_cost = cost;
+    }
   }
-  return 1;
+  return best;
 }
 
 template <typename T, typename OutT, bool SHUF, bool GLU>
@@ -602,6 +615,7 @@ static int tiled_by_shape(int shape, const T* A, long lda, const T* W, long ldw,
   if constexpr (BIG) {
     // bfloat16 and shuffled weights: the kernels that copy straight into LDS, if K allows
     if (K % 32 == 0 && K >= 32 && lda % 8 == 0) {
+      if (shape == 4) return launch_dma<OutT, 4, 3, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
       if constexpr ((TW_DMA_SHAPES & 8) != 0)
         if (shape == 3) return launch_dma<OutT, 4, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
       if constexpr ((TW_DMA_SHAPES & 4) != 0)
@@ -609,10 +623,10 @@ static int tiled_by_shape(int shape, const T* A, long lda, const T* W, long ldw,
       if constexpr ((TW_DMA_SHAPES & 2) != 0)
         if (shape == 1) return launch_dma<OutT, 2, 2, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
     }
-    if (shape == 3)
+    if (shape == 3 || shape == 4)             // (K no multiple of 32: the register-staged 256x256 tile for both)
       return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   }
-  if (shape == 3) return TW_ERR_BAD_ARGUMENT;
+  if (shape == 3 || shape == 4) return TW_ERR_BAD_ARGUMENT;
   if (shape == 2)
     return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
@@ -639,7 +653,7 @@ static int tiled_by_layout(int shuffled, int glu, int shape, const void* A, long
 int tw_tiled_linear(int dtype, int out_f32, int shuffled, int glu, int shape, const void* A, long lda,
                     const void* W, long ldw, const float* bias, const float* residual, long ldr, void* C,
                     long ldc, float* partial, long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  TW_REQUIRE(shape >= 0 && shape <= 3);
+  TW_REQUIRE(shape >= 0 && shape <= 4);
   if (dtype == TW_DTYPE_F32)
     return tiled_by_layout<float, float>(shuffled, glu, shape, A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   if (dtype != TW_DTYPE_BF16) return TW_ERR_BAD_ARGUMENT;

@@ -168,7 +168,7 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
     t = dict(atol=2e-5 * scale, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2 * scale, rtol=2e-2)
     shuffled = ops.shuffle_weight(w)
     torch.testing.assert_close(shuffled.to_rows(), w, atol=0, rtol=0)          # an exact permutation
-    big = (ops.GEMM_TILED_256,) if dtype == torch.bfloat16 else ()     # 256x256 tiles: bfloat16, shuffled weights
+    big = (ops.GEMM_TILED_256, ops.GEMM_TILED_256X192) if dtype == torch.bfloat16 else ()   # bfloat16, shuffled weights
     if not big:                                                        # ... and refused otherwise
         with pytest.raises(Exception, match="refused its arguments"):
             ops.linear(x, shuffled, torch.empty((m, n), dtype=dtype, device=device), force=ops.GEMM_TILED_256)
@@ -237,7 +237,7 @@ def test_linear_glu(ops, device, dtype, m, inter, k):
         u = xd @ up.double().cpu().T + (bu.double().cpu() if b is not None else 0)
         want = torch.nn.functional.silu(g) * u
         for weight in layouts:
-            big = [ops.GEMM_TILED_256] if (dtype == torch.bfloat16 and weight is not w) else []
+            big = [ops.GEMM_TILED_256, ops.GEMM_TILED_256X192] if (dtype == torch.bfloat16 and weight is not w) else []
             for force in forces + big:
                 out = torch.full((m, inter), float("nan"), dtype=dtype, device=device)
                 ops.linear_glu(x, weight, out, bias=b, force=force)
