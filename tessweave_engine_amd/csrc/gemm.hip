@@ -18,6 +18,7 @@
 // blocks of 16 rows (gate rows 16j.., then up rows 16j.., for j = 0, 1, ...). The kernels form
 // C[M, N/2][.., 16j + i] = silu(gate_j[i]) * up_j[i] in their epilogues, in float32 from the
 // accumulators, so the [M, N] intermediate never reaches memory.
+#include <type_traits>
 #include "tw_common.h"
 #include "gemm_shared.h"
 
@@ -38,7 +39,7 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p
 // MFMA steps the workgroup copies the activations' K slice [16*MT rows][U*64 B]
 // to LDS once (instead of every wave reading it from L2); each wave streams its
 // own 16 weight rows from global memory into registers (every weight byte is read by exactly
-// one wave). Two stages in flight. splits == 1: the epilogue runs here. splits > 1: float32
+// one wave). Two stages of weights in flight. splits == 1: the epilogue runs here. splits > 1: float32
 // partial sums go to partial[split][M][N] and splitk_reduce_kernel (or the caller's next
 // kernel) adds them, always in the same order, so results do not depend on timing.
 // =====================================================================================
@@ -92,36 +93,30 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
     x_dst[i] = row * XROW + c * 16;
   }
 
+  // Loads carry no predicate: addresses are clamped to the last valid step or chunk (always inside
+  // the matrix), and activation chunks outside this workgroup's K range are replaced by zeros on
+  // their way to LDS, so whatever weight was read beside them adds nothing. Without conditional
+  // loads the compiler's wait counts are exact, which the order of the pipeline below relies on.
   Frag wf[2][U], xg[XLOADS];
-  auto load_w = [&](const int buf, int s0, bool whole) {
+  const int chunk_end = min(step_end * 4, chunks);
+  auto load_w = [&](const int buf, int s0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int chunk = (s0 + u) * 4 + g;
-      if (SHUF) {
-        if (whole || (s0 + u) < step_end)
-          wf[buf][u] = tw_load_frag_stream(w_row + (size_t)(s0 + u) * 64 * EPF);
-        else
-          wf[buf][u] = Elem<T>::zero();
-      } else if (whole || ((s0 + u) < step_end && chunk < chunks))
-        wf[buf][u] = tw_load_frag(w_row + (size_t)chunk * EPF);
+      if (SHUF)
+        wf[buf][u] = tw_load_frag_stream(w_row + (size_t)min(s0 + u, steps - 1) * 64 * EPF);
       else
-        wf[buf][u] = Elem<T>::zero();
+        wf[buf][u] = tw_load_frag(w_row + (size_t)min((s0 + u) * 4 + g, chunks - 1) * EPF);
     }
   };
-  auto load_x = [&](int s0, bool whole) {
-#pragma unroll
-    for (int i = 0; i < XLOADS; ++i) {
-      const int chunk = s0 * 4 + x_chunk[i];
-      if (whole || (chunk < step_end * 4 && chunk < chunks))
-        xg[i] = tw_load_frag(x_src[i] + (size_t)chunk * EPF);
-      else
-        xg[i] = Elem<T>::zero();
-    }
-  };
-  auto store_x = [&](int buf) {
+  auto load_x = [&](int s0) {
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i)
-      *reinterpret_cast<Frag*>(lds + buf * XSTAGE + x_dst[i]) = xg[i];
+      xg[i] = tw_load_frag(x_src[i] + (size_t)min(s0 * 4 + x_chunk[i], chunks - 1) * EPF);
+  };
+  auto store_x = [&](int buf, int s0) {
+#pragma unroll
+    for (int i = 0; i < XLOADS; ++i)
+      *reinterpret_cast<Frag*>(lds + buf * XSTAGE + x_dst[i]) = s0 * 4 + x_chunk[i] < chunk_end ? xg[i] : Elem<T>::zero();
   };
   auto multiply = [&](const int buf) {
 #pragma unroll
@@ -132,37 +127,39 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
         tw_mma16(acc[mt], wf[buf][u], xf);
       }
   };
-  auto whole_stage = [&](int s0) { return s0 + U <= step_end && (s0 + U) * 4 <= chunks; };
+  // Two stages i, i + 1 (i even: stage i has its weights in register set 0 and its activations in
+  // LDS buffer 0). Per stage: request the next stage's activations, multiply this stage, request
+  // the weights of the stage after next into the registers just used, then move the activations to
+  // LDS. Loads return in order, so the wait for the activations leaves the newest weight loads in
+  // flight: a wave that stalls there has one to two stages of weights on their way.
+  auto stage_pair = [&](int i, auto more1, auto more2, auto more3) {
+    const int s0 = step_begin + i * U;
+    if (more1) load_x(s0 + U);
+    __builtin_amdgcn_sched_barrier(0);           // the compiler would sink the loads below the waits
+    multiply(0);
+    if (more2) load_w(0, s0 + 2 * U);
+    __builtin_amdgcn_sched_barrier(0);
+    if (more1) store_x(1, s0 + U);
+    __syncthreads();
+    if (!more1) return;
+    if (more2) load_x(s0 + 2 * U);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1);
+    if (more3) load_w(1, s0 + 3 * U);
+    __builtin_amdgcn_sched_barrier(0);
+    if (more2) store_x(0, s0 + 2 * U);
+    __syncthreads();
+  };
 
   if (n_stages > 0) {
-    {
-      const bool whole = whole_stage(step_begin);
-      load_w(0, step_begin, whole);
-      load_x(step_begin, whole);
-      store_x(0);
-    }
+    load_x(step_begin);
+    load_w(0, step_begin);
+    if (n_stages > 1) load_w(1, step_begin + U);
+    store_x(0, step_begin);
     __syncthreads();
-    for (int i = 0; i < n_stages; i += 2) {
-      const int s0 = step_begin + i * U;
-      const bool more1 = i + 1 < n_stages, more2 = i + 2 < n_stages;
-      if (more1) {
-        const bool whole = whole_stage(s0 + U);
-        load_w(1, s0 + U, whole);
-        load_x(s0 + U, whole);
-      }
-      multiply(0);
-      if (more1) store_x(1);
-      __syncthreads();
-      if (!more1) break;
-      if (more2) {
-        const bool whole = whole_stage(s0 + 2 * U);
-        load_w(0, s0 + 2 * U, whole);
-        load_x(s0 + 2 * U, whole);
-      }
-      multiply(1);
-      if (more2) store_x(0);
-      __syncthreads();
-    }
+    int i = 0;
+    for (; i + 3 < n_stages; i += 2) stage_pair(i, std::true_type{}, std::true_type{}, std::true_type{});
+    for (; i < n_stages; i += 2) stage_pair(i, i + 1 < n_stages, i + 2 < n_stages, i + 3 < n_stages);
   }
 
   // acc[mt][j] = sum_k W[n0 + 4g + j][k] * A[16 mt + r][k]
