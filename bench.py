@@ -24,6 +24,15 @@ QWEN25_7B = dict(
     vocab_size=152064, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False,
     use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
 
+# Further shapes of the same architecture (--shape): sizes only, everything else as above.
+SHAPES = {
+    "7b": ("Qwen2.5-7B shape", {}),
+    "14b": ("Qwen2.5-14B shape", dict(num_hidden_layers=48, hidden_size=5120, num_attention_heads=40,
+                                      num_key_value_heads=8, intermediate_size=13824, rms_norm_eps=1e-5)),
+    "32b": ("Qwen2.5-32B shape", dict(num_hidden_layers=64, hidden_size=5120, num_attention_heads=40,
+                                      num_key_value_heads=8, intermediate_size=27648, rms_norm_eps=1e-5)),
+}
+
 HBM_PEAK_GBS = 8000.0
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
 
@@ -35,7 +44,8 @@ def parse():
     p.add_argument("--warmup", type=int, default=16)
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=4096)
-    p.add_argument("--layers", type=int, default=0, help="fewer layers than the 7B shape has (0: all 28)")
+    p.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes (default: the 7B shape)")
+    p.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all of them)")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--points", default="1,64", help="further decode batch sizes to measure")
@@ -124,7 +134,8 @@ def main():
     from tessweave_engine_amd.config import config_from_dict
     from tessweave_engine_amd.weights import random_model
 
-    cfg = dict(QWEN25_7B)
+    shape_name, sizes = SHAPES[args.shape]
+    cfg = dict(QWEN25_7B, **sizes)
     layers_full = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -165,13 +176,13 @@ def main():
         points[f"decode_b{b}"] = round(tps, 1)
 
     line = {
-        "metric": f"decode tok/s @ batch {args.batch}, Qwen2.5-7B shape {'bf16' if args.dtype == 'bfloat16' else 'fp32'} "
+        "metric": f"decode tok/s @ batch {args.batch}, {shape_name} {'bf16' if args.dtype == 'bfloat16' else 'fp32'} "
                   f"(+ prefill tok/s @ {t}, decode @ batch {args.points or '-'})",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform-random token ids, random weights N(0, 0.02)",
-        "config": {"model": "Qwen2.5-7B shape", "layers": c.num_hidden_layers, "layers_full": layers_full,
+        "config": {"model": shape_name, "layers": c.num_hidden_layers, "layers_full": layers_full,
                    "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
                    "head_dim": c.head_dim, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
                    "global_batch": args.batch, "seq_len": args.context,

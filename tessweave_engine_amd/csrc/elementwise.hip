@@ -72,56 +72,71 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ 
     dst[h] = tw_from_float<T>(src[h] * scale * w[h]);
 }
 
-// The same for hidden % 4 == 0 with at most 4 * blockDim.x elements per row: every
-// thread owns ONE group of 4 consecutive elements, kept in registers between the
-// two passes; the partial sums are read with independent 16-byte loads. (The sum
+// The same for hidden % 4 == 0 with at most 4 * G * blockDim.x elements per row: every
+// thread owns G groups of 4 consecutive elements (blockDim.x groups apart), kept in registers
+// between the two passes; the partial sums are read with independent 16-byte loads. (The sum
 // of squares is associated differently from the kernel above: results of the two
 // kernels agree to rounding, not to the bit.)
-template <typename T>
+template <typename T, int G>
 __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restrict__ w, T* __restrict__ out,
                                     const int* __restrict__ rows, int hidden, float eps,
                                     const float* __restrict__ add, int add_splits, size_t add_stride) {
   __shared__ float lds[16];
   const int o = blockIdx.x;
   const int r = rows ? rows[o] : o;
-  const int h = threadIdx.x * 4;
-  const bool mine = h < hidden;
   float* src = x + (size_t)r * hidden;
-  f32x4 v = {0.f, 0.f, 0.f, 0.f};
-  f32x4 wv = {0.f, 0.f, 0.f, 0.f};
-  if (mine) {
-    // Every load of the row is issued before the first one is waited for (the kernel's time is a
-    // chain of memory latencies): the row itself, the weight, and the partial sums 8 at a time.
-    // The partial sums are still added one after the other in index order, then the row.
-    const f32x4 xv = *reinterpret_cast<const f32x4*>(src + h);
-    if (add) wv = *reinterpret_cast<const f32x4*>(w + h);      // (few rows; with many, the weight is read below)
-    if (add) {
-      const float* p = add + (size_t)r * hidden + h;
-      for (int s0 = 0; s0 < add_splits; s0 += 8) {
-        f32x4 a[8];
+  f32x4 v[G], wv[G], xv[G];
+  int h[G];
+  bool mine[G];
+  // Every load of the row is issued before the first one is waited for (the kernel's time is a
+  // chain of memory latencies): the row itself, the weight, and the partial sums 8 at a time.
+  // The partial sums are still added one after the other in index order, then the row.
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          a[i] = s0 + i < add_splits ? *reinterpret_cast<const f32x4*>(p + (size_t)(s0 + i) * add_stride)
-                                     : f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (s0 + i < add_splits) v = v + a[i];
-      }
-      v = v + xv;
-      if (!rows) *reinterpret_cast<f32x4*>(src + h) = v;
-    } else {
-      v = xv;
+  for (int gi = 0; gi < G; ++gi) {
+    h[gi] = (gi * (int)blockDim.x + (int)threadIdx.x) * 4;
+    mine[gi] = h[gi] < hidden;
+    v[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+    wv[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+    xv[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (mine[gi]) {
+      xv[gi] = *reinterpret_cast<const f32x4*>(src + h[gi]);
+      if (add) wv[gi] = *reinterpret_cast<const f32x4*>(w + h[gi]);   // (few rows; with many, the weight is read below)
     }
   }
-  float ss = mine ? ((v[0] * v[0] + v[1] * v[1]) + v[2] * v[2]) + v[3] * v[3] : 0.f;
+  float ss = 0.f;
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) {
+    if (mine[gi]) {
+      if (add) {
+        const float* p = add + (size_t)r * hidden + h[gi];
+        for (int s0 = 0; s0 < add_splits; s0 += 8) {
+          f32x4 a[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            a[i] = s0 + i < add_splits ? *reinterpret_cast<const f32x4*>(p + (size_t)(s0 + i) * add_stride)
+                                       : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (s0 + i < add_splits) v[gi] = v[gi] + a[i];
+        }
+        v[gi] = v[gi] + xv[gi];
+        if (!rows) *reinterpret_cast<f32x4*>(src + h[gi]) = v[gi];
+      } else {
+        v[gi] = xv[gi];
+      }
+      ss += ((v[gi][0] * v[gi][0] + v[gi][1] * v[gi][1]) + v[gi][2] * v[gi][2]) + v[gi][3] * v[gi][3];
+    }
+  }
   ss = tw_block_sum(ss, lds);
   const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
-  if (mine) {
-    if (!add) wv = *reinterpret_cast<const f32x4*>(w + h);
-    T* dst = out + (size_t)o * hidden + h;
+#pragma unroll
+  for (int gi = 0; gi < G; ++gi) {
+    if (!mine[gi]) continue;
+    if (!add) wv[gi] = *reinterpret_cast<const f32x4*>(w + h[gi]);
+    T* dst = out + (size_t)o * hidden + h[gi];
     T packed[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) packed[e] = tw_from_float<T>(v[e] * scale * wv[e]);
+    for (int e = 0; e < 4; ++e) packed[e] = tw_from_float<T>(v[gi][e] * scale * wv[gi][e]);
     if (sizeof(T) == 2 && ((uintptr_t)out % 8 == 0))
       *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(packed);      // hidden % 4 == 0: aligned
     else if (sizeof(T) == 4 && ((uintptr_t)out % 16 == 0))
@@ -133,30 +148,30 @@ __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restri
   }
 }
 
-// Many rows, nothing to add: one WAVE per row (4 rows per workgroup), a row of up to 4096 elements
-// in registers as up to 16 groups of 4, every load issued at once, and no barrier: the sum of squares
+// Many rows, nothing to add: one WAVE per row (4 rows per workgroup), a row of up to 256 * NG elements
+// in registers as up to NG groups of 4, every load issued at once, and no barrier: the sum of squares
 // is a wave reduction. (With one workgroup of 896 threads per row, 2,048 rows of 3,584 took 15 us.)
-template <typename T>
+template <typename T, int NG>
 __global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                            T* __restrict__ out, int n_rows, int hidden, float eps) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= n_rows) return;
   const float* src = x + (size_t)row * hidden;
-  f32x4 v[16];
+  f32x4 v[NG];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < NG; ++i) {
     const int h = (i * 64 + lane) * 4;
     v[i] = h < hidden ? *reinterpret_cast<const f32x4*>(src + h) : f32x4{0.f, 0.f, 0.f, 0.f};
   }
 #pragma unroll
-  for (int i = 0; i < 16; ++i) ss += ((v[i][0] * v[i][0] + v[i][1] * v[i][1]) + v[i][2] * v[i][2]) + v[i][3] * v[i][3];
+  for (int i = 0; i < NG; ++i) ss += ((v[i][0] * v[i][0] + v[i][1] * v[i][1]) + v[i][2] * v[i][2]) + v[i][3] * v[i][3];
   ss = tw_wave_sum(ss);
   const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
   T* dst = out + (size_t)row * hidden;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < NG; ++i) {
     const int h = (i * 64 + lane) * 4;
     if (h >= hidden) continue;
     const f32x4 wv = *reinterpret_cast<const f32x4*>(w + h);
@@ -170,6 +185,27 @@ __global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const float* __restri
   }
 }
 
+template <typename T>
+static void launch_rmsnorm_vec4(int groups_per_thread, int n_out, int threads, hipStream_t stream, float* x,
+                                const float* w, T* out, const int* rows, int hidden, float eps, const float* add,
+                                int add_splits, size_t add_stride) {
+  if (groups_per_thread == 1)
+    rmsnorm_vec4_kernel<T, 1><<<n_out, threads, 0, stream>>>(x, w, out, rows, hidden, eps, add, add_splits, add_stride);
+  else if (groups_per_thread == 2)
+    rmsnorm_vec4_kernel<T, 2><<<n_out, threads, 0, stream>>>(x, w, out, rows, hidden, eps, add, add_splits, add_stride);
+  else
+    rmsnorm_vec4_kernel<T, 4><<<n_out, threads, 0, stream>>>(x, w, out, rows, hidden, eps, add, add_splits, add_stride);
+}
+
+template <typename T>
+static void launch_rmsnorm_wave(int n_out, hipStream_t stream, const float* x, const float* w, T* out, int hidden,
+                                float eps) {
+  if (hidden <= 4096)
+    rmsnorm_wave_kernel<T, 16><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, out, n_out, hidden, eps);
+  else
+    rmsnorm_wave_kernel<T, 32><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, out, n_out, hidden, eps);
+}
+
 extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, const int* rows,
                           int n_out, int hidden, float eps, const float* add, int add_splits,
                           long add_stride, float* row_scratch, hipStream_t stream) {
@@ -177,24 +213,25 @@ extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, co
   TW_REQUIRE(add == nullptr || (add_splits > 0 && (rows == nullptr || row_scratch != nullptr)));
   if (n_out == 0) return 0;
   if (out_dtype != TW_DTYPE_F32 && out_dtype != TW_DTYPE_BF16) return TW_ERR_BAD_ARGUMENT;
-  if (add == nullptr && rows == nullptr && n_out >= 256 && hidden % 4 == 0 && hidden <= 4096 &&
+  if (add == nullptr && rows == nullptr && n_out >= 256 && hidden % 4 == 0 && hidden <= 8192 &&
       (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
     if (out_dtype == TW_DTYPE_F32)
-      rmsnorm_wave_kernel<float><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, (float*)out, n_out, hidden, eps);
+      launch_rmsnorm_wave<float>(n_out, stream, x, w, (float*)out, hidden, eps);
     else
-      rmsnorm_wave_kernel<bf16_t><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, (bf16_t*)out, n_out, hidden, eps);
+      launch_rmsnorm_wave<bf16_t>(n_out, stream, x, w, (bf16_t*)out, hidden, eps);
     return TW_LAUNCH_RESULT();
   }
-  // rows of up to 4096 elements: one group of 4 elements per thread, everything in registers
-  if (hidden % 4 == 0 && hidden <= 4096 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+  // rows of up to 16384 elements: one, two or four groups of 4 elements per thread, everything in registers
+  if (hidden % 4 == 0 && hidden <= 16384 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
       (add == nullptr || ((uintptr_t)add % 16 == 0 && add_stride % 4 == 0))) {
-    const int threads = (hidden / 4 + 63) / 64 * 64;
+    const int per_thread = hidden <= 4096 ? 1 : (hidden <= 8192 ? 2 : 4);
+    const int threads = (hidden / 4 + per_thread * 64 - 1) / (per_thread * 64) * 64;
     if (out_dtype == TW_DTYPE_F32)
-      rmsnorm_vec4_kernel<float><<<n_out, threads, 0, stream>>>(x, w, (float*)out, rows, hidden, eps, add,
-                                                                add_splits, (size_t)add_stride);
+      launch_rmsnorm_vec4<float>(per_thread, n_out, threads, stream, x, w, (float*)out, rows, hidden, eps, add,
+                                 add_splits, (size_t)add_stride);
     else
-      rmsnorm_vec4_kernel<bf16_t><<<n_out, threads, 0, stream>>>(x, w, (bf16_t*)out, rows, hidden, eps, add,
-                                                                 add_splits, (size_t)add_stride);
+      launch_rmsnorm_vec4<bf16_t>(per_thread, n_out, threads, stream, x, w, (bf16_t*)out, rows, hidden, eps, add,
+                                  add_splits, (size_t)add_stride);
     return TW_LAUNCH_RESULT();
   }
   const int threads = hidden >= 2048 ? 512 : 256;

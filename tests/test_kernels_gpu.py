@@ -37,7 +37,8 @@ def test_embed_gather(ops, device, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden,eps", [(64, 1e-6), (200, 1e-5), (3000, 1e-2)])
+@pytest.mark.parametrize("hidden,eps", [(64, 1e-6), (200, 1e-5), (3000, 1e-2), (5120, 1e-5), (8196, 1e-6), (16384, 1e-6),
+                                        (16390, 1e-6)])       # one, two and four groups per thread; the generic kernel
 def test_rmsnorm(ops, device, dtype, hidden, eps):
     x = rand((7, hidden), torch.float32, device, 3.0)
     w = (1 + rand((hidden,), torch.float32, device, 0.1, seed=1))
