@@ -10,6 +10,10 @@ run through the scheduler (admission, planning, the step function, greedy
 sampling on the device, commit), so the last timed step reads 4,096 keys per
 request. One JSON line is printed: decoded tokens a second, a 2,048-token
 prefill, the decode step's HBM roofline, and decode at batch 1 and 64.
+
+Other sizes of the architecture: --shape 14b|32b. --serve measures continuous
+batching under Poisson arrivals instead (prompts of 128..4,096 tokens, 256
+generated tokens each, prompt portions of 512) and prints its own JSON line.
 """
 from __future__ import annotations
 
@@ -52,6 +56,11 @@ def parse():
     p.add_argument("--no-graphs", action="store_true")
     p.add_argument("--prefill-only", action="store_true", help="measure only the prefill (profiling runs)")
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--serve", action="store_true",
+                   help="instead: continuous batching of --requests requests (prompts of 128..4096 tokens, 256 "
+                        "generated each, Poisson arrivals at --rate a second, prompt portions of 512)")
+    p.add_argument("--requests", type=int, default=64)
+    p.add_argument("--rate", type=float, default=16.0, help="mean arrivals a second (0: all at once)")
     return p.parse_args()
 
 
@@ -99,6 +108,54 @@ def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, s
     return batch * steps / elapsed, elapsed / steps * 1000, replays
 
 
+def serve_run(model, torch, args):
+    """Continuous batching under arrivals: requests join while others decode; one JSON-ready dict."""
+    from tessweave_engine_amd.config import EngineConfig
+    from tessweave_engine_amd.engine import Engine
+
+    page, chunk, outputs, longest = 16, 512, 256, 4096
+    n, active = args.requests, min(args.requests, 64)
+    config = EngineConfig(block_size=page, kv_blocks=active * ((longest + outputs) // page + 1),
+                          max_context=longest + outputs, max_active=active, max_queue=n, prefill_chunk=chunk,
+                          min_prefill_chunk=16, prefix_cache=False, dtype=args.dtype,
+                          max_step_tokens=active + chunk, use_graphs=not args.no_graphs)
+    engine = Engine(model, config)
+    g = torch.Generator().manual_seed(args.seed)
+    lengths = torch.randint(128, longest + 1, (n,), generator=g).tolist()
+    prompts = [torch.randint(0, model.config.vocab_size, (k,), generator=g).tolist() for k in lengths]
+    gaps = torch.empty(n).exponential_(args.rate, generator=g).tolist() if args.rate > 0 else [0.0] * n
+    arrivals, t = [], 0.0
+    for gap in gaps:
+        t += gap
+        arrivals.append(t)
+    engine.generate(prompts[:2], max_tokens=4, ignore_eos=True)          # untimed: first launches, workspace
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    requests, nxt, steps0 = [], 0, engine.stats()["steps"]
+    while nxt < n or engine.active or engine.waiting or engine._inflight is not None:
+        now = time.perf_counter() - t0
+        while nxt < n and arrivals[nxt] <= now:
+            requests.append(engine.submit(prompts[nxt], max_tokens=outputs, ignore_eos=True))
+            nxt += 1
+        if not engine.step() and nxt < n:
+            time.sleep(max(0.0, min(0.001, arrivals[nxt] - (time.perf_counter() - t0))))
+    engine.flush()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert all(len(r.output) == outputs for r in requests), sorted(len(r.output) for r in requests)[:4]
+    ttft = sorted((r.first_token - r.created) * 1000 for r in requests)
+    stats = engine.stats()
+    engine.close()
+    generated, prompt_tokens = n * outputs, sum(lengths)
+    return {"metric": "continuous batching, generated tokens a second", "value": round(generated / elapsed, 1),
+            "unit": "tokens/s", "total_tokens_per_s": round((generated + prompt_tokens) / elapsed, 1),
+            "seconds": round(elapsed, 3), "requests": n, "rate": args.rate, "prompt_tokens": prompt_tokens,
+            "generated_tokens": generated, "ttft_ms_mean": round(sum(ttft) / n, 1),
+            "ttft_ms_p50": round(ttft[n // 2], 1), "ttft_ms_p99": round(ttft[min(n - 1, int(n * 0.99))], 1),
+            "steps": stats["steps"] - steps0, "graph_replays": stats["graph_replays"], "prefill_chunk": chunk,
+            "max_active": active}
+
+
 def prefill_run(model, torch, tokens, dtype, seed, repeats=3):
     from tessweave_engine_amd.cache import CacheManager
     from tessweave_engine_amd.engine import StepEntry, Stepper
@@ -144,6 +201,12 @@ def main():
     c = config
     use_graphs = not args.no_graphs
 
+    if args.serve:
+        line = serve_run(model, torch, args)
+        line.update({"model": shape_name, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                     "data": "synthetic: uniform-random token ids, random weights N(0, 0.02)"})
+        print(json.dumps(line))
+        return 0
     if args.prefill_only:
         ms = prefill_run(model, torch, args.prefill_tokens, args.dtype, args.seed)
         print(json.dumps({"prefill_ms": round(ms, 3), "tokens": args.prefill_tokens,
