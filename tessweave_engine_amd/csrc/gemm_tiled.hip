@@ -515,11 +515,11 @@ static int tiled_splits(int M, int N, int K, int epf, int bm, int bn) {
 template <typename T, typename OutT, int WM, int WN, bool SHUF, bool GLU>
 static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
                         const float* residual, long ldr, OutT* C, long ldc, float* partial,
-                        long partial_bytes, int M, int N, int K, hipStream_t stream) {
+                        long partial_bytes, int M, int N, int K, int want_splits, hipStream_t stream) {
   constexpr int BM = 64 * WM, BN = 64 * WN, KCH = 8;
   constexpr int EPF = Elem<T>::kPerFrag;
   const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
-  int splits = GLU ? 1 : tiled_splits(M, N, K, EPF, BM, BN);
+  int splits = GLU ? 1 : (want_splits > 0 ? want_splits : tiled_splits(M, N, K, EPF, BM, BN));
   if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4 || (uintptr_t)partial % 16 != 0)) splits = 1;
   const long n_blocks = (long)tiles_m * tiles_n * splits;
   TW_REQUIRE(n_blocks < (1L << 30));
@@ -551,11 +551,11 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
 template <typename OutT, int WM, int WN, bool GLU>
 static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias,
                       const float* residual, long ldr, OutT* C, long ldc, float* partial, long partial_bytes,
-                      int M, int N, int K, hipStream_t stream) {
+                      int M, int N, int K, int want_splits, hipStream_t stream) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   TW_REQUIRE(K % 32 == 0 && K >= 32 && lda % 8 == 0);
   const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
-  int splits = GLU ? 1 : tiled_splits(M, N, K, 8, BM, BN);
+  int splits = GLU ? 1 : (want_splits > 0 ? want_splits : tiled_splits(M, N, K, 8, BM, BN));
   if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4 || (uintptr_t)partial % 16 != 0)) splits = 1;
   const long n_blocks = (long)tiles_m * tiles_n * splits;
   TW_REQUIRE(n_blocks < (1L << 30));
@@ -589,15 +589,16 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
 #ifndef TW_DMA_SHAPES
 #define TW_DMA_SHAPES 0xC      /* bit s: shape s uses the direct-to-LDS kernel (at 128x128 it gains nothing) */
 #endif
+static const int kTileM[5] = {0, 128, 128, 256, 256}, kTileN[5] = {0, 128, 256, 256, 192};
+static const double kTileRate[5] = {0, 0.80, 0.93, 1.15, 1.00};
+
 static int choose_shape(bool big_ok, int M, int N) {
   if (!big_ok) return 1;
-  const int bm[5] = {0, 128, 128, 256, 256}, bn[5] = {0, 128, 256, 256, 192};
-  const double rate[5] = {0, 0.80, 0.93, 1.15, 1.00};
   int best = 1;
   double best_cost = 0;
   for (int shape = 1; shape <= 4; ++shape) {
-    const long tiles = (long)tw_div_up(M, bm[shape]) * tw_div_up(N, bn[shape]);
-    const double cost = (double)tw_div_up(tiles, 256) * bm[shape] * bn[shape] / rate[shape];
+    const long tiles = (long)tw_div_up(M, kTileM[shape]) * tw_div_up(N, kTileN[shape]);
+    const double cost = (double)tw_div_up(tiles, 256) * kTileM[shape] * kTileN[shape] / kTileRate[shape];
     if (shape == 1 || cost < best_cost) {
       best = shape;
       best_cost = cost;
@@ -606,30 +607,70 @@ static int choose_shape(bool big_ok, int M, int N) {
   return best;
 }
 
+// Estimated seconds of `shape` with K dealt to `splits` workgroups per tile: the rounds of workgroups
+// over 256 CUs at the shape's relative rate (4.42e-13 s per unit of tile area and element of K: a
+// 128x256 tile over K = 18,944 takes 295 us), plus, with splits, what splitk_reduce moves: the partial
+// sums written and read, the residual and the result, at the 6.5 TB/s such just-written data streams at.
+static double plan_seconds(int shape, int splits, int M, int N, int K) {
+  const long tiles = (long)tw_div_up(M, kTileM[shape]) * tw_div_up(N, kTileN[shape]);
+  double t = (double)tw_div_up(tiles * splits, 256) * kTileM[shape] * kTileN[shape] / kTileRate[shape] *
+             ((double)K / splits) * 4.42e-13;
+  if (splits > 1) t += (2.0 * splits + 2.0) * M * N * 4.0 / 6.5e12;
+  return t;
+}
+
+// Shape and K ranges of a product (splits 0: the launcher's own rule for few tiles). Beside the choice
+// above, 256x256 tiles with 2 to 4 K ranges are taken where they fill one round of CUs that whole tiles
+// leave partly idle and K is long enough to pay for the reduction: the down projection of a 2,048-token
+// prompt (N = 3,584, K = 18,944) has 224 tiles of 128x256 or 112 of 256x256; two K ranges of the latter
+// run at the large tile's rate on 224 CUs (295 -> 265 us with the reduction).
+struct TilePlan { int shape, splits; };
+static TilePlan choose_plan(bool big_ok, bool glu, int M, int N, int K, int epf) {
+  TilePlan plan = {choose_shape(big_ok, M, N), 0};
+  if (!big_ok || glu || K % 32 != 0) return plan;
+  const int own = tiled_splits(M, N, K, epf, kTileM[plan.shape], kTileN[plan.shape]);
+  double best = plan_seconds(plan.shape, own, M, N, K) * 0.95;
+  const long tiles = (long)tw_div_up(M, 256) * tw_div_up(N, 256);
+  for (int splits = 2; splits <= 4; ++splits) {
+    if (tiles * splits > 256 || K / splits < 2048) continue;
+    const double t = plan_seconds(3, splits, M, N, K);
+    if (t < best) {
+      best = t;
+      plan = {3, splits};
+    }
+  }
+  return plan;
+}
+
 template <typename T, typename OutT, bool SHUF, bool GLU>
 static int tiled_by_shape(int shape, const T* A, long lda, const T* W, long ldw, const float* bias,
                           const float* residual, long ldr, OutT* C, long ldc, float* partial,
                           long partial_bytes, int M, int N, int K, hipStream_t stream) {
   constexpr bool BIG = sizeof(T) == 2 && SHUF;
-  if (shape == 0) shape = choose_shape(BIG, M, N);
+  int splits = 0;                                   // a forced shape keeps the launcher's own rule
+  if (shape == 0) {
+    const TilePlan plan = choose_plan(BIG, GLU, M, N, K, Elem<T>::kPerFrag);
+    shape = plan.shape;
+    splits = plan.splits;
+  }
   if constexpr (BIG) {
     // bfloat16 and shuffled weights: the kernels that copy straight into LDS, if K allows
     if (K % 32 == 0 && K >= 32 && lda % 8 == 0) {
-      if (shape == 4) return launch_dma<OutT, 4, 3, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+      if (shape == 4) return launch_dma<OutT, 4, 3, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
       if constexpr ((TW_DMA_SHAPES & 8) != 0)
-        if (shape == 3) return launch_dma<OutT, 4, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+        if (shape == 3) return launch_dma<OutT, 4, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
       if constexpr ((TW_DMA_SHAPES & 4) != 0)
-        if (shape == 2) return launch_dma<OutT, 2, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+        if (shape == 2) return launch_dma<OutT, 2, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
       if constexpr ((TW_DMA_SHAPES & 2) != 0)
-        if (shape == 1) return launch_dma<OutT, 2, 2, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+        if (shape == 1) return launch_dma<OutT, 2, 2, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
     }
     if (shape == 3 || shape == 4)             // (K no multiple of 32: the register-staged 256x256 tile for both)
-      return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+      return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
   }
   if (shape == 3 || shape == 4) return TW_ERR_BAD_ARGUMENT;
   if (shape == 2)
-    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
-  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
+  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
 }
 
 template <typename T, typename OutT>
@@ -664,7 +705,13 @@ int tw_tiled_linear(int dtype, int out_f32, int shuffled, int glu, int shape, co
 
 long tw_tiled_workspace_bytes(int dtype, int rows, int N, int K) {
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
-  // split-K is used only where 128x128 tiles are chosen
+  // enough for whichever kernel runs: the 128x128 tiles' own rule, or the plan for shuffled bfloat16 weights
   const int splits = tiled_splits(rows, N, K, epf, 128, 128);
-  return splits > 1 ? (long)splits * rows * N * 4 : 0;
+  long bytes = splits > 1 ? (long)splits * rows * N * 4 : 0;
+  if (dtype == TW_DTYPE_BF16) {
+    const TilePlan plan = choose_plan(true, false, rows, N, K, epf);
+    const int s = plan.splits > 0 ? plan.splits : tiled_splits(rows, N, K, epf, kTileM[plan.shape], kTileN[plan.shape]);
+    if (s > 1 && (long)s * rows * N * 4 > bytes) bytes = (long)s * rows * N * 4;
+  }
+  return bytes;
 }

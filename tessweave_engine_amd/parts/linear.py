@@ -93,8 +93,9 @@ class Linear(Part):
                     self._ws_floats[i] = ops.linear_workspace_bytes(w.dtype, 64, rows, w.shape[1]) // 4
                 if self._ws_floats[i]:
                     ws = ctx.workspace.get("linear.splitk", (self._ws_floats[i],), torch.float32)
-            elif x.shape[0] <= 1024:
-                # a few hundred rows against a matrix with few column tiles: the tiled kernel splits K too
+            else:
+                # few tiles for the chip (a few hundred rows, or large tiles against a matrix with few
+                # columns and a long K): the tiled kernel splits K too
                 floats = ops.linear_workspace_bytes(w.dtype, x.shape[0], rows, w.shape[1]) // 4
                 if floats:
                     ws = ctx.workspace.get("linear.splitk", (floats,), torch.float32)

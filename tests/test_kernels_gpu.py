@@ -196,6 +196,31 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
         w = w_rows
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 3584, 16384), (1100, 3000, 12288), (2048, 3584, 8192)])
+def test_linear_large_tiles_over_k_ranges(ops, device, m, n, k):
+    """Many rows, few columns, long K (a down projection): the chosen plan may be 256x256 tiles whose K is
+    dealt to two to four workgroups, finished by the reduction kernel; with and without workspace."""
+    dtype = torch.bfloat16
+    x = rand((m, k), dtype, device, 1.0, seed=1)
+    w = rand((n, k), dtype, device, 0.05, seed=2)
+    bias = rand((n,), torch.float32, device, 0.5, seed=3)
+    res = rand((m, n), torch.float32, device, 1.0, seed=4)
+    want = (x.double() @ w.double().T).cpu()
+    shuffled = ops.shuffle_weight(w)
+    ws_bytes = ops.linear_workspace_bytes(dtype, m, n, k)
+    assert ws_bytes >= (2 * m * n * 4 if k >= 12288 else 0)      # long K: at least two K ranges are planned
+    ws = torch.empty(max(ws_bytes, 16) // 4, dtype=torch.float32, device=device)
+    scale = math.sqrt(k) * 0.05
+    for workspace in (ws, None):
+        out = torch.full((m, n), float("nan"), dtype=dtype, device=device)
+        ops.linear(x, shuffled, out, workspace=workspace)
+        torch.testing.assert_close(out.double().cpu(), want, atol=2e-2 * scale, rtol=2e-2)
+        acc = res.clone()
+        ops.linear(x, shuffled, acc, bias=bias, residual=acc, workspace=workspace)
+        torch.testing.assert_close(acc.double().cpu(), want + bias.double().cpu() + res.double().cpu(),
+                                   atol=2e-5 * scale + 1e-5, rtol=1e-5)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 389, 2048), (17, 130, 4096), (64, 96, 9472)])
 def test_linear_partials(ops, device, dtype, m, n, k):
