@@ -293,9 +293,7 @@ static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const f
       A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
   int err = TW_LAUNCH_RESULT();
   if (err || splits == 1 || PARTIAL) return err;
-  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
-                                                                             ldr, C, ldc, M, N);
-  return TW_LAUNCH_RESULT();
+  return launch_splitk_reduce<OutT>(partial, splits, bias, residual, ldr, C, ldc, M, N, stream);
 }
 
 template <typename T, typename OutT, bool PARTIAL, bool SHUF, bool GLU>

@@ -542,9 +542,7 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
                                            (int)n_blocks, splits, partial);
   int err = TW_LAUNCH_RESULT();
   if (err || splits == 1) return err;
-  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
-                                                                             ldr, C, ldc, M, N);
-  return TW_LAUNCH_RESULT();
+  return launch_splitk_reduce<OutT>(partial, splits, bias, residual, ldr, C, ldc, M, N, stream);
 }
 
 
@@ -575,9 +573,7 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
                                            (int)n_blocks, splits, partial);
   int err = TW_LAUNCH_RESULT();
   if (err || splits == 1) return err;
-  splitk_reduce_kernel<OutT><<<tw_div_up((long)M * N, 256), 256, 0, stream>>>(partial, splits, bias, residual,
-                                                                             ldr, C, ldc, M, N);
-  return TW_LAUNCH_RESULT();
+  return launch_splitk_reduce<OutT>(partial, splits, bias, residual, ldr, C, ldc, M, N, stream);
 }
 
 // Which tile (1: 128x128, 2: 128x256, 3: 256x256, 4: 256x192): the one with the least estimated time,
