@@ -463,3 +463,171 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, device):
         stepper.close()
     finally:
         unregister_architecture("ToyDecayForCausalLM")
+
+
+# ---- more toy parts defined here: a feed-forward with routing, another position encoding, a windowed layer ----
+def test_toy_routed_feed_forward_scaled_partial_rotary_and_a_window(tmp_path, device):
+    """Built from outside the package: a feed-forward that routes each token to one of two SwiGLU experts
+    (softmax gate, top 1), a position encoding that rotates only half of each head with positions divided
+    by a factor, and a layer whose attention sees a window of 12 keys beside a layer that sees all of them
+    (two cache groups; the window's pages return while the request runs). Float32, prompt portions and
+    decoded tokens of two requests in one batch, against plain formulas written out below."""
+    from dataclasses import dataclass
+    from safetensors.torch import save_file
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.config import register_architecture, unregister_architecture
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.kernels import ops
+    from tessweave_engine_amd.parts import (DecoderModel, FeedForward, GroupedQueryAttention, LayerRun, OutputHead,
+                                            PositionEncoding, PreNormBlock, RMSNorm, SwiGLU, TokenEmbedding,
+                                            fold_pending)
+    from tessweave_engine_amd.weights import VECTOR, TensorSpec, load_model, random_tensors
+
+    H, HEADS, KV, D, ROT, FACTOR, THETA, WINDOW, INTER, VOCAB = 48, 3, 1, 16, 8, 4.0, 1000.0, 12, 40, 53
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str = "ToyRoutedForCausalLM"
+        vocab_size: int = VOCAB
+        max_position_embeddings: int = 256
+        eos_token_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return dict(architectures=[self.architecture], model_type="toy_routed", vocab_size=self.vocab_size)
+
+    class ScaledPartialRotary(PositionEncoding):
+        """cos/sin of (position / factor) * theta^(-2j/rot) for the first `rot` elements of a head."""
+        graph_safe = False                                     # written with torch operations
+
+        def __init__(self, rot, theta, factor):
+            self.rotary_dim, self.theta, self.factor = rot, theta, factor
+
+        def tables(self, ctx):
+            hit = ctx.shared.get(("toy-rotary", id(self)))
+            if hit is None:
+                inv = self.theta ** (-torch.arange(0, self.rotary_dim, 2, dtype=torch.float32, device=ctx.device) / self.rotary_dim)
+                angle = (ctx.positions.float() / self.factor)[:, None] * inv[None, :]
+                hit = ctx.shared[("toy-rotary", id(self))] = (angle.cos().contiguous(), angle.sin().contiguous())
+            return hit
+
+    class RoutedSwiGLU(FeedForward):
+        """x += p_e(h) * expert_e(h), e = argmax of softmax(router @ h) (lowest index on ties)."""
+        graph_safe = False
+
+        def __init__(self, prefix, hidden, inter, experts):
+            self.prefix, self.hidden = prefix, hidden
+            self.experts = [SwiGLU(f"{prefix}experts.{e}.", hidden, inter) for e in range(experts)]
+
+        def parts(self):
+            return list(self.experts)
+
+        def tensor_specs(self):
+            router = TensorSpec(self.prefix + "router.weight", (len(self.experts), self.hidden), VECTOR)   # kept in float32
+            return [router] + [s for e in self.experts for s in e.tensor_specs()]
+
+        def bind(self, tensors, dtype, device):
+            self.router = tensors.pop(self.prefix + "router.weight").float()
+            for e in self.experts:
+                e.bind(tensors, dtype, device)
+
+        def forward(self, ctx, h, x):
+            probs = torch.softmax(h.float() @ self.router.T, -1)            # router logits in float32
+            choice = probs.argmax(-1)
+            for e, expert in enumerate(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                out = torch.zeros(rows.numel(), self.hidden, dtype=torch.float32, device=x.device)
+                fold_pending(out, expert.forward(ctx, h[rows].contiguous(), out))
+                x[rows] += probs[rows, e, None] * out
+            return None
+
+    def build_toy(c):
+        emb = TokenEmbedding("emb", c.vocab_size, H)
+        rotary = ScaledPartialRotary(ROT, THETA, FACTOR)
+        blocks = [PreNormBlock(RMSNorm(f"l{i}.n1", H, 1e-5),
+                               GroupedQueryAttention(f"l{i}.att.", H, HEADS, KV, D, rotary, qkv_bias=(i == 0), window=window),
+                               RMSNorm(f"l{i}.n2", H, 1e-5), RoutedSwiGLU(f"l{i}.ff.", H, INTER, 2))
+                  for i, window in enumerate((WINDOW, None))]
+        return DecoderModel(c, emb, blocks, RMSNorm("final", H, 1e-5), OutputHead("head", c.vocab_size, H, tied_to=emb))
+
+    register_architecture("ToyRoutedForCausalLM", "toy_routed", ToyConfig, build_toy)
+    try:
+        cfg = ToyConfig()
+        (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+        tensors = random_tensors(build_toy(cfg).tensor_specs(), 5, std=0.3)
+        save_file(tensors, str(tmp_path / "model.safetensors"))
+        model = load_model(tmp_path, dtype="float32", device="cuda:0")
+        layout = model.cache_layout()
+        assert len(layout.groups) == 2 and not model.graph_safe_model          # a windowed group beside a full one
+        w = {k: v.float() for k, v in tensors.items()}
+
+        def rotate(t, pos):
+            inv = THETA ** (-torch.arange(0, ROT, 2, dtype=torch.float32) / ROT)
+            angle = (pos.float() / FACTOR)[:, None] * inv[None, :]
+            cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+            lo, hi, rest = t[..., :ROT // 2], t[..., ROT // 2:ROT], t[..., ROT:]
+            return torch.cat((lo * cos - hi * sin, hi * cos + lo * sin, rest), -1)
+
+        def plain_toy(tokens):
+            x = w["emb.weight"][torch.tensor(tokens)]
+            t, pos = len(tokens), torch.arange(len(tokens))
+            used = set()
+            for i, window in enumerate((WINDOW, None)):
+                p = f"l{i}."
+                hn = plain.rms_norm(x, w[p + "n1.weight"], 1e-5)
+                q, k, v = (hn @ w[p + f"att.{n}_proj.weight"].T + (w[p + f"att.{n}_proj.bias"] if i == 0 else 0.0) for n in "qkv")
+                q, k = rotate(q.reshape(t, HEADS, D), pos), rotate(k.reshape(t, KV, D), pos)
+                att = plain.attention(q, k, v.reshape(t, KV, D), pos, window=window)
+                x = x + att.reshape(t, HEADS * D) @ w[p + "att.o_proj.weight"].T
+                hn = plain.rms_norm(x, w[p + "n2.weight"], 1e-5)
+                probs = torch.softmax(hn @ w[p + "ff.router.weight"].T, -1)
+                rows = []
+                for r in range(t):
+                    e = int(probs[r].argmax())
+                    used.add((i, e))
+                    rows.append(probs[r, e] * plain.swiglu(hn[r:r + 1], w[p + f"ff.experts.{e}.gate_proj.weight"],
+                                                            w[p + f"ff.experts.{e}.up_proj.weight"],
+                                                            w[p + f"ff.experts.{e}.down_proj.weight"])[0])
+                x = x + torch.stack(rows)
+            return plain.rms_norm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T, used
+
+        g = torch.Generator().manual_seed(2)
+        seqs = {name: torch.randint(0, VOCAB, (n,), generator=g).tolist() for name, n in (("a", 45), ("b", 30))}
+        wants = {name: plain_toy(toks) for name, toks in seqs.items()}
+        assert set().union(*(u for _, u in wants.values())) == {(0, 0), (0, 1), (1, 0), (1, 1)}   # every routing branch runs
+        page = 4
+        cache = CacheManager(layout, page, 24, 2, dtype="float32", device=model.device, prefix_cache=False,
+                             max_request_tokens=48)
+        stepper = Stepper(model, cache, max_step_tokens=32)
+        a, b = cache.open("a"), cache.open("b")
+        got = {"a": [], "b": []}
+
+        def run(*items):
+            entries = [StepEntry(seq, seqs[name][lo:hi], list(range(hi - lo))) for name, seq, lo, hi in items]
+            out, row = stepper.step(entries).cpu(), 0
+            for name, _, lo, hi in items:
+                got[name].append(out[row:row + hi - lo].clone())
+                row += hi - lo
+        run(("a", a, 0, 17))
+        run(("a", a, 17, 18), ("b", b, 0, 11))               # a decodes beside b's prompt portion
+        run(("b", b, 11, 30), ("a", a, 18, 19))
+        free_before = [len(p.free) for p in cache.pools]
+        for t in range(19, 45):
+            run(("a", a, t, t + 1))
+        for name in seqs:
+            torch.testing.assert_close(torch.cat(got[name]), wants[name][0], atol=3e-5, rtol=3e-5)
+        # the windowed group gave pages back while request a went on; the full group only took more
+        windowed = [g for g, grp in enumerate(layout.groups) if grp.spec.window][0]
+        held = [len(a.tables[g]) - sum(1 for p in a.tables[g] if p < 0) for g in range(2)]
+        assert held[windowed] <= WINDOW // page + 2 < held[1 - windowed]
+        assert len(cache.pools[1 - windowed].free) < free_before[1 - windowed]
+        cache.close(a), cache.close(b)
+        cache.check()
+        stepper.close()
+    finally:
+        unregister_architecture("ToyRoutedForCausalLM")
