@@ -514,3 +514,33 @@ def test_random_arrivals_cancellations_and_both_ways_of_reading(seed):
         results.append(out)
     assert {i: v for i, v in results[0].items() if v[1] is not None and results[1][i][1] is not None} == \
            {i: v for i, v in results[1].items() if v[1] is not None and results[0][i][1] is not None}
+
+
+def test_adaptive_portions_follow_the_measured_time_within_their_bounds():
+    """The reference's feedback (flow_engine/engine.py:262-268): an EMA (0.8 / 0.2) of milliseconds per prompt
+    token, the next portion = target / EMA, kept within [min_prefill_chunk, prefill_chunk]. Off by default."""
+    e, s = make(prefill_chunk=64, min_prefill_chunk=4, target_step_ms=10.0, adaptive_chunk=True, max_context=128,
+                kv_blocks=64)
+    assert e.chunk == 64
+    e._adapt_chunk(64.0, 64)                    # 1 ms a token: 10 tokens fit the target
+    assert e.chunk == 10
+    e._adapt_chunk(6.4, 64)                     # EMA 0.8 * 1 + 0.2 * 0.1 = 0.82
+    assert e.chunk == 12
+    for _ in range(60):
+        e._adapt_chunk(0.64, 64)                # ever faster: capped at prefill_chunk
+    assert e.chunk == 64
+    for _ in range(60):
+        e._adapt_chunk(6400.0, 64)              # ever slower: never below min_prefill_chunk
+    assert e.chunk == 4
+    # the next prompt portion has that size, and the prompt still completes
+    r = e.submit(list(range(1, 40)), 3)
+    e.step()
+    assert s.batches[-1] == [(r.seq.id, 0, 4, [])]
+    drain(e)
+    assert r.output == expected(list(range(1, 40)), 3)
+    e.close()
+    fixed, s2 = make(prefill_chunk=8, min_prefill_chunk=1)
+    r2 = fixed.submit(list(range(1, 30)), 2)
+    drain(fixed)
+    assert fixed.chunk == 8 and all(n <= 8 for batch in s2.batches for (_, _, n, _) in batch)
+    fixed.close()
