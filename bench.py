@@ -132,13 +132,16 @@ def serve_run(model, torch, args):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     requests, nxt, steps0 = [], 0, engine.stats()["steps"]
-    while nxt < n or engine.active or engine.waiting or engine._inflight is not None:
+    while True:
         now = time.perf_counter() - t0
         while nxt < n and arrivals[nxt] <= now:
             requests.append(engine.submit(prompts[nxt], max_tokens=outputs, ignore_eos=True))
             nxt += 1
-        if not engine.step() and nxt < n:
-            time.sleep(max(0.0, min(0.001, arrivals[nxt] - (time.perf_counter() - t0))))
+        if engine.step():                       # False: nothing admitted and no token unread
+            continue
+        if nxt == n:
+            break
+        time.sleep(max(0.0, min(0.001, arrivals[nxt] - (time.perf_counter() - t0))))
     engine.flush()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
