@@ -34,7 +34,7 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p
 }
 
 // =====================================================================================
-// Skinny kernel (M <= 16*MT rows), workgroup-cooperative. The 4 waves of a workgroup own 4
+// Skinny kernel (M <= 16*MT rows), workgroup-cooperative. The WAVES (4, or 2) waves of a workgroup own
 // neighbouring tiles of 16 output columns and the SAME K range. Per stage of U
 // MFMA steps the workgroup copies the activations' K slice [16*MT rows][U*64 B]
 // to LDS once (instead of every wave reading it from L2); each wave streams its
@@ -48,9 +48,11 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p
 // PARTIAL: always write float32 partial sums partial[split][M][N] (splits >= 1), no epilogue.
 // SHUF: W is in the shuffled layout (ldw = its k_steps): every weight load is 1 KB of consecutive
 // memory, needs no predicate (the layout is zero padded) and bypasses the caches.
-// GLU (splits == 1 only): the workgroup's 4 tiles are gate, up, gate, up; C gets 32 columns.
-template <typename T, typename OutT, int MT, int U, bool PARTIAL, bool SHUF, bool GLU>
-__global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restrict__ A, long lda,
+// GLU (splits == 1 only): the workgroup's tiles are gate, up(, gate, up); C gets half as many columns.
+// WAVES = 2 halves the workgroups' size and doubles their number: used where that spreads them more
+// evenly over the CUs (the kernel's time is that of the fullest CU).
+template <typename T, typename OutT, int MT, int U, int WAVES, bool PARTIAL, bool SHUF, bool GLU>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const T* __restrict__ A, long lda,
                                                               const T* __restrict__ W, long ldw,
                                                               const float* __restrict__ bias,
                                                               const float* residual, long ldr, OutT* C,
@@ -60,14 +62,15 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
   constexpr int EPF = Elem<T>::kPerFrag;
   constexpr int XROW = TW_XROW(U);
   constexpr int XSTAGE = MT * 16 * XROW;
-  constexpr int XLOADS = MT * U / 4;                   // activation fragments per thread per stage
-  static_assert(U % 4 == 0, "a stage is copied by 256 threads in whole rounds");
+  constexpr int THREADS = WAVES * 64;
+  constexpr int XLOADS = MT * U / WAVES;               // activation fragments per thread per stage
+  static_assert(U % 4 == 0 && (WAVES == 4 || WAVES == 2), "a stage is copied by all threads in whole rounds");
   __shared__ __attribute__((aligned(16))) char lds[2 * XSTAGE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int group = blockIdx.x % n_groups, split = blockIdx.x / n_groups;
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = group * 64 + wave * 16;
+  const int n0 = group * (16 * WAVES) + wave * 16;
 
   const int chunks = K / EPF;
   const int steps = (chunks + 3) / 4;
@@ -82,12 +85,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
 
   const T* w_row = SHUF ? W + ((size_t)min(n0 / 16, (N + 15) / 16 - 1) * ldw * 64 + lane) * EPF
                         : W + (size_t)min(n0 + r, N - 1) * ldw;
-  // this thread's share of the activation slice: fragment f = i*256 + tid -> (row f / (4U), chunk f % (4U))
+  // this thread's share of the activation slice: fragment f = i*THREADS + tid -> (row f / (4U), chunk f % (4U))
   const T* x_src[XLOADS];
   int x_dst[XLOADS], x_chunk[XLOADS];
 #pragma unroll
   for (int i = 0; i < XLOADS; ++i) {
-    const int f = i * 256 + tid, row = f / (4 * U), c = f % (4 * U);
+    const int f = i * THREADS + tid, row = f / (4 * U), c = f % (4 * U);
     x_src[i] = A + (size_t)min(row, M - 1) * lda;
     x_chunk[i] = c;
     x_dst[i] = row * XROW + c * 16;
@@ -167,7 +170,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
     // the waves swap their tiles through LDS (every wave is past its last LDS read: the loop
     // ends with a barrier), then each thread forms outputs from a (gate, up) pair
     constexpr int GROW = 17;                                  // floats per staged row, padded
-    static_assert(4 * MT * 16 * GROW * 4 <= 2 * XSTAGE, "the GLU exchange fits the pipeline's LDS");
+    static_assert(WAVES * MT * 16 * GROW * 4 <= 2 * XSTAGE, "the GLU exchange fits the pipeline's LDS");
     float* ex = reinterpret_cast<float*>(lds);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -177,9 +180,10 @@ __global__ __launch_bounds__(256) void gemm_skinny_lds_kernel(const T* __restric
         ex[(wave * MT * 16 + mt * 16 + r) * GROW + 4 * g + j] = acc[mt][j] + (bias && col < N ? bias[col] : 0.f);
       }
     __syncthreads();
-    for (int o = tid; o < MT * 16 * 32; o += 256) {
-      const int row = o >> 5, c = o & 31, pair = c >> 4, i = c & 15;
-      const int col = group * 32 + c;                         // output column
+    constexpr int OUT_COLS = 8 * WAVES;                       // output columns of the workgroup
+    for (int o = tid; o < MT * 16 * OUT_COLS; o += THREADS) {
+      const int row = o / OUT_COLS, c = o % OUT_COLS, pair = c >> 4, i = c & 15;
+      const int col = group * OUT_COLS + c;                   // output column
       if (row >= M || col >= N / 2) continue;
       const float gv = ex[((2 * pair) * MT * 16 + row) * GROW + i];
       const float uv = ex[((2 * pair + 1) * MT * 16 + row) * GROW + i];
@@ -277,20 +281,37 @@ extern "C" long tw_linear_workspace_bytes(int dtype, int max_rows, int N, int K)
   return bytes;
 }
 
+// The fullest CU's share of `workgroups` spread over 256 CUs, relative to an even spread.
+static double cu_imbalance(long workgroups) {
+  return workgroups <= 256 ? 1.0 : (double)tw_div_up(workgroups, 256) * 256.0 / (double)workgroups;
+}
+
 template <typename T, typename OutT, int MT, bool PARTIAL, bool SHUF, bool GLU>
 static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const float* bias,
                              const float* residual, long ldr, OutT* C, long ldc, float* partial,
                              long partial_bytes, int M, int N, int K, hipStream_t stream) {
   constexpr int EPF = Elem<T>::kPerFrag;
   constexpr int U = MT == 1 ? 8 : 4;
-  const int groups = tw_div_up(N, 64);
   int splits = GLU ? 1 : skinny_lds_splits(N, K, EPF);
   if (PARTIAL) {
     TW_REQUIRE(partial != nullptr && partial_bytes >= (long)splits * M * N * 4);
   } else if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4)) {
     splits = 1;
   }
-  gemm_skinny_lds_kernel<T, OutT, MT, U, PARTIAL, SHUF, GLU><<<groups * splits, 256, 0, stream>>>(
+  // One K range and at most 16 rows (the gated projection of a decode step, the head): workgroups of two
+  // waves where twice as many of them lie more evenly on the CUs (N = 37,888: 592 workgroups are 2.3 a CU,
+  // three on some; 1,184 are 4.6, five on some). With more rows every workgroup stages its own copy of
+  // the activations, so the larger workgroups stay.
+  if constexpr (MT == 1 && !PARTIAL) {
+    if (splits == 1 && cu_imbalance(tw_div_up(N, 32)) < cu_imbalance(tw_div_up(N, 64)) - 0.03) {
+      const int groups = tw_div_up(N, 32);
+      gemm_skinny_lds_kernel<T, OutT, MT, U, 2, PARTIAL, SHUF, GLU><<<groups, 128, 0, stream>>>(
+          A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, 1);
+      return TW_LAUNCH_RESULT();
+    }
+  }
+  const int groups = tw_div_up(N, 64);
+  gemm_skinny_lds_kernel<T, OutT, MT, U, 4, PARTIAL, SHUF, GLU><<<groups * splits, 256, 0, stream>>>(
       A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, M, N, K, groups, splits);
   int err = TW_LAUNCH_RESULT();
   if (err || splits == 1 || PARTIAL) return err;

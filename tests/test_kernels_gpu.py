@@ -149,6 +149,7 @@ LINEAR_SHAPES = [  # m, n, k
     (64, 256, 512), (65, 200, 136), (130, 389, 64), (300, 520, 776),
     (130, 96, 4096), (257, 260, 2056),      # few tiles, long K: the tiled kernel splits K as well
     (300, 520, 800), (513, 300, 4128),      # K a multiple of 32: the larger tiles copy straight into LDS
+    (8, 18950, 64), (16, 18944, 32),        # few rows, one K range, many columns: workgroups of two waves
 ]
 
 
@@ -241,7 +242,8 @@ def test_linear_partials(ops, device, dtype, m, n, k):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 64), (8, 208, 320), (17, 48, 1032), (64, 1040, 256), (65, 80, 64),
-                                       (200, 400, 320), (130, 16, 101), (520, 272, 200), (520, 272, 320)])
+                                       (200, 400, 320), (130, 16, 101), (520, 272, 200), (520, 272, 320),
+                                       (8, 9472, 64), (3, 9488, 96)])     # so many columns that few rows run in workgroups of two waves
 def test_linear_glu(ops, device, dtype, m, inter, k):
     """silu(x gate^T + b) * (x up^T + b) from interleaved rows, every kernel and both layouts."""
     x = rand((m, k), dtype, device, 1.0, seed=1)
