@@ -1097,15 +1097,26 @@ static int check_common(const AttnArgs& a) {
   return 0;
 }
 
+// Key ranges per (sequence, kv head) of the decode kernel. One workgroup per CU is enough to stream (a
+// wave keeps two 16 KB blocks in flight), and the kernel's time is that of the fullest CU: with `units`
+// (sequence, kv head) pairs and s ranges each, ceil(units * s / 256) rounds of 1 / s of a pair's keys.
+// The s with the least of that is taken, a percent per range added for the merge (288 workgroups, a
+// few more than CUs, would take twice as long as 240).
 extern "C" int tw_attn_decode_splits(int n_seqs, int q_heads, int kv_heads, int max_kv_len) {
   const int G = q_heads / kv_heads;
-  const int units = n_seqs * kv_heads * ((G + 15) / 16);
-  // one workgroup per CU is enough: a wave keeps two 16 KB blocks in flight
-  int splits = tw_div_up(256, units > 0 ? units : 1);
-  const int by_len = tw_div_up(max_kv_len, 256);
-  if (splits > by_len) splits = by_len;
-  if (splits > 64) splits = 64;
-  return splits < 1 ? 1 : splits;
+  const long units = (long)n_seqs * kv_heads * ((G + 15) / 16);
+  int most = tw_div_up(max_kv_len, 256);                   // at least 256 keys a range
+  if (most > 64) most = 64;
+  int best = 1;
+  double best_cost = 0;
+  for (int s = 1; s <= most; ++s) {
+    const double cost = (double)tw_div_up(units * s, 256) / s * (1.0 + 0.01 * s);
+    if (s == 1 || cost < best_cost) {
+      best = s;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 extern "C" long tw_attn_decode_workspace_floats(int n_seqs, int q_heads, int head_dim, int splits) {
