@@ -507,6 +507,8 @@ static int tiled_splits(int M, int N, int K, int epf, int bm, int bn) {
   if (tiles >= 192) return 1;
   const int k_tiles = tw_div_up(K, 8 * epf);
   long splits = tw_div_up(384, tiles);
+  const long resident = (long)bm * bn <= 128 * 128 ? 512 : 256;   // workgroups the chip holds at once
+  if (splits > resident / tiles) splits = resident / tiles;       // never a few more than that: a second round
   if (splits > k_tiles / 8) splits = k_tiles / 8;
   if (splits > 8) splits = 8;
   return splits < 1 ? 1 : (int)splits;
