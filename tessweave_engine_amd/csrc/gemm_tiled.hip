@@ -618,7 +618,7 @@ static double plan_seconds(int shape, int splits, int M, int N, int K) {
 }
 
 // Shape and K ranges of a product (splits 0: the launcher's own rule for few tiles). Beside the choice
-// above, 256x256 tiles with 2 to 8 K ranges are taken where they fill one round of CUs that whole tiles
+// above, 128x256 or 256x256 tiles with 2 to 8 K ranges are taken where they fill one round of CUs that whole tiles
 // leave partly idle and K is long enough to pay for the reduction: the down projection of a 2,048-token
 // prompt (N = 3,584, K = 18,944) has 224 tiles of 128x256 or 112 of 256x256; two K ranges of the latter
 // run at the large tile's rate on 224 CUs (295 -> 265 us with the reduction).
@@ -628,13 +628,15 @@ static TilePlan choose_plan(bool big_ok, bool glu, int M, int N, int K, int epf)
   if (!big_ok || glu || K % 32 != 0) return plan;
   const int own = tiled_splits(M, N, K, epf, kTileM[plan.shape], kTileN[plan.shape]);
   double best = plan_seconds(plan.shape, own, M, N, K) * 0.95;
-  const long tiles = (long)tw_div_up(M, 256) * tw_div_up(N, 256);
-  for (int splits = 2; splits <= 8; ++splits) {
-    if (tiles * splits > 256 || K / splits < 2048) continue;
-    const double t = plan_seconds(3, splits, M, N, K);
-    if (t < best) {
-      best = t;
-      plan = {3, splits};
+  for (int shape = 2; shape <= 3; ++shape) {               // 128x256 and 256x256: one workgroup a CU
+    const long tiles = (long)tw_div_up(M, kTileM[shape]) * tw_div_up(N, kTileN[shape]);
+    for (int splits = 2; splits <= 8; ++splits) {
+      if (tiles * splits > 256 || K / splits < 2048) continue;
+      const double t = plan_seconds(shape, splits, M, N, K);
+      if (t < best) {
+        best = t;
+        plan = {shape, splits};
+      }
     }
   }
   return plan;
