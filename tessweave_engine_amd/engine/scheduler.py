@@ -29,7 +29,6 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-import math
 import queue
 import threading
 import time
