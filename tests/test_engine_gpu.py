@@ -94,6 +94,48 @@ def test_long_decoding_and_the_first_tokens(tiny):
         stepper.close()
 
 
+def test_a_cache_full_of_nan_changes_nothing(tiny):
+    """Every page starts as NaN, as memory that is only reserved may: pages a request does not own and the
+    unused tail of its last page are never read into a result (the kernels' loads carry no predicate, so
+    this is the masks' work). Prompt portions, single tokens and a mixed batch, both precisions."""
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.weights import load_model
+    page = tiny["page"]
+    a_tokens, b_tokens = prompts_for(tiny, [2 * page + 3, page + 1], seed=33)
+    want = {"a": plain.forward(tiny["config"], tiny["weights"], a_tokens),
+            "b": plain.forward(tiny["config"], tiny["weights"], b_tokens)}
+    for dtype in ("float32", "bfloat16"):
+        model = load_model(tiny["folder"], dtype=dtype, device="cuda:0")
+        cache = CacheManager(model.cache_layout(), page, 12, 2, dtype=dtype, device=model.device, prefix_cache=False,
+                             max_request_tokens=4 * page)
+        for pool in cache.storage:
+            pool.fill_(float("nan"))
+        stepper = Stepper(model, cache, max_step_tokens=64, use_graphs=False)
+        a, b = cache.open("a"), cache.open("b")
+        got = {"a": [], "b": []}
+
+        def run(*items):
+            entries = [StepEntry(seq, toks[lo:hi], list(range(hi - lo))) for _, seq, toks, lo, hi in items]
+            out, row = stepper.step(entries).cpu(), 0
+            for name, _, _, lo, hi in items:
+                got[name].append(out[row:row + hi - lo].clone())
+                row += hi - lo
+        run(("a", a, a_tokens, 0, page - 1))                              # ends inside the first page
+        run(("a", a, a_tokens, page - 1, page + 2), ("b", b, b_tokens, 0, 1))   # crosses a page edge beside a first token
+        run(("b", b, b_tokens, 1, page + 1), ("a", a, a_tokens, page + 2, page + 3))
+        for t in range(page + 3, len(a_tokens)):
+            run(("a", a, a_tokens, t, t + 1))
+        for name in got:
+            have = torch.cat(got[name])
+            assert torch.isfinite(have).all(), (tiny["name"], dtype, name)
+            if dtype == "float32":
+                torch.testing.assert_close(have, want[name], atol=5e-6, rtol=2e-5)
+            else:
+                assert float((have - want[name]).abs().max()) <= 0.02 * float(want[name].abs().max())
+        stepper.close()
+
+
 def test_sampling_seed_is_independent_of_other_requests(tiny):
     """tests/test_engine.py:251-260 of the reference, with the device sampler."""
     p = prompts_for(tiny, [5, 4], seed=2)
