@@ -165,12 +165,30 @@ class CacheManager:
         seq.tables[0] = list(shared)
         self.table_rows[0][seq.state_slot, :len(shared)] = shared
         seq.computed = seq.cached = len(shared) * self.page_size
-        pool.hits += seq.cached
         return seq.cached
 
-    def publish(self, seq, tokens, namespace="local"):
+    def admit(self, seq_id, prompt, total_tokens, largest_step, namespace="local"):
+        """Open a request, share what the prefix index holds of PROMPT and promise it every further page
+        that TOTAL_TOKENS can need. Raises CapacityError, with nothing held and nothing evicted, if a
+        request slot or the pages are not to be had now. Prefix hits are counted only for admitted requests
+        (flow_engine/engine.py:109)."""
+        seq = self.open(seq_id)
+        try:
+            self.acquire_prefix(seq, prompt, namespace)
+            self.reserve(seq, total_tokens, largest_step)
+        except CapacityError:
+            self.close(seq)
+            raise
+        if seq.cached:
+            self.pools[0].hits += seq.cached
+        return seq
+
+    def publish(self, seq, tokens, namespace="local", computed=None):
+        """Offer the full blocks of TOKENS that SEQ holds keys and values for (its first COMPUTED tokens,
+        by default everything it has computed) to the prefix index."""
         if self.prefix_cache:
-            self.pools[0].publish(tokens, seq.computed, seq.tables[0], namespace)
+            upto = seq.computed if computed is None else min(int(computed), seq.computed)
+            self.pools[0].publish(tokens, upto, seq.tables[0], namespace)
 
     def first_needed_block(self, group, computed):
         """First logical block of GROUP that a query at position >= COMPUTED can see."""

@@ -1,25 +1,49 @@
-"""Host-side ownership of one group's physical pages.
+"""Who owns which physical page of one cache group (host side only; no tensors here).
 
-Reference behaviour followed (flow_engine/cache.py:24-91): a reference count per
-page, a LIFO free list, `allocate` evicting least-recently-used prefix entries
-when the free list is short, `release` with an underflow check, and a prefix
-index keyed by chained SHA-256 over (namespace, parent key, the block's tokens
-as little-endian int64); only full blocks are keyed, lookup never covers the
-last prompt token, a page is free only when neither a request nor the index
-holds it.
+A page carries a use count: one for every live request whose block table names
+it and one if the prefix index names it. It is on the free list exactly while
+that count is zero. Requests may also be PROMISED pages: a promise sets free
+pages aside without choosing them, and is redeemed page by page as the request
+grows, so a request admitted with a promise for its worst case can never be
+starved by later arrivals.
 
-Added: `promised` pages. A request may be promised pages at admission that it
-takes later, one by one; promised pages cannot be given to anyone else.
+The prefix index maps the key of a FULL block of tokens to the page that holds
+its keys and values. The key format is a contract shared with the reference
+(flow_engine/cache.py:60-65): the root is sha256(namespace), and every block's
+key is sha256(parent key + the block's token ids as little-endian int64), so a
+key names the whole prefix up to and including its block. What the reference
+fixes besides the format: lookups never cover a prompt's last token, whose
+logits must be computed (cache.py:69-70); a hit refreshes an entry's age
+(cache.py:75); pages come off the free list last-in first-out (cache.py:25,55);
+a use count below zero is an error (cache.py:36-37).
+
+Eviction differs from the reference's (cache.py:49-54), which pops entries
+oldest first whether or not that frees anything and so can empty the index on
+behalf of a request that then still does not fit. Here a request for pages is
+first checked against what eviction COULD free; only then are entries dropped,
+oldest first, and only entries whose page nobody else uses. Within one prefix
+chain deeper blocks are kept older than their parents, so a chain is eaten from
+its tail and what stays is still reachable from the root.
 """
 from __future__ import annotations
 
 from collections import OrderedDict
 import hashlib
-import struct
 
 
 class CapacityError(RuntimeError):
     """Not enough free pages (or state slots); the caller waits or refuses."""
+
+
+def block_keys(tokens, page_size, namespace):
+    """Keys of the full blocks of TOKENS, root first."""
+    key = hashlib.sha256(namespace.encode()).digest()
+    keys = []
+    for end in range(page_size, len(tokens) + 1, page_size):
+        packed = b"".join(int(t).to_bytes(8, "little", signed=True) for t in tokens[end - page_size:end])
+        key = hashlib.sha256(key + packed).digest()
+        keys.append(key)
+    return keys
 
 
 class PagePool:
@@ -28,106 +52,113 @@ class PagePool:
             raise ValueError("pages and page_size must be positive")
         self.capacity = int(pages)
         self.page_size = int(page_size)
-        self.refs = [0] * self.capacity
-        self.free = list(reversed(range(self.capacity)))
-        self.prefixes: OrderedDict[bytes, int] = OrderedDict()
+        self.refs = [0] * self.capacity                       # use count per page
+        self.free = list(range(self.capacity - 1, -1, -1))    # a stack: page 0 is handed out first
+        self.prefixes: OrderedDict[bytes, int] = OrderedDict()   # block key -> page, oldest entry first
         self.prefix_cache = bool(prefix_cache)
         self.promised = 0
-        self.hits = 0
+        self.hits = 0            # prompt tokens served from the index (counted by whoever admits the request)
         self.evictions = 0
 
-    # ---- ownership ----------------------------------------------------
-    def _release_one(self, page):
+    # ---- use counts -------------------------------------------------------------------
+    def _use(self, page):
+        self.refs[page] += 1
+
+    def _unuse(self, page):
         if not 0 <= page < self.capacity:
             raise RuntimeError(f"page id {page} out of range")
-        if self.refs[page] <= 0:
+        left = self.refs[page] - 1
+        if left < 0:
             raise RuntimeError("KV reference underflow")
-        self.refs[page] -= 1
-        if not self.refs[page]:
+        self.refs[page] = left
+        if left == 0:
             self.free.append(page)
 
     def release(self, pages):
+        """Drop one use of every page in PAGES (-1 marks a block that is not held)."""
         for page in pages:
             if page >= 0:
-                self._release_one(page)
+                self._unuse(page)
 
-    def _evictable(self):
-        return sum(1 for page in self.prefixes.values() if self.refs[page] == 1)
+    # ---- free pages, promises, eviction -------------------------------------------------
+    def _index_only(self):
+        """Keys, oldest first, of entries whose page only the index uses."""
+        return [key for key, page in self.prefixes.items() if self.refs[page] == 1]
 
     def available(self):
         """Pages that a new promise or an unpromised allocation could still get."""
-        return len(self.free) + self._evictable() - self.promised
+        return len(self.free) + len(self._index_only()) - self.promised
 
-    def _make_room(self, count, others):
-        # Evict least-recently-used prefix entries while the free list is short
-        # (flow_engine/cache.py:49-54). An evicted entry whose page a request
-        # still holds frees nothing; the loop goes on to the next entry.
-        while len(self.free) - others < count and self.prefixes:
-            _, page = self.prefixes.popitem(last=False)
-            self._release_one(page)
-            self.evictions += 1
-        if len(self.free) - others < count:
+    def _free_up(self, count, set_aside):
+        """Make COUNT pages free beyond the SET_ASIDE ones that stay promised to others.
+
+        Raises CapacityError, and leaves the index as it is, if eviction could not free enough.
+        """
+        short = count + set_aside - len(self.free)
+        if short <= 0:
+            return
+        victims = self._index_only()
+        if len(victims) < short:
             raise CapacityError("KV capacity exhausted; request must wait or reduce its token budget")
+        for key in victims[:short]:
+            self._unuse(self.prefixes.pop(key))
+            self.evictions += 1
 
     def allocate(self, count, promised=0):
-        """Take COUNT pages; PROMISED of them were promised to the caller before."""
-        if count < 0 or promised < 0 or promised > count or promised > self.promised:
+        """Take COUNT pages; PROMISED of them redeem a promise made before."""
+        if count < 0 or not 0 <= promised <= min(count, self.promised):
             raise ValueError("negative allocation")
-        self._make_room(count, self.promised - promised)
-        result = [self.free.pop() for _ in range(count)]
-        for page in result:
-            self.refs[page] = 1
+        self._free_up(count, self.promised - promised)
         self.promised -= promised
-        return result
+        taken = [self.free.pop() for _ in range(count)]
+        for page in taken:
+            self.refs[page] = 1
+        return taken
 
     def promise(self, count):
-        """Set COUNT free pages aside for later `allocate(..., promised=...)` calls."""
+        """Set COUNT pages aside for later `allocate(..., promised=...)` calls."""
         if count < 0:
             raise ValueError("negative promise")
-        self._make_room(count, self.promised)
+        self._free_up(count, self.promised)
         self.promised += count
 
     def unpromise(self, count):
-        if count < 0 or count > self.promised:
+        if not 0 <= count <= self.promised:
             raise RuntimeError("promise underflow")
         self.promised -= count
 
-    # ---- prefix index -------------------------------------------------
-    def _keys(self, tokens, namespace):
-        parent = hashlib.sha256(namespace.encode()).digest()
-        size = self.page_size
-        for start in range(0, len(tokens) - size + 1, size):
-            chunk = tokens[start:start + size]
-            parent = hashlib.sha256(parent + struct.pack(f"<{len(chunk)}q", *chunk)).digest()
-            yield parent
-
+    # ---- prefix index -------------------------------------------------------------------
     def acquire_prefix(self, tokens, namespace="local"):
-        table = []
-        if self.prefix_cache:
-            # At least the last prompt token must run to recover its logits.
-            for key in self._keys(tokens[:-1], namespace):
-                page = self.prefixes.get(key)
-                if page is None:
-                    break
-                self.prefixes.move_to_end(key)
-                self.refs[page] += 1
-                table.append(page)
-        return table
+        """Pages of the longest indexed prefix of TOKENS, each with one more use; never the last token's block."""
+        if not self.prefix_cache:
+            return []
+        usable = (len(tokens) - 1) // self.page_size * self.page_size
+        found = []
+        for key in block_keys(tokens[:usable], self.page_size, namespace):
+            page = self.prefixes.get(key)
+            if page is None:
+                break
+            found.append((key, page))
+        for key, page in reversed(found):       # the root ends up youngest, the deepest block oldest of the chain
+            self.prefixes.move_to_end(key)
+            self._use(page)
+        return [page for _, page in found]
 
     def publish(self, tokens, computed, table, namespace="local"):
+        """Enter the full blocks of TOKENS[:COMPUTED] (pages TABLE[i]) that the index does not know yet."""
         if not self.prefix_cache:
             return
-        for i, key in enumerate(self._keys(tokens[:computed], namespace)):
-            if key not in self.prefixes and table[i] >= 0:
-                self.prefixes[key] = table[i]
-                self.refs[table[i]] += 1
+        fresh = [(key, table[i]) for i, key in enumerate(block_keys(tokens[:computed], self.page_size, namespace))
+                 if key not in self.prefixes and table[i] >= 0]
+        for key, page in reversed(fresh):
+            self.prefixes[key] = page
+            self._use(page)
 
     def clear_prefixes(self):
-        for page in self.prefixes.values():
-            self._release_one(page)
-        self.prefixes.clear()
+        while self.prefixes:
+            self._unuse(self.prefixes.popitem()[1])
 
-    # ---- checks ---------------------------------------------------------
+    # ---- checks ---------------------------------------------------------------------------
     def check(self, tables=()):
         """Raise if a page is lost, free and held at once, or counted wrongly.
 
@@ -148,5 +179,5 @@ class PagePool:
                 raise AssertionError(f"page {page}: {self.refs[page]} references counted, {held[page]} held")
             if (page in free) != (self.refs[page] == 0):
                 raise AssertionError(f"page {page} is {'free' if page in free else 'held'} with {self.refs[page]} references")
-        if self.promised < 0 or self.promised > len(self.free):
+        if not 0 <= self.promised <= len(self.free):
             raise AssertionError("more pages promised than are free")

@@ -81,40 +81,66 @@ def resolve_device_dtype(args):
     return "cuda:0", dtype
 
 
-def make_engine(args):
-    """(Engine, tokenizer or None) from parsed `generate` options."""
+_PROMPT_OPTIONS = ("--prompt", "--prompt-ids")
+
+
+def without_prompts(argv):
+    """ARGV with the value of every prompt option replaced: what a user asks never reaches a log file."""
+    shown, hide_next = [], False
+    for word in argv:
+        name, eq, _ = word.partition("=")
+        if hide_next:
+            shown.append("[REDACTED]")
+            hide_next = False
+        elif name in _PROMPT_OPTIONS and eq:
+            shown.append(name + "=[REDACTED]")
+        else:
+            shown.append(word)
+            hide_next = word in _PROMPT_OPTIONS
+    return shown
+
+
+def _engine_config(args, dtype):
     from .config import EngineConfig
+    return EngineConfig(
+        dtype=dtype, max_context=args.max_context, kv_blocks=args.kv_blocks, block_size=args.block_size,
+        max_active=args.max_active, prefix_cache=not args.no_prefix_cache,
+        prefill_chunk=args.prefill_chunk, min_prefill_chunk=min(16, args.prefill_chunk),
+        target_step_ms=args.target_step_ms, adaptive_chunk=args.adaptive_chunk,
+        max_step_tokens=args.max_step_tokens, use_graphs=not args.no_graphs, lookahead=not args.no_lookahead)
+
+
+def _chat_tokenizer(folder):
+    """The model folder's own tokenizer (files only: no model code of the library runs, nothing is fetched).
+    Without a chat template a text prompt is refused rather than wrapped in a guessed one (flow_engine/cli.py:40-42)."""
+    from transformers import AutoTokenizer
+    tokenizer = AutoTokenizer.from_pretrained(str(folder), local_files_only=True, trust_remote_code=False)
+    if not tokenizer.chat_template:
+        raise ValueError("a tokenizer chat_template is required; no template will be guessed")
+    return tokenizer
+
+
+def make_engine(args, argv=None):
+    """(Engine, tokenizer or None) from parsed `generate` options (flow_engine/cli.py:14-45).
+
+    ARGV is the command line to record in the log's first event (default: the process's own), prompts removed.
+    """
     from .engine import Engine, Trace
     from .weights import load_model
     import torch
 
     device, dtype = resolve_device_dtype(args)
-    trace = Trace(args.log)
-    argv = list(sys.argv)
-    for i, argument in enumerate(argv):            # prompts never reach the log
-        if argument in ("--prompt", "--prompt-ids") and i + 1 < len(argv):
-            argv[i + 1] = "[REDACTED]"
-        elif argument.startswith(("--prompt=", "--prompt-ids=")):
-            argv[i] = argument.split("=")[0] + "=[REDACTED]"
-    trace.emit("launch", argv=argv, python=sys.version, torch=torch.__version__, device=device, dtype=dtype)
-    print(f"Loading local weights: {args.model} ({device}, {dtype})", file=sys.stderr, flush=True)
+    engine_config = _engine_config(args, dtype)          # a bad option fails before any weight is read
     folder = Path(args.model).resolve(strict=True)
+    trace = Trace(args.log)
+    trace.emit("launch", argv=without_prompts(sys.argv if argv is None else argv), python=sys.version,
+               torch=torch.__version__, device=device, dtype=dtype)
+    print(f"reading weights from {folder} onto {device} as {dtype}", file=sys.stderr, flush=True)
     model = load_model(folder, dtype=dtype, device=device, packed=not args.unfused)
-    config = model.config
-    engine_config = EngineConfig(
-        block_size=args.block_size, kv_blocks=args.kv_blocks, max_context=args.max_context,
-        max_active=args.max_active, prefill_chunk=args.prefill_chunk,
-        min_prefill_chunk=min(16, args.prefill_chunk), target_step_ms=args.target_step_ms,
-        prefix_cache=not args.no_prefix_cache, dtype=dtype, max_step_tokens=args.max_step_tokens,
-        adaptive_chunk=args.adaptive_chunk, use_graphs=not args.no_graphs, lookahead=not args.no_lookahead)
-    tokenizer = None
-    if getattr(args, "prompt", None):
-        from transformers import AutoTokenizer          # tokenizer files only; no model code of the library runs
-        tokenizer = AutoTokenizer.from_pretrained(str(folder), local_files_only=True, trust_remote_code=False)
-        if not tokenizer.chat_template:
-            raise ValueError("a tokenizer chat_template is required; no template will be guessed")
+    tokenizer = _chat_tokenizer(folder) if getattr(args, "prompt", None) else None
     engine = Engine(model, engine_config, trace)
-    trace.emit("loaded", engine=asdict(engine_config), model=config.describe(), kv_bytes=engine.cache.allocated_bytes)
+    trace.emit("loaded", engine=asdict(engine_config), model=model.config.describe(),
+               kv_bytes=engine.cache.allocated_bytes)
     return engine, tokenizer
 
 
@@ -184,26 +210,27 @@ def main(argv=None):
         out = write_model_folder(args.out, config, args.seed, args.std, args.store_dtype)
         print(str(out))
     else:
-        engine, tokenizer = make_engine(args)
-        try:
-            ids = _prompt_ids(args, tokenizer)
-            r = engine.submit(ids, args.max_tokens, temperature=args.temperature, seed=args.seed,
-                              ignore_eos=args.ignore_eos)
-            engine.start()
-            while True:
-                event = r.events.get()
-                if event["type"] == "done":
-                    if event["error"]:
-                        raise RuntimeError(event["error"])
-                    break
-            if tokenizer is not None:
-                print(tokenizer.decode(r.output, skip_special_tokens=True))
-            else:
-                print(" ".join(str(t) for t in r.output))
-            print(json.dumps(event), file=sys.stderr)
-        finally:
-            engine.close()
+        _generate(args, ["flow-inference", *argv] if argv is not None else None)
     return 0
+
+
+def _generate(args, argv):
+    """`generate`: one request through the engine's worker thread; the tokens (or their text) on standard
+    output, the terminal event with its usage counts on standard error (flow_engine/cli.py:107-118)."""
+    engine, tokenizer = make_engine(args, argv)
+    try:
+        request = engine.submit(_prompt_ids(args, tokenizer), args.max_tokens, temperature=args.temperature,
+                                seed=args.seed, ignore_eos=args.ignore_eos)
+        engine.start()
+        verdict = next(event for event in iter(request.events.get, None) if event["type"] == "done")
+        if verdict["error"]:
+            raise RuntimeError(verdict["error"])
+        generated = request.output
+        print(tokenizer.decode(generated, skip_special_tokens=True) if tokenizer is not None
+              else " ".join(map(str, generated)))
+        print(json.dumps(verdict), file=sys.stderr)
+    finally:
+        engine.close()
 
 
 if __name__ == "__main__":

@@ -34,6 +34,8 @@ class EngineConfig:
                     "prefill_chunk", "min_prefill_chunk"):
             if getattr(self, key) <= 0:
                 raise ValueError(f"{key} must be positive")
+        if self.block_size % 4:
+            raise ValueError("block_size must be a multiple of 4: the attention kernels read a page's keys four at a time")
         if self.prefill_chunk < self.min_prefill_chunk or self.target_step_ms <= 0:
             raise ValueError("invalid prefill control bounds")
         if self.dtype not in ("bfloat16", "float32"):

@@ -4,6 +4,17 @@ The reference has no registry: it whitelists `model_type` and serves both of
 its families with one class (flow_engine/config.py:26, flow_engine/model.py:105).
 Here config.json's `architectures[0]` (or, if absent, its `model_type`) selects
 an entry; the entry's builder assembles a model out of parts.
+
+What a configuration class must offer (the engine, the loader and the command
+line read nothing else off it):
+
+    from_dict(dict) -> config      parse config.json's own keys; raise ConfigError for what is not supported
+    to_dict() -> dict              the keys back, so that a model folder can be written from a configuration
+    describe() -> dict             what `inspect` and the log show
+    architecture: str              the name it is registered under
+    vocab_size: int                token ids are checked against it
+    max_position_embeddings: int   the engine's `max_context` may not exceed it
+    eos_token_ids: tuple[int]      tokens that end a request (merged from generation_config.json if present)
 """
 from __future__ import annotations
 

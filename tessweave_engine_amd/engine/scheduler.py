@@ -8,13 +8,17 @@ turn decodes all ready requests and advances prompts round-robin
 (engine.py:249-260); the portion that completes a prompt samples the first
 token (engine.py:223-237); EOS is emitted and counted, then the request stops
 (engine.py:169-174); pages are published to the prefix index on a normal finish
-and released on any finish (engine.py:123-146).
+and released on any finish (engine.py:123-146); a consumer that lets its bounded
+event queue fill up loses the request, never the engine (engine.py:115-121).
 
 Differences: the decode tokens and the prompt portions of a turn are ONE mixed
 batch for the step function, under a token budget (`max_step_tokens`); several
 prompts may advance in a turn if the budget allows; the portion size is fixed
 unless `adaptive_chunk` asks for the reference's wall-clock feedback
-(engine.py:262-268); sampling runs on the device.
+(engine.py:262-268); sampling runs on the device; the full blocks of a prompt
+are entered into the prefix index as soon as the step that computes them has
+been issued, so requests that are live at the same time share them (the
+reference shares only what a finished request leaves, engine.py:127-128).
 
 Lookahead (`EngineConfig.lookahead`, on the GPU): a turn is put on the device
 BEFORE the tokens of the turn before it are read. A request's newest token is then
@@ -28,7 +32,8 @@ tokens a request gets are the same with and without lookahead.
 from __future__ import annotations
 
 from collections import deque
-from dataclasses import dataclass, field
+from dataclasses import dataclass
+import contextlib
 import queue
 import threading
 import time
@@ -40,28 +45,40 @@ from ..sampling.sampler import validate_temperature
 from .step import StepEntry
 from .trace import Trace
 
-FINAL = ("stop", "length", "cancelled", "error")
+#: a request's status is "waiting", "active" or the reason it ended
+ENDED_NORMALLY = ("stop", "length")
+ENDED = ENDED_NORMALLY + ("cancelled", "error")
+EVENT_QUEUE_DEPTH = 256          # flow_engine/engine.py:32
 
 
-@dataclass
 class Request:
-    id: str
-    prompt: list
-    max_tokens: int
-    temperature: float
-    seed: int
-    namespace: str
-    ignore_eos: bool = False
-    tokens: list = field(default_factory=list)       # prompt + generated
-    output: list = field(default_factory=list)       # generated
-    seq: object = None                               # cache.Sequence while admitted
-    issued: int = 0                                  # generated tokens, those still on the device included
-    feed_row: int = -1                               # row of the newest token in the sampler's output while unread
-    cached: int = 0                                  # prompt tokens taken from the prefix index
-    status: str = "waiting"
-    created: float = field(default_factory=time.perf_counter)
-    first_token: float | None = None
-    events: queue.Queue = field(default_factory=lambda: queue.Queue(maxsize=256))
+    """One generation request, from `submit` to its terminal event.
+
+    `events` carries {"type": "token", "token_id": t} for every generated token and one final
+    {"type": "done", ...}. It is bounded; a request made with stream=False has no token events (its
+    tokens are read from `output` once it has ended) and can therefore not overrun the queue.
+    """
+
+    def __init__(self, prompt, max_tokens, temperature, seed, namespace, ignore_eos, stream=True):
+        self.id = uuid.uuid4().hex
+        self.prompt = list(prompt)
+        self.max_tokens = max_tokens
+        self.temperature = temperature
+        self.seed = int(seed)
+        self.namespace = namespace
+        self.ignore_eos = bool(ignore_eos)
+        self.stream = bool(stream)
+        self.tokens = list(prompt)      # prompt + generated
+        self.output = []                # generated
+        self.seq = None                 # cache.Sequence while admitted
+        self.issued = 0                 # generated tokens, those still on the device included
+        self.feed_row = -1              # row of the newest token in the sampler's output while unread
+        self.cached = 0                 # prompt tokens taken from the prefix index
+        self.published = 0              # prompt tokens whose full blocks were offered to the prefix index
+        self.status = "waiting"
+        self.created = time.perf_counter()
+        self.first_token = None
+        self.events = queue.Queue(maxsize=EVENT_QUEUE_DEPTH)
 
     @property
     def computed(self):
@@ -70,6 +87,14 @@ class Request:
     @property
     def prefilling(self):
         return self.computed < len(self.prompt)
+
+    @property
+    def ended(self):
+        return self.status in ENDED
+
+    def usage(self):
+        n_in, n_out = len(self.prompt), len(self.output)
+        return {"prompt_tokens": n_in, "completion_tokens": n_out, "total_tokens": n_in + n_out}
 
 
 @dataclass
@@ -116,50 +141,60 @@ class Engine:
         self.prefill_cursor = 0
         self.chunk = self.config.prefill_chunk
         self.prefill_ms_per_token = None
-        self.counters = {"submitted": 0, "finished": 0, "cancelled": 0, "failed": 0,
-                         "generated_tokens": 0, "prefill_tokens": 0, "steps": 0}
+        self.counters = dict.fromkeys(("submitted", "finished", "cancelled", "failed", "generated_tokens",
+                                       "prefill_tokens", "steps"), 0)
 
     # ---- requests in -------------------------------------------------------------------
-    def submit(self, tokens, max_tokens=128, temperature=0.0, seed=0, namespace="local", ignore_eos=False):
+    def _refuse_unless_valid(self, tokens, max_tokens):
+        """What `submit` refuses for good (flow_engine/engine.py:75-82): ids outside the vocabulary, a
+        budget beyond the configured context, a request that the whole cache could not hold."""
+        vocab = self.model_config.vocab_size
+        if len(tokens) == 0:
+            raise ValueError("an empty prompt cannot be run")
+        for t in tokens:
+            if type(t) is not int or not 0 <= t < vocab:
+                raise ValueError(f"prompt token {t!r} is no id in [0, {vocab})")
+        if type(max_tokens) is not int or max_tokens < 1:
+            raise ValueError("max_tokens must be a positive integer")
+        total = len(tokens) + max_tokens
+        if total > self.config.max_context:
+            raise ValueError(f"prompt ({len(tokens)}) + max_tokens ({max_tokens}) exceeds the configured "
+                             f"context of {self.config.max_context}")
+        if not self.cache.fits(total, self.config.step_token_budget):
+            raise ValueError(f"{total} tokens need more pages than the cache has; raise --kv-blocks or ask for fewer")
+
+    def submit(self, tokens, max_tokens=128, temperature=0.0, seed=0, namespace="local", ignore_eos=False,
+               stream=True):
+        """Queue a request; returns its `Request`. ValueError: it can never run. CapacityError: the queue is full."""
         with self.lock:
             if self.fatal:
                 raise RuntimeError(f"engine failed: {self.fatal}")
-            vocab = self.model_config.vocab_size
-            if not tokens or any(type(t) is not int or t < 0 or t >= vocab for t in tokens):
-                raise ValueError("prompt must contain valid token ids")
-            if type(max_tokens) is not int or max_tokens < 1 or len(tokens) + max_tokens > self.config.max_context:
-                raise ValueError("prompt_tokens + max_tokens exceeds the configured context")
+            self._refuse_unless_valid(tokens, max_tokens)
             temperature = validate_temperature(temperature)
-            if not self.cache.fits(len(tokens) + max_tokens, self.config.step_token_budget):
-                raise ValueError("this request alone exceeds the KV pool; increase --kv-blocks or reduce tokens")
             if len(self.waiting) >= self.config.max_queue:
                 raise CapacityError("waiting queue is full")
-            r = Request(uuid.uuid4().hex, list(tokens), max_tokens, temperature, int(seed), namespace, bool(ignore_eos))
-            r.tokens = list(tokens)
+            r = Request(tokens, max_tokens, temperature, seed, namespace, ignore_eos, stream)
             self.requests[r.id] = r
             self.waiting.append(r)
             self.counters["submitted"] += 1
-            self.trace.emit("submit", request_id=r.id, prompt_tokens=len(tokens), max_tokens=max_tokens,
-                            temperature=temperature, seed=seed)
-            self.wake.set()
-            return r
+            self.trace.emit("submit", request_id=r.id, prompt_tokens=len(r.prompt), max_tokens=max_tokens,
+                            temperature=temperature, seed=r.seed)
+        self.wake.set()
+        return r
 
     def _admit(self):
-        """FIFO: the head of the queue is admitted when a request slot and all its pages can be promised."""
+        """Admit from the head of the queue while a request slot and every page the head can ever need are
+        to be had. A head that does not fit stops admission: nobody overtakes it, so it cannot starve."""
+        budget = self.config.step_token_budget
         while self.waiting and len(self.active) < self.config.max_active:
             r = self.waiting[0]
             try:
-                seq = self.cache.open(r.id)
+                r.seq = self.cache.admit(r.id, r.prompt, len(r.prompt) + r.max_tokens, budget, r.namespace)
             except CapacityError:
-                break
-            try:
-                self.cache.acquire_prefix(seq, r.prompt, r.namespace)
-                self.cache.reserve(seq, len(r.prompt) + r.max_tokens, self.config.step_token_budget)
-            except CapacityError:
-                self.cache.close(seq)
-                break       # no skipping ahead: a large request is not starved by small ones
+                return
             self.waiting.popleft()
-            r.seq, r.cached, r.status = seq, seq.cached, "active"
+            r.cached = r.published = r.seq.cached
+            r.status = "active"
             self.active.append(r)
             self.trace.emit("admit", request_id=r.id, reused_tokens=r.cached, **self.cache.stats())
 
@@ -222,6 +257,7 @@ class Engine:
                     tokens = r.tokens[begin:begin + p.count]
                 entries.append(StepEntry(r.seq, tokens, [p.count - 1] if p.samples else []))
             logits = self.stepper.step(entries)
+            self._publish_prompt_blocks(portions)
             sampled = [p for p in portions if p.samples]
             arguments = (logits, [p.request.temperature for p in sampled], [p.request.seed for p in sampled],
                          [p.request.issued for p in sampled])
@@ -256,10 +292,28 @@ class Engine:
                 self._adapt_chunk(elapsed, n_prompt)
             return True
 
+    def _publish_prompt_blocks(self, portions):
+        """Offer the prompt blocks that the step just issued completes to the prefix index.
+
+        Safe before the step has finished: whoever takes such a page reads it in a later step, and all
+        device work is ordered on one stream; the owner itself writes only beyond its computed length, so
+        a published page is never written again.
+        """
+        if not self.cache.prefix_cache:
+            return
+        page = self.cache.page_size
+        for p in portions:
+            r = p.request
+            if not p.prompt or r.seq is None or r.seq.closed:
+                continue
+            whole = min(r.computed, len(r.prompt)) // page * page
+            if whole > r.published:
+                self.cache.publish(r.seq, r.prompt[:whole], r.namespace, computed=whole)
+                r.published = whole
+
     def _sampling_stream(self):
         stream = getattr(self.stepper, "stream", None)
         if stream is None:
-            import contextlib
             return contextlib.nullcontext()
         import torch
         return torch.cuda.stream(stream)
@@ -270,7 +324,7 @@ class Engine:
             self._collect()
 
     def _collect(self, turn=None):
-        """Read the tokens a turn sampled (waiting for them if need be) and commit them to their requests."""
+        """Read the tokens a turn sampled (waiting for them if need be) and hand them to their requests."""
         if turn is None:
             turn, self._inflight = self._inflight, None
         if turn is None:
@@ -278,8 +332,8 @@ class Engine:
         pending, rows = turn
         ids = pending.result() if hasattr(pending, "result") else pending
         for r, row in rows:
-            if r.id in self.requests and r.status == "active":     # else it ended meanwhile: the token is dropped
-                self._commit(r, int(ids[row]))
+            if r.status == "active":         # else it ended meanwhile: the token is dropped
+                self._accept(r, int(ids[row]))
 
     def _adapt_chunk(self, elapsed_ms, prompt_tokens):
         # The reference's feedback (engine.py:262-268): EMA of prompt ms/token, portion sized to the turn budget.
@@ -291,96 +345,102 @@ class Engine:
         self.chunk = max(self.config.min_prefill_chunk, min(self.config.prefill_chunk, estimate))
 
     # ---- tokens out, requests out -----------------------------------------------------
-    def _emit(self, r, event):
-        try:
-            r.events.put_nowait(event)
-            return True
-        except queue.Full:
-            self._finish(r, "error", "consumer too slow; bounded output queue exhausted")
-            return False
-
-    def _commit(self, r, token):
+    def _accept(self, r, token):
+        """A sampled token reaches its request: record it, tell the consumer, and end the request if this
+        token is an EOS (it is still delivered and counted) or the last one asked for."""
+        now = time.perf_counter()
         r.tokens.append(token)
         r.output.append(token)
         self.counters["generated_tokens"] += 1
         if r.first_token is None:
-            r.first_token = time.perf_counter()
-            self.trace.emit("first_token", request_id=r.id, ttft_ms=(r.first_token - r.created) * 1000)
-        if not self._emit(r, {"type": "token", "token_id": token}):
-            return False
-        if not r.ignore_eos and token in self.model_config.eos_token_ids:
-            self._finish(r, "stop")
-            return False
-        if len(r.output) >= r.max_tokens:
-            self._finish(r, "length")
-            return False
-        return True
+            r.first_token = now
+            self.trace.emit("first_token", request_id=r.id, ttft_ms=(now - r.created) * 1000)
+        if r.stream:
+            try:
+                r.events.put_nowait({"type": "token", "token_id": token})
+            except queue.Full:
+                self._retire(r, "error", "consumer too slow; bounded output queue exhausted")
+                return
+        if token in self.model_config.eos_token_ids and not r.ignore_eos:
+            self._retire(r, "stop")
+        elif len(r.output) >= r.max_tokens:
+            self._retire(r, "length")
 
-    def _finish(self, r, reason, error=None):
-        if r.id not in self.requests:
+    def _retire(self, r, reason, error=None):
+        """The one place a request ends, for any reason: out of the engine's lists, cache given back (its
+        full blocks published first if it ended normally), counters, and the terminal event, which always
+        fits: a consumer that stopped reading loses its unread tokens, not the verdict."""
+        if r.ended:
             return
-        if r in self.active:
-            if reason not in ("error", "cancelled"):
-                self.cache.publish(r.seq, r.tokens, r.namespace)
-            self.active.remove(r)
-        elif r in self.waiting:
+        was, r.status = r.status, reason
+        self.requests.pop(r.id, None)
+        if was == "waiting":
             self.waiting.remove(r)
+        else:
+            self.active.remove(r)
         if r.seq is not None:
+            if reason in ENDED_NORMALLY:
+                self.cache.publish(r.seq, r.tokens, r.namespace)
             self.cache.close(r.seq)
             r.seq = None
-        r.status = reason
-        del self.requests[r.id]
-        self.counters[{"cancelled": "cancelled", "error": "failed"}.get(reason, "finished")] += 1
-        end = {"type": "done", "finish_reason": reason, "error": error,
-               "usage": {"prompt_tokens": len(r.prompt), "completion_tokens": len(r.output),
-                         "total_tokens": len(r.prompt) + len(r.output)},
-               "cached_tokens": r.cached, "elapsed_s": time.perf_counter() - r.created}
-        if r.events.full():          # a terminal event always fits
-            while not r.events.empty():
-                r.events.get_nowait()
-        r.events.put_nowait(end)
-        self.trace.emit("finish", request_id=r.id, **{k: v for k, v in end.items() if k != "type"})
+        tally = "finished" if reason in ENDED_NORMALLY else "cancelled" if reason == "cancelled" else "failed"
+        self.counters[tally] += 1
+        verdict = {"finish_reason": reason, "error": error, "usage": r.usage(), "cached_tokens": r.cached,
+                   "elapsed_s": time.perf_counter() - r.created}
+        while True:
+            try:
+                r.events.put_nowait({"type": "done", **verdict})
+                break
+            except queue.Full:
+                with contextlib.suppress(queue.Empty):
+                    r.events.get_nowait()
+        self.trace.emit("finish", request_id=r.id, **verdict)
 
     def cancel(self, request_id):
+        """End a waiting or running request now; unknown and ended ids are ignored."""
         with self.lock:
             r = self.requests.get(request_id)
-            if r:
-                self._finish(r, "cancelled")
+            if r is not None:
+                self._retire(r, "cancelled")
 
     # ---- worker thread -------------------------------------------------------------------
     def start(self):
+        """Run turns on a worker thread until `close`; the thread sleeps while there is nothing to do."""
         if self.running:
             return
         self.running = True
-        self.thread = threading.Thread(target=self._loop, name="tessweave-model-worker", daemon=True)
+        self.thread = threading.Thread(target=self._work, name="tessweave-model-worker", daemon=True)
         self.thread.start()
 
-    def _loop(self):
-        while self.running:
-            try:
+    def _work(self):
+        try:
+            while self.running:
                 if not self.step():
-                    self.wake.wait(.05)
+                    self.wake.wait(0.05)
                     self.wake.clear()
-            except Exception as exc:      # any failure of a step ends the engine, never a request silently
-                self._fail(exc)
-                self.running = False
+        except Exception as exc:          # a failing step ends the engine and tells every request; none is lost silently
+            self._fail(exc)
+        finally:
+            self.running = False
 
     def _fail(self, exc):
         with self.lock:
             self.fatal = f"{type(exc).__name__}: {exc}"
             self.trace.emit("fatal", error=self.fatal)
             for r in list(self.requests.values()):
-                self._finish(r, "error", self.fatal)
+                self._retire(r, "error", self.fatal)
 
     def close(self):
+        """Stop the worker (waiting for the step it is in: storage is never freed under running kernels),
+        cancel what is left, empty the prefix index and drop the captured graphs."""
         self.running = False
         self.wake.set()
-        if self.thread:
-            self.thread.join()           # storage is never freed while kernels are in flight
-            self.thread = None
+        thread, self.thread = self.thread, None
+        if thread is not None:
+            thread.join()
         with self.lock:
             for r in list(self.requests.values()):
-                self._finish(r, "cancelled")
+                self._retire(r, "cancelled")
             self.cache.clear_prefixes()
             if hasattr(self.stepper, "close"):
                 self.stepper.close()
@@ -394,16 +454,23 @@ class Engine:
         raise RuntimeError("engine did not finish")
 
     def generate(self, prompts, max_tokens=128, temperature=0.0, seed=0, ignore_eos=False):
-        """Token ids generated for each prompt (a list of id lists); runs on the calling thread."""
-        requests, pending = [], list(prompts)
-        while pending or self.requests:
-            while pending and len(self.waiting) < self.config.max_queue:
-                requests.append(self.submit(pending.pop(0), max_tokens, temperature, seed, ignore_eos=ignore_eos))
+        """Token ids generated for each prompt (a list of id lists); runs on the calling thread.
+
+        Prompt i samples with seed SEED + i, so equal prompts do not draw equal streams. The requests
+        have no token events, so any `max_tokens` is fine.
+        """
+        prompts = list(prompts)
+        requests = []
+        while len(requests) < len(prompts) or self.requests:
+            while len(requests) < len(prompts) and len(self.waiting) < self.config.max_queue:
+                i = len(requests)
+                requests.append(self.submit(prompts[i], max_tokens, temperature, seed + i, ignore_eos=ignore_eos,
+                                            stream=False))
             if not self.step() and self.waiting:
                 raise RuntimeError("a waiting request can never be admitted")
-        failed = [r for r in requests if r.status == "error"]
-        if failed:
-            raise RuntimeError("generation failed")
+        for r in requests:
+            if r.status == "error":
+                raise RuntimeError(f"generation failed: {r.events.get_nowait().get('error')}")
         return [r.output for r in requests]
 
     def stats(self):

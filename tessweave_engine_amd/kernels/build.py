@@ -64,15 +64,41 @@ def library_name():
     return f"libtessweave_hip_{source_hash()}.so"
 
 
-def _candidate_dirs():
-    yield CSRC / "_lib"
+def _in_tree_dir():
+    return CSRC / "_lib"
+
+
+def _user_dir():
     user = os.getuid() if hasattr(os, "getuid") else 0
-    yield Path(tempfile.gettempdir()) / f"tessweave_engine_amd_{user}"
+    return Path(tempfile.gettempdir()) / f"tessweave_engine_amd_{user}"
+
+
+def _candidate_dirs():
+    yield _in_tree_dir()
+    yield _user_dir()
+
+
+def _only_ours(folder):
+    """Is FOLDER (under the shared temporary directory) a real directory that belongs to this user and
+    that nobody else can write to? A library is neither loaded from nor built into anything else: the
+    library's name is computable from public sources, so a folder another user made could hold a planted one."""
+    try:
+        st = os.lstat(folder)
+    except OSError:
+        return False
+    import stat
+    if not stat.S_ISDIR(st.st_mode):
+        return False
+    if hasattr(os, "getuid") and st.st_uid != os.getuid():
+        return False
+    return not st.st_mode & (stat.S_IWGRP | stat.S_IWOTH)
 
 
 def find_library():
     name = library_name()
     for folder in _candidate_dirs():
+        if folder == _user_dir() and not _only_ours(folder):
+            continue
         path = folder / name
         if path.exists():
             return path
@@ -82,7 +108,12 @@ def find_library():
 def _writable_dir():
     for folder in _candidate_dirs():
         try:
-            folder.mkdir(parents=True, exist_ok=True)
+            if folder == _user_dir():
+                folder.mkdir(mode=0o700, exist_ok=True)
+                if not _only_ours(folder):
+                    raise OSError(f"{folder} is not this user's private folder")
+            else:
+                folder.mkdir(parents=True, exist_ok=True)
             probe = folder / f".probe_{os.getpid()}"
             probe.write_bytes(b"")
             probe.unlink()

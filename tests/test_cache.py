@@ -12,15 +12,17 @@ def full_layout(layers=2):
 
 
 def test_pool_reference_vectors():
-    # flow_engine tests/test_engine.py:149-158: eviction keeps a page a request still holds
+    # flow_engine tests/test_engine.py:149-158: eviction never gives away a page a request still holds.
+    # (The reference drops the index entry on the failed attempt, refs == 1; here an attempt that cannot
+    # succeed leaves the index alone, so the page keeps both uses.)
     p = PagePool(2, 4)
     table = p.allocate(1)
     p.publish([1, 2, 3, 4], 4, table)
     with pytest.raises(CapacityError):
         p.allocate(2)
-    assert p.refs[table[0]] == 1
+    assert p.refs[table[0]] == 2 and len(p.prefixes) == 1 and p.evictions == 0
     p.release(table)
-    assert len(p.allocate(2)) == 2
+    assert len(p.allocate(2)) == 2 and not p.prefixes and p.evictions == 1
     # underflow and negative counts
     q = PagePool(2, 4)
     t = q.allocate(1)
@@ -46,6 +48,27 @@ def test_prefix_keys_full_blocks_namespaces_and_last_token():
     t2 = off.allocate(3)
     off.publish(tokens, 9, t2)
     assert off.acquire_prefix(tokens) == [] and not off.prefixes
+
+
+def test_eviction_takes_unused_entries_oldest_first_and_a_chain_from_its_tail():
+    p = PagePool(6, 2)
+    a = p.allocate(3)
+    p.publish([1, 2, 3, 4, 5, 6], 6, a)                 # one chain of three blocks
+    b = p.allocate(1)
+    p.publish([9, 9], 2, b)                             # a younger, unrelated entry
+    p.release(a + b)
+    assert len(p.free) == 2 and p.available() == 6
+    held = p.acquire_prefix([1, 2, 7])                  # touches the chain's root and pins its page
+    assert held == a[:1]
+    got = p.allocate(4)                                 # needs two evictions: the chain's tail goes first
+    assert p.evictions == 2 and set(got) >= {a[2], a[1]}
+    assert p.acquire_prefix([1, 2, 3]) == a[:1] and p.acquire_prefix([9, 9, 0]) == b
+    # a request that cannot be satisfied even by evicting everything leaves the index as it is
+    before = list(p.prefixes)
+    with pytest.raises(CapacityError):
+        p.allocate(3)
+    assert list(p.prefixes) == before
+    p.check([got, held, a[:1], b])
 
 
 def test_promises_set_pages_aside():
@@ -202,3 +225,16 @@ def test_ensure_is_all_or_nothing_across_groups():
     with pytest.raises(ValueError):
         m.ensure(s, 33)
     assert m.slot_of(s, 0, 5) == s.tables[0][1] * 4 + 1
+
+
+def test_slot_arithmetic_vector_of_the_reference():
+    """docs/ARCHITECTURE.md:51-53 of the reference: position 37, pages of 16, table[2] = 7 -> slot 117."""
+    m = CacheManager(full_layout(), 16, 9, 2, max_request_tokens=48)
+    seq = m.open("r")
+    m.pools[0].free = [0, 8, 6, 5, 4, 3, 7, 2, 1]            # pages come off the end: 1, 2, then 7
+    m.ensure(seq, 38)
+    assert seq.tables[0] == [1, 2, 7]
+    assert m.slot_of(seq, 0, 37) == 117 and m.slot_of(seq, 0, 0) == 16 and m.slot_of(seq, 0, 31) == 47
+    assert m.table_rows[0][seq.state_slot].tolist() == [1, 2, 7]
+    m.close(seq)
+    m.check()

@@ -48,6 +48,14 @@ def test_doctor_inspect_random_weights_and_replay(tmp_path, capsys):
     assert [e["event"] for e in shown] == ["admit", "step", "first_token", "finish", "fatal"]
 
 
+def test_prompts_are_taken_out_of_a_command_line():
+    argv = ["flow-inference", "generate", "m", "--prompt", "tell me", "--max-tokens", "3", "--prompt-ids=1,2,3",
+            "--prompt-ids", "4,5", "--prompt=x y", "--prompt-file", "ids.txt", "--prompt"]
+    assert cli.without_prompts(argv) == ["flow-inference", "generate", "m", "--prompt", "[REDACTED]", "--max-tokens", "3",
+                                         "--prompt-ids=[REDACTED]", "--prompt-ids", "[REDACTED]", "--prompt=[REDACTED]",
+                                         "--prompt-file", "ids.txt", "--prompt"]
+
+
 @pytest.mark.gpu
 def test_generate_prints_the_tokens_and_logs_the_run(tmp_path, capsys, device):
     make_folder(tmp_path / "model", "A")
@@ -67,8 +75,10 @@ def test_generate_prints_the_tokens_and_logs_the_run(tmp_path, capsys, device):
         assert usage["type"] == "done" and usage["error"] is None
     kinds = [json.loads(line)["event"] for line in log.read_text().splitlines()]
     assert kinds[:2] == ["launch", "loaded"] and {"admit", "step", "first_token", "finish"} <= set(kinds)
-    text = log.read_text()
-    assert "[REDACTED]" in text or "--prompt-ids" not in text       # prompts never reach the log
+    launches = [json.loads(line) for line in log.read_text().splitlines() if json.loads(line)["event"] == "launch"]
+    shown = launches[0]["argv"]                                      # the command line given to main(), prompt removed
+    assert shown[shown.index("--prompt-ids") + 1] == "[REDACTED]" and shown[:3] == ["flow-inference", "generate", str(tmp_path / "model")]
+    assert ",".join(str(t) for t in prompt) not in log.read_text()
     shown = [json.loads(line)["event"] for line in run(capsys, "replay", str(log)).splitlines()]
     assert shown and set(shown) <= {"step", "admit", "finish", "first_token", "fatal"}
     with pytest.raises(SystemExit):

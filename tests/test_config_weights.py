@@ -193,3 +193,18 @@ def test_tied_head_sharded_index_and_unsafe_names(tmp_path):
     with pytest.raises(WeightError) as info:
         read_tensors(folder, specs_b, torch.float32, "cpu")
     assert info.value.missing == ["lm_head.weight"]
+
+
+def test_cache_bytes_per_token_vector_of_the_reference():
+    """Qwen2.5-0.5B (24 layers, 2 key/value heads of 64): 24 KiB a token in 32-bit, 12 KiB in 16-bit
+    (the reference's docs/ARCHITECTURE.md:64 and flow_engine/config.py:64-65), from the
+    configuration class and from the cache layout of the model built for it."""
+    from tessweave_engine_amd.config import build_model, config_from_dict
+    cfg = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=24, hidden_size=896,
+               num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864, vocab_size=151936,
+               max_position_embeddings=32768)
+    config = config_from_dict(cfg)
+    assert config.head_dim == 64
+    assert config.kv_bytes_per_token(4) == 24 * 1024 and config.kv_bytes_per_token(2) == 12 * 1024
+    layout = build_model(config).cache_layout()
+    assert layout.bytes_per_token(4) == 24 * 1024 and layout.bytes_per_token(2) == 12 * 1024

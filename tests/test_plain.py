@@ -81,14 +81,6 @@ def test_attention_reduces_to_library_routines():
     torch.testing.assert_close(win[8:], plain.attention(q[8:], k[6:], v[6:], pos[8:], pos[6:]))
 
 
-def test_reference_kernel_vector_tables():
-    """Slot arithmetic vector of the reference's docs: position 37, page 16, table[2] = 7 -> slot 117."""
-    table, page, position = {2: 7}, 16, 37
-    assert table[position // page] * page + position % page == 117
-    # KV bytes per token, Qwen2.5-0.5B (24 layers, 2 kv heads, head 64): 24 KiB in fp32, 12 KiB in 16-bit
-    assert 2 * 24 * 2 * 64 * 4 == 24 * 1024 and 2 * 24 * 2 * 64 * 2 == 12 * 1024
-
-
 def test_swiglu_equals_library_and_order_of_halves():
     x = torch.randn(3, 10, dtype=torch.float64)
     g, u, dn = torch.randn(14, 10, dtype=torch.float64), torch.randn(14, 10, dtype=torch.float64), torch.randn(10, 14, dtype=torch.float64)

@@ -246,7 +246,11 @@ def test_cancel_queue_limit_and_slow_consumer():
     e.cancel(b.id)
     e.cancel(a.id)
     assert not e.step() and (a.status, b.status) == ("cancelled", "cancelled")
-    assert len(e.cache.pools[0].free) == e.cache.pools[0].capacity
+    pool = e.cache.pools[0]
+    # a's first full prompt block was computed and entered into the prefix index before the cancel: it stays
+    # there, evictable; everything else is free
+    assert len(pool.prefixes) == 1 and len(pool.free) == pool.capacity - 1 and pool.available() == pool.capacity
+    e.cache.check()
     e.close()
     e, s = make(max_queue=1)
     r = e.submit([1, 2], 4)
@@ -544,3 +548,73 @@ def test_adaptive_portions_follow_the_measured_time_within_their_bounds():
     drain(fixed)
     assert fixed.chunk == 8 and all(n <= 8 for batch in s2.batches for (_, _, n, _) in batch)
     fixed.close()
+
+
+def test_generate_takes_more_tokens_than_an_event_queue_holds_and_seeds_each_prompt():
+    cfg = dict(CFG, max_position_embeddings=1024)
+    config = EngineConfig(block_size=4, kv_blocks=200, max_context=400, prefill_chunk=4, min_prefill_chunk=1,
+                          dtype="float32")
+    model = build_model(config_from_dict(cfg))
+    cache = CacheManager(model.cache_layout(), 4, 200, config.max_active, max_request_tokens=400)
+    stepper = FakeStepper(cache)
+    stepper.full = {}
+    e = Engine(model, config, stepper=stepper, cache=cache, sampler=FakeSampler())
+    submit, made = e.submit, []
+
+    def tracked(tokens, *a, **k):
+        r = submit(tokens, *a, **k)
+        stepper.full[r.id] = r.tokens
+        made.append(r)
+        return r
+    e.submit = tracked
+    outs = e.generate([[3, 1, 4], [3, 1, 4]], max_tokens=300, temperature=0.5, seed=40)
+    assert [len(o) for o in outs] == [300, 300] and outs[0] == expected([3, 1, 4], 300)
+    assert [r.seed for r in made] == [40, 41] and all(r.status == "length" for r in made)
+    assert all(r.events.qsize() == 1 for r in made)                   # only the terminal event
+    # a streaming consumer that never reads still loses its request after 256 tokens, as before
+    r = tracked([3, 1, 4], 300)
+    drain(e)
+    assert r.status == "error" and len(r.output) == 257
+    e.close()
+
+
+def test_prompt_blocks_are_shared_while_their_first_owner_still_runs():
+    e, s = make(max_active=2, prefill_chunk=8, max_step_tokens=8)
+    prompt = [2, 3, 4, 5, 6, 7, 8, 9, 10]
+    a = e.submit(prompt, 6)
+    e.step()                                            # a's first 8 prompt tokens: two full blocks
+    assert a.status == "active" and a.published == 8 and len(e.cache.pools[0].prefixes) == 2
+    b = e.submit(prompt, 6)
+    e.step()
+    assert b.status == "active" and b.cached == 8 and a.status == "active"
+    assert e.cache.stats()["prefix_hit_tokens"] == 8
+    drain(e)
+    assert a.output == b.output == expected(prompt, 6)
+    # b never ran the shared tokens
+    assert [(start, n) for batch in s.batches for (rid, start, n, _) in batch if rid == b.id][0] == (8, 1)
+    e.close()
+    e.cache.check()
+    assert len(e.cache.pools[0].free) == 32
+
+
+def test_a_head_of_queue_that_does_not_fit_earns_no_hits_and_costs_no_index_entries():
+    e, s = make(kv_blocks=6, max_active=2)
+    first = e.submit([1, 2, 3, 4, 5, 6, 7, 8, 9], 3)      # 3 pages
+    drain(e)
+    assert len(e.cache.pools[0].prefixes) == 2
+    long_ = e.submit([7] * 9, 11)                         # 5 pages, admitted; evicts nothing yet needed
+    e.step()
+    entries = len(e.cache.pools[0].prefixes)
+    again = e.submit([1, 2, 3, 4, 5, 6, 7, 8, 9], 3)      # shares 2 pages if they survived, needs 1 more: must wait
+    waited = 0
+    for _ in range(3):
+        e.step()
+        if again.status == "waiting":
+            waited += 1
+            assert e.cache.stats()["prefix_hit_tokens"] == 0
+            assert len(e.cache.pools[0].prefixes) >= entries
+    assert waited == 3
+    drain(e)
+    assert again.output == first.output and long_.status == "length"
+    e.close()
+    e.cache.check()
