@@ -22,17 +22,25 @@ class GroupedQueryAttention(Mixer):
                  o_bias=False, window=None, scale=None, packed=True):
         if q_heads % kv_heads:
             raise ValueError("q_heads must be a multiple of kv_heads")
-        if head_dim % 16 or not 16 <= head_dim <= 256:
-            raise ValueError("the attention kernels take head sizes in steps of 16 from 16 to 256; "
-                             f"head_dim {head_dim} is refused")
+        if head_dim % 2 or not 2 <= head_dim <= 256:
+            raise ValueError(f"the attention kernels take even head sizes up to 256; head_dim {head_dim} is refused")
         self.prefix = prefix
-        self.hidden, self.q_heads, self.kv_heads, self.head_dim = int(hidden), int(q_heads), int(kv_heads), int(head_dim)
+        self.hidden, self.q_heads, self.kv_heads = int(hidden), int(q_heads), int(kv_heads)
+        # The kernels work on heads of a multiple of 16 elements. A head of another size is laid out with a
+        # tail of zeros on the device: zero rows in the q/k/v matrices and biases, zero columns in the output
+        # matrix. Zero elements add nothing to a score, zero values give zero outputs, which meet zero columns:
+        # the result is exactly that of the unpadded head. `head_dim` is the size on the device from here on;
+        # the scale and the rotation keep the checkpoint's size.
+        self.checkpoint_head_dim = int(head_dim)
+        self.head_dim = (int(head_dim) + 15) // 16 * 16
+        pad = (self.checkpoint_head_dim, self.head_dim)
         self.position = position
         self.window = window
-        self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
+        self.scale = float(scale) if scale is not None else self.checkpoint_head_dim ** -0.5
         self.qkv = Linear([prefix + "q_proj", prefix + "k_proj", prefix + "v_proj"], hidden,
-                          [q_heads * head_dim, kv_heads * head_dim, kv_heads * head_dim], bias=qkv_bias, packed=packed)
-        self.o = Linear([prefix + "o_proj"], q_heads * head_dim, [hidden], bias=o_bias)
+                          [q_heads * head_dim, kv_heads * head_dim, kv_heads * head_dim], bias=qkv_bias, packed=packed,
+                          pad_out=pad)
+        self.o = Linear([prefix + "o_proj"], q_heads * head_dim, [hidden], bias=o_bias, pad_in=pad)
 
     def parts(self):
         return [self.qkv, self.o, self.position]

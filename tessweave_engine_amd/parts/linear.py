@@ -14,12 +14,29 @@ from ..weights.spec import MATRIX, VECTOR, NORMAL, TensorSpec
 from .base import Part
 
 
+def pad_groups(t, dim, unit, to):
+    """T with every group of UNIT consecutive entries along DIM followed by TO - UNIT zeros."""
+    if to == unit:
+        return t
+    shape = list(t.shape)
+    groups = shape[dim] // unit
+    out = t.new_zeros(shape[:dim] + [groups, to] + shape[dim + 1:])
+    out.narrow(dim + 1, 0, unit).copy_(t.reshape(shape[:dim] + [groups, unit] + shape[dim + 1:]))
+    return out.reshape(shape[:dim] + [groups * to] + shape[dim + 1:])
+
+
 class Linear(Part):
-    def __init__(self, names, in_features, out_features, bias=False, packed=True, glu=False):
+    def __init__(self, names, in_features, out_features, bias=False, packed=True, glu=False,
+                 pad_out=None, pad_in=None):
         """names[i] is the checkpoint prefix of the i-th matrix ("...q_proj"), out_features[i] its rows.
 
         glu: the two matrices are a gate and an up projection; if they can be packed with their
         rows interleaved (`gated` is then true after bind), `forward_glu` gives silu(gate) * up.
+        pad_out = (unit, to): on the device every group of `unit` output rows (a head) is followed by
+        `to - unit` rows of zeros (and zero biases), so the layer's output has groups of `to` columns
+        whose tail is exactly zero. pad_in = (unit, to): the same for groups of input columns (the
+        input then has groups of `to` columns, whose tails meet zeros). The checkpoint's tensors keep
+        their own shapes.
         """
         self.names = list(names)
         self.in_features = int(in_features)
@@ -27,6 +44,11 @@ class Linear(Part):
         self.has_bias = bool(bias)
         self.packed = bool(packed)
         self.glu = bool(glu)
+        self.pad_out = tuple(int(v) for v in pad_out) if pad_out and pad_out[0] != pad_out[1] else None
+        self.pad_in = tuple(int(v) for v in pad_in) if pad_in and pad_in[0] != pad_in[1] else None
+        for pad, sizes in ((self.pad_out, self.out_features), (self.pad_in, [self.in_features])):
+            if pad and (pad[1] < pad[0] or any(n % pad[0] for n in sizes)):
+                raise ValueError("padded groups must divide the layer's sizes and may only grow")
         self.gated = False
         self.weights = []       # one tensor if packed, else one per name
         self.biases = []
@@ -47,8 +69,13 @@ class Linear(Part):
     def bind(self, tensors, dtype, device):
         weights = [tensors.pop(name + ".weight") for name in self.names]
         biases = [tensors.pop(name + ".bias") for name in self.names] if self.has_bias else []
+        if self.pad_out:
+            weights = [pad_groups(w, 0, *self.pad_out) for w in weights]
+            biases = [pad_groups(b, 0, *self.pad_out) for b in biases]
+        if self.pad_in:
+            weights = [pad_groups(w, 1, *self.pad_in) for w in weights]
         self.gated = (self.glu and self.packed and len(weights) == 2 and
-                      self.out_features[0] == self.out_features[1] and self.out_features[0] % 16 == 0)
+                      weights[0].shape == weights[1].shape and weights[0].shape[0] % 16 == 0)
         if self.gated:
             weights = [ops.interleave_glu_rows(*weights)]
             biases = [ops.interleave_glu_rows(*biases)] if biases else []

@@ -1,0 +1,243 @@
+"""The sizes the benchmark times, against the plain implementation.
+
+The other GPU tests stop at a few hundred keys and four requests. What `bench.py` measures runs elsewhere
+in the same kernels: decode attention over thousands of keys cut into as many ranges as the launcher itself
+chooses (most of them empty for a short request in a batch sized for long ones), decode batches of 33-64
+rows (the widest instantiation of the streaming matrix kernel), graphs captured for an engine that is
+opened for thousands of tokens, and a 2,048-token prompt portion through the largest matrix tiles and the
+128-row attention tiles in one step. Each is compared here with the plain implementation, in both precisions.
+"""
+import math
+
+import pytest
+import torch
+
+import plain_model as plain
+from test_kernels_gpu import ATTN_TOL, build_paged
+from tiny_configs import make_folder
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops(device):
+    from tessweave_engine_amd.kernels import ops as o
+    return o
+
+
+def decode_case(ops, device, dtype, heads, kv_heads, d, page, lengths, k, v, q, splits_list, window=0):
+    n_seqs = len(lengths)
+    pages_total = sum(math.ceil(n / page) for n in lengths) + 3
+    keys, values, table = build_paged(k, v, lengths, page, pages_total, device, dtype, seed=len(lengths))
+    want = torch.stack([plain.attention(q[i:i + 1].float(), k[i], v[i], torch.tensor([lengths[i] - 1]),
+                                        window=window or None)[0] for i in range(n_seqs)])
+    qd = q.reshape(n_seqs, heads * d).to(dtype).to(device)
+    q_start = torch.arange(n_seqs + 1, dtype=torch.int32, device=device)
+    kv_len = torch.tensor(lengths, dtype=torch.int32, device=device)
+    for splits, generic in splits_list:
+        out = torch.full((n_seqs, heads * d), float("nan"), dtype=dtype, device=device)
+        ws = torch.full((max(1, ops.attn_decode_workspace_floats(n_seqs, heads, d, splits)),), float("nan"), device=device)
+        ops.attn_decode(qd, keys, values, table, q_start, kv_len, 0, n_seqs, out, heads, kv_heads, d, d ** -0.5,
+                        window=window, splits=splits, workspace=ws, generic=generic)
+        torch.testing.assert_close(out.float().cpu().reshape(n_seqs, heads, d), want, **ATTN_TOL[dtype],
+                                   msg=lambda m: f"splits {splits} generic {generic}: {m}")
+    return want
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("head_dim", [64, 128, 256])
+def test_decode_attention_with_many_key_ranges_most_of_them_empty(ops, device, dtype, head_dim):
+    """16, 33 and 64 key ranges over requests of 5, 3,000, 1 and 700 keys: a short request leaves most ranges
+    empty (their partial results must count for nothing), and the merge kernel runs past the ranges one pass
+    of its loop takes."""
+    heads, kv_heads, page = 8, 2, 16
+    lengths = [5, 3000, 1, 700]
+    g = torch.Generator().manual_seed(head_dim)
+    k = [torch.randn(n, kv_heads, head_dim, generator=g).to(dtype).float() for n in lengths]
+    v = [torch.randn(n, kv_heads, head_dim, generator=g).to(dtype).float() for n in lengths]
+    q = torch.randn(len(lengths), heads, head_dim, generator=g).to(dtype)
+    decode_case(ops, device, dtype, heads, kv_heads, head_dim, page, lengths, k, v, q,
+                [(16, False), (33, False), (64, False), (16, True), (33, True), (64, True)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("longest,batch", [(4096, 1), (4096, 8), (32000, 1), (32000, 3)])
+def test_decode_attention_at_the_benchmarks_lengths_with_the_launchers_own_ranges(ops, device, dtype, longest, batch):
+    """28 query heads over 4 key/value heads of 128 (the 7B layer), 4,096 and 32,000 keys, the number of
+    key ranges that the launcher picks for this batch. Every head's query points at ONE key on an edge (first,
+    last, page and block edges, the edges of the chosen ranges), so a dropped or doubled key is off by O(1)
+    in bfloat16 too; the other requests of the batch are short and leave most ranges empty."""
+    heads, kv_heads, d, page = 28, 4, 128, 16
+    splits = ops.attn_decode_splits(batch, heads, kv_heads, longest)
+    assert splits > 1
+    span = math.ceil(longest / splits)
+    targets = [0, 1, 15, 16, 31, 32, 33, 63, 64, 255, 256, span - 1, span, span + 1, 2 * span - 1, 2 * span,
+               longest // 2, longest - span - 1, longest - span, longest - 257, longest - 65, longest - 64, longest - 33,
+               longest - 32, longest - 17, longest - 16, longest - 2, longest - 1]
+    assert len(targets) == heads and all(0 <= t < longest for t in targets)
+    lengths = [longest] + [37, 1500, 9, 2048, 1, 640, 100][:batch - 1]
+    g = torch.Generator().manual_seed(longest + batch)
+    unit = torch.nn.functional.normalize(torch.randn(heads, d, generator=g), dim=1)
+    k = [torch.randn(n, kv_heads, d, generator=g) * 0.1 for n in lengths]
+    v = [torch.randn(n, kv_heads, d, generator=g) for n in lengths]
+    group = heads // kv_heads
+    owner = {}
+    for h, p in enumerate(targets):
+        k[0][p, h // group] = unit[h] * 30.0           # several heads of a group have their own far key
+        owner[p, h // group] = h                       # (two heads of a group may name the same key: the later one has it)
+    k = [t.to(dtype).float() for t in k]
+    v = [t.to(dtype).float() for t in v]
+    q = torch.randn(len(lengths), heads, d, generator=g)
+    q[0] = unit * 12.0
+    q = q.to(dtype)
+    want = decode_case(ops, device, dtype, heads, kv_heads, d, page, lengths, k, v, q,
+                       [(splits, False), (splits, True), (1, False)])
+    # the vectors do what they are for: each head of the long request returns (nearly) its target's value
+    hits = 0
+    for h, p in enumerate(targets):
+        if owner[p, h // group] == h:
+            hits += 1
+            assert (want[0, h] - v[0][p, h // group]).abs().max() < 0.05, (h, p)
+    assert hits >= 20
+
+
+# ---- the engine opened for thousands of tokens, a decode batch of 48 from graphs ----------------------------
+@pytest.fixture(scope="module")
+def long_model(tmp_path_factory, device):
+    folder = tmp_path_factory.mktemp("longA")
+    cfg, page = make_folder(folder, "A")
+    cfg = dict(cfg, max_position_embeddings=8192)
+    import json
+    (folder / "config.json").write_text(json.dumps(cfg))
+    config, weights = plain.read_folder(folder)
+    return dict(folder=folder, page=page, cfg=cfg, config=config, weights=weights)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_decode_batch_of_48_requests_short_and_long_from_graphs(long_model, dtype):
+    """An engine opened for 4,224 tokens a request: the captured decode step sizes its key ranges by that, and
+    the batch holds requests of 3 to 4,100 tokens. Six decode steps (one eager, one captured, four replayed) of
+    48 requests, every logits row against the plain implementation."""
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.weights import load_model
+    page, vocab = long_model["page"], long_model["cfg"]["vocab_size"]
+    n_req, n_decode, capacity = 48, 6, 4224
+    g = torch.Generator().manual_seed(48)
+    prompt_lens = [4100, 1500, 3, 700] + torch.randint(1, 200, (n_req - 4,), generator=g).tolist()
+    tokens = [torch.randint(0, vocab, (n + n_decode,), generator=g).tolist() for n in prompt_lens]
+    want = [plain.forward(long_model["config"], long_model["weights"], t) for t in tokens]
+    model = load_model(long_model["folder"], dtype=dtype, device="cuda:0")
+    pages = sum(math.ceil((n + n_decode) / page) for n in prompt_lens)
+    cache = CacheManager(model.cache_layout(), page, pages, n_req, dtype=dtype, device=model.device,
+                         prefix_cache=False, max_request_tokens=capacity)
+    stepper = Stepper(model, cache, max_step_tokens=512, max_step_seqs=n_req)
+    seqs = [cache.open(f"r{i}") for i in range(n_req)]
+    worst = 0.0
+
+    def check(got, rows):
+        nonlocal worst
+        for r, (i, pos) in enumerate(rows):
+            w = want[i][pos]
+            err = float((got[r] - w).abs().max())
+            worst = max(worst, err)
+            if dtype == "float32":
+                assert torch.allclose(got[r], w, atol=5e-6, rtol=2e-5), (i, pos, err)
+            else:
+                assert err <= 0.02 * float(w.abs().max()), (i, pos, err)
+    # prompts: the long ones in portions of 512, the short ones several to a step
+    for i in (0, 1, 3):
+        for a in range(0, prompt_lens[i], 512):
+            b = min(prompt_lens[i], a + 512)
+            got = stepper.step([StepEntry(seqs[i], tokens[i][a:b], [b - a - 1])]).cpu()
+            check(got, [(i, b - 1)])
+    rest = [i for i in range(n_req) if i not in (0, 1, 3)]
+    for a in range(0, len(rest), 8):
+        batch = rest[a:a + 8]
+        got = stepper.step([StepEntry(seqs[i], tokens[i][:prompt_lens[i]], [prompt_lens[i] - 1]) for i in batch]).cpu()
+        check(got, [(i, prompt_lens[i] - 1) for i in batch])
+    # decode: all 48 in every step
+    for s in range(n_decode):
+        got = stepper.step([StepEntry(seqs[i], [tokens[i][prompt_lens[i] + s]], [0]) for i in range(n_req)]).cpu()
+        check(got, [(i, prompt_lens[i] + s) for i in range(n_req)])
+    assert stepper.graph_replays >= n_decode - 2
+    print(f"48 requests, {dtype}: worst difference {worst:.3e}")
+    for seq in seqs:
+        cache.close(seq)
+    cache.check()
+    stepper.close()
+
+
+# ---- one layer at the 7B width: a 2,048-token portion in one step, then decoding past 4,096 keys ------------
+WIDE = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2",
+    num_hidden_layers=1, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
+    intermediate_size=18944, vocab_size=1031, rope_theta=1e6, rms_norm_eps=1e-6,
+    tie_word_embeddings=False, use_sliding_window=False, max_position_embeddings=8192, hidden_act="silu")
+
+
+def plain_on_device(config, weights, tokens, dtype, device, rows):
+    """The plain implementation's logits at ROWS, its tensors moved to the GPU (torch's float64 there) so that
+    4,104 tokens through a 7B-width layer take seconds. Only the last layer's rows are cut; nothing else changes."""
+    w = {k: t.to(device=device, dtype=dtype) for k, t in weights.items()}
+    logits = _forward_on(config, w, tokens, device)
+    return logits[rows].cpu()
+
+
+def _forward_on(config, w, tokens, device):
+    # plain.forward builds its index tensors on the CPU; run it under a default device instead
+    with torch.device(device):
+        return plain.forward(config, w, tokens)
+
+
+@pytest.fixture(scope="module")
+def wide_long(tmp_path_factory, device):
+    from tessweave_engine_amd.config import config_from_dict
+    from tessweave_engine_amd.weights import write_model_folder
+    folder = tmp_path_factory.mktemp("wide_long")
+    write_model_folder(folder, config_from_dict(WIDE), 11)
+    g = torch.Generator().manual_seed(2048)
+    n = 4096 + 8
+    tokens = torch.randint(0, WIDE["vocab_size"], (n,), generator=g).tolist()
+    rows = [0, 1, 127, 128, 1000, 2047, 2048, 2049, 4094, 4095] + list(range(4096, n))
+    config, weights = plain.read_folder(folder, torch.float32)
+    exact = plain_on_device(config, weights, tokens, torch.float64, device, rows)
+    single = plain_on_device(config, weights, tokens, torch.float32, device, rows)
+    return dict(folder=folder, tokens=tokens, rows=rows, exact=exact, single=single)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_2048_token_portion_in_one_step_then_decoding_past_4096_keys(wide_long, dtype):
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.weights import load_model
+    tokens, rows = wide_long["tokens"], wide_long["rows"]
+    model = load_model(wide_long["folder"], dtype=dtype, device="cuda:0")
+    page = 16
+    cache = CacheManager(model.cache_layout(), page, math.ceil(len(tokens) / page) + 1, 2, dtype=dtype,
+                         device=model.device, prefix_cache=False, max_request_tokens=len(tokens) + page)
+    stepper = Stepper(model, cache, max_step_tokens=2048, max_step_seqs=2)
+    seq = cache.open("r")
+    got = {}
+    for a in (0, 2048):                                         # two portions of 2,048 tokens, each ONE step
+        want_rows = [r - a for r in rows if a <= r < a + 2048]
+        out = stepper.step([StepEntry(seq, tokens[a:a + 2048], want_rows)]).cpu()
+        for j, r in enumerate(want_rows):
+            got[r + a] = out[j].clone()
+    for p in range(4096, len(tokens)):                          # then single tokens over 4,097+ keys
+        got[p] = stepper.step([StepEntry(seq, [tokens[p]], [0])]).cpu()[0].clone()
+    assert stepper.graph_replays >= len(tokens) - 4096 - 2
+    worst_engine = worst_plain = 0.0
+    for j, r in enumerate(rows):
+        exact = wide_long["exact"][j].float()
+        err = float((got[r] - exact).abs().max())
+        worst_engine = max(worst_engine, err)
+        worst_plain = max(worst_plain, float((wide_long["single"][j] - exact).abs().max()))
+        if dtype == "bfloat16":
+            assert err <= 0.02 * float(exact.abs().max()), (r, err)
+    print(f"2,048-token portions + decode past 4,096 keys, {dtype}: engine off by {worst_engine:.3e}, "
+          f"plain float32 off by {worst_plain:.3e}")
+    if dtype == "float32":
+        assert worst_engine <= 4 * worst_plain + 1e-6, (worst_engine, worst_plain)
+    cache.close(seq)
+    stepper.close()
