@@ -42,11 +42,13 @@ def random_tensors(specs, seed, std=DEFAULT_STD, store_dtype=torch.bfloat16, dev
             for s in specs if s.optional_alias_of is None}
 
 
-def write_model_folder(folder, config, seed, std=DEFAULT_STD, store_dtype="bfloat16"):
+def write_model_folder(folder, config, seed, std=DEFAULT_STD, store_dtype="bfloat16", device="cpu"):
     """Write config.json and model.safetensors for CONFIG; returns the folder path.
 
     Values are rounded to STORE_DTYPE before writing, so a float32 run and a
-    bfloat16 run of the same folder use the same weight values.
+    bfloat16 run of the same folder use the same weight values. DEVICE is where
+    the values are drawn: a GPU draws billions of values in a moment, but its
+    generator's stream is not the CPU's, so the same seed gives other values there.
     """
     from safetensors.torch import save_file
     from ..config import build_model
@@ -54,9 +56,9 @@ def write_model_folder(folder, config, seed, std=DEFAULT_STD, store_dtype="bfloa
     folder = Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
     model = build_model(config)
-    tensors = random_tensors(model.tensor_specs(), seed, std, resolve_dtype(store_dtype))
+    tensors = random_tensors(model.tensor_specs(), seed, std, resolve_dtype(store_dtype), device)
     (folder / "config.json").write_text(json.dumps(config.to_dict(), indent=2) + "\n")
-    save_file({k: v.contiguous() for k, v in tensors.items()}, str(folder / "model.safetensors"))
+    save_file({k: v.contiguous().cpu() for k, v in tensors.items()}, str(folder / "model.safetensors"))
     return folder
 
 

@@ -12,12 +12,12 @@ import torch
 from safetensors import safe_open
 
 
-def read_folder(folder, dtype=torch.float32):
-    """(config dict, {tensor name: tensor in DTYPE}) of a model folder."""
+def read_folder(folder, dtype=torch.float32, device="cpu"):
+    """(config dict, {tensor name: tensor in DTYPE on DEVICE}) of a model folder."""
     folder = Path(folder)
     config = json.loads((folder / "config.json").read_text())
     tensors = {}
-    with safe_open(str(folder / "model.safetensors"), framework="pt", device="cpu") as f:
+    with safe_open(str(folder / "model.safetensors"), framework="pt", device=str(device)) as f:
         for key in f.keys():
             tensors[key] = f.get_tensor(key).to(dtype)
     return config, tensors
