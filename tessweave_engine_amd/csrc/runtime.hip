@@ -3,6 +3,8 @@
 
 extern "C" const char* tw_error_string(int code) {
   if (code == TW_ERR_BAD_ARGUMENT) return "a kernel launcher refused its arguments (shape, alignment or size)";
+  if (code == TW_ERR_TOO_LARGE)
+    return "the input is larger than this entry point's built-in scratch memory holds (tw_sample_rows_static: at most 256 rows)";
   return hipGetErrorString((hipError_t)code);
 }
 

@@ -4,6 +4,9 @@
 // counter-based generator keyed by (the request's seed, the index of the token
 // being drawn), so a request's stream does not depend on what else is in the batch.
 #include "tw_common.h"
+#include "tw_sampling.h"
+
+#include <mutex>
 
 __host__ __device__ static inline uint64_t tw_splitmix64(uint64_t x) {
   x += 0x9E3779B97F4A7C15ull;
@@ -175,6 +178,16 @@ __global__ __launch_bounds__(TW_SAMPLE_THREADS) void sample_pick_kernel(
   }
 }
 
+static int sample_launch(const float* logits, long ld, int rows, int vocab, const float* temperature,
+                         const uint64_t* seeds, const int* counters, int* out, SamplePartial* partial,
+                         hipStream_t stream) {
+  sample_scan_kernel<<<dim3(TW_SAMPLE_CHUNKS, rows), TW_SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, temperature, partial);
+  int err = TW_LAUNCH_RESULT();
+  if (err) return err;
+  sample_pick_kernel<<<rows, TW_SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, temperature, seeds, counters, partial, out);
+  return TW_LAUNCH_RESULT();
+}
+
 extern "C" long tw_sample_workspace_bytes(int rows) { return (long)rows * TW_SAMPLE_CHUNKS * sizeof(SamplePartial); }
 
 // logits [rows][ld] float32; temperature (may be null: all greedy), seeds, counters per row;
@@ -186,10 +199,44 @@ extern "C" int tw_sample_rows(const float* logits, long ld, int rows, int vocab,
   TW_REQUIRE(temperature == nullptr || (seeds != nullptr && counters != nullptr));
   if (rows == 0) return 0;
   TW_REQUIRE(workspace != nullptr && workspace_bytes >= tw_sample_workspace_bytes(rows) && (uintptr_t)workspace % 16 == 0);
-  SamplePartial* partial = (SamplePartial*)workspace;
-  sample_scan_kernel<<<dim3(TW_SAMPLE_CHUNKS, rows), TW_SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, temperature, partial);
-  int err = TW_LAUNCH_RESULT();
+  return sample_launch(logits, ld, rows, vocab, temperature, seeds, counters, out, (SamplePartial*)workspace, stream);
+}
+
+// ---- the same without a workspace from the caller: partial results in the library's own device image ----
+// `scratch` is a name of HOST code here: the device address behind it differs per GPU and is looked up
+// once per device (below); kernels only ever get that looked-up pointer.
+static __device__ __align__(256) unsigned char scratch[TW_SAMPLE_STATIC_MAX_ROWS * TW_SAMPLE_CHUNKS * sizeof(SamplePartial)];
+
+#define TW_SAMPLE_MAX_DEVICES 64
+static void* g_scratch_of_device[TW_SAMPLE_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+// The address of `scratch` on the CURRENT device, looked up on the first call there.
+static int scratch_on_current_device(void** out) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return (int)e;
+  if (device < 0 || device >= TW_SAMPLE_MAX_DEVICES) return TW_ERR_BAD_ARGUMENT;
+  std::lock_guard<std::mutex> guard(g_scratch_mutex);
+  if (g_scratch_of_device[device] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (ptr == nullptr) return (int)hipErrorInvalidSymbol;
+    g_scratch_of_device[device] = ptr;
+  }
+  *out = g_scratch_of_device[device];
+  return 0;
+}
+
+extern "C" int tw_sample_rows_static(const float* logits, long ld, int rows, int vocab, const float* temperature,
+                                     const uint64_t* seeds, const int* counters, int* out, hipStream_t stream) {
+  TW_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab);
+  TW_REQUIRE(temperature == nullptr || (seeds != nullptr && counters != nullptr));
+  if (rows > TW_SAMPLE_STATIC_MAX_ROWS) return TW_ERR_TOO_LARGE;
+  if (rows == 0) return 0;
+  void* partial = nullptr;
+  const int err = scratch_on_current_device(&partial);
   if (err) return err;
-  sample_pick_kernel<<<rows, TW_SAMPLE_THREADS, 0, stream>>>(logits, ld, vocab, temperature, seeds, counters, partial, out);
-  return TW_LAUNCH_RESULT();
+  return sample_launch(logits, ld, rows, vocab, temperature, seeds, counters, out, (SamplePartial*)partial, stream);
 }

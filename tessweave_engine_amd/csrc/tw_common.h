@@ -12,6 +12,7 @@
 #define TW_DTYPE_BF16 1
 
 #define TW_ERR_BAD_ARGUMENT 10001   // a launcher refused its arguments (shape, alignment, size)
+#define TW_ERR_TOO_LARGE 10002      // an input exceeds the fixed capacity of an entry point that brings its own scratch memory
 
 typedef __bf16 bf16_t;
 typedef float f32x4 __attribute__((ext_vector_type(4)));

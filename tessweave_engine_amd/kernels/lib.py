@@ -36,6 +36,7 @@ _SIGNATURES = {
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),
     "tw_sample_rows": (I, [P, L, I, I, P, P, P, P, P, L, P]),
+    "tw_sample_rows_static": (I, [P, L, I, I, P, P, P, P, P]),
 }
 
 
