@@ -9,7 +9,12 @@ random prompt of 4096 - W - K tokens, then W untimed and K timed decode steps
 run through the scheduler (admission, planning, the step function, greedy
 sampling on the device, commit), so the last timed step reads 4,096 keys per
 request. One JSON line is printed: decoded tokens a second, a 2,048-token
-prefill, the decode step's HBM roofline, and decode at batch 1 and 64.
+prefill, the decode step's HBM roofline (against the nominal 8 TB/s and against
+what a plain streaming reader reaches on this device, measured in the same run),
+and further points: decode at batch 1 and 64 at the same context; the same batch
+of 8 with the engine opened for 32,768 tokens a request (`decode_b8_open32k`);
+and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
+(`gen512_b*`, decoded tokens a second over the generated part).
 
 Other sizes of the architecture: --shape 14b|32b. --serve measures continuous
 batching under Poisson arrivals instead (prompts of 128..4,096 tokens, 256
@@ -53,6 +58,10 @@ def parse():
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--points", default="1,64", help="further decode batch sizes to measure")
+    p.add_argument("--max-context", type=int, default=0,
+                   help="tokens a request may hold, which the engine is opened for (0: the context + 1)")
+    p.add_argument("--no-extra-points", action="store_true",
+                   help="skip decode_b8_open32k and the gen512_b* points (1,024-token prompts + 512 generated)")
     p.add_argument("--no-graphs", action="store_true")
     p.add_argument("--prefill-only", action="store_true", help="measure only the prefill (profiling runs)")
     p.add_argument("--seed", type=int, default=0)
@@ -64,7 +73,7 @@ def parse():
     return p.parse_args()
 
 
-def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, seed):
+def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, seed, max_context=0):
     """Tokens/s and ms/step of STEPS decode steps at BATCH, ending at CONTEXT keys per request."""
     from tessweave_engine_amd.config import EngineConfig
     from tessweave_engine_amd.engine import Engine
@@ -74,14 +83,14 @@ def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, s
     page = 16
     blocks = batch * ((context + page - 1) // page + 1)
     chunk = 2048
-    config = EngineConfig(block_size=page, kv_blocks=blocks, max_context=context + 1, max_active=batch,
+    config = EngineConfig(block_size=page, kv_blocks=blocks, max_context=max_context or context + 1, max_active=batch,
                           max_queue=batch, prefill_chunk=chunk, min_prefill_chunk=16, prefix_cache=False,
                           dtype=dtype, max_step_tokens=batch + chunk, use_graphs=use_graphs)
     engine = Engine(model, config)
     g = torch.Generator().manual_seed(seed)
     vocab = model.config.vocab_size
     requests = [engine.submit(torch.randint(0, vocab, (prompt_len,), generator=g).tolist(),
-                              max_tokens=steps + warmup + 1, ignore_eos=True) for _ in range(batch)]
+                              max_tokens=steps + warmup + 1, ignore_eos=True, stream=False) for _ in range(batch)]
     # Prompts, untimed: all but the last token of every prompt goes through the step function
     # directly, so that every request samples its first token in the same step and they decode in lockstep.
     from tessweave_engine_amd.engine import StepEntry
@@ -135,7 +144,7 @@ def serve_run(model, torch, args):
     while True:
         now = time.perf_counter() - t0
         while nxt < n and arrivals[nxt] <= now:
-            requests.append(engine.submit(prompts[nxt], max_tokens=outputs, ignore_eos=True))
+            requests.append(engine.submit(prompts[nxt], max_tokens=outputs, ignore_eos=True, stream=False))
             nxt += 1
         if engine.step():                       # False: nothing admitted and no token unread
             continue
@@ -157,6 +166,27 @@ def serve_run(model, torch, args):
             "ttft_ms_p50": round(ttft[n // 2], 1), "ttft_ms_p99": round(ttft[min(n - 1, int(n * 0.99))], 1),
             "steps": stats["steps"] - steps0, "graph_replays": stats["graph_replays"], "prefill_chunk": chunk,
             "max_active": active}
+
+
+def read_ceiling(torch, device, gigabytes=4):
+    """GB/s of a plain streaming reader (non-temporal 1 KB loads per wave, no arithmetic) over GIGABYTES of
+    device memory: the read bandwidth this device gives a kernel that does nothing else."""
+    from tessweave_engine_amd.kernels import ops
+    buffer = torch.empty(gigabytes << 30, dtype=torch.uint8, device=device)
+    buffer.zero_()
+    out = torch.zeros(1, dtype=torch.float32, device=device)
+    best = None
+    for _ in range(5):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        n = ops.probe_read(buffer, out, blocks=4096)
+        end.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(end)
+        best = ms if best is None else min(best, ms)
+    del buffer
+    torch.cuda.empty_cache()
+    return n / (best / 1000) / 1e9
 
 
 def prefill_run(model, torch, tokens, dtype, seed, repeats=3):
@@ -216,7 +246,7 @@ def main():
                           "tokens_per_s": round(args.prefill_tokens / (ms / 1000), 1)}))
         return 0
     value, ms_per_step, replays = decode_run(model, torch, args.batch, args.context, args.steps, args.warmup,
-                                             args.dtype, use_graphs, args.seed)
+                                             args.dtype, use_graphs, args.seed, args.max_context)
     element = 2 if args.dtype == "bfloat16" else 4
     layer_weights = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
         + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
@@ -238,8 +268,21 @@ def main():
     points = {}
     for b in [int(v) for v in args.points.split(",") if v]:
         steps = min(args.steps, 64)
-        tps, _, _ = decode_run(model, torch, b, args.context, steps, 8, args.dtype, use_graphs, args.seed)
+        tps, _, _ = decode_run(model, torch, b, args.context, steps, 8, args.dtype, use_graphs, args.seed,
+                               args.max_context)
         points[f"decode_b{b}"] = round(tps, 1)
+    if not args.no_extra_points:
+        # the same batch with the engine opened for 32,768 tokens a request (launch shapes must follow the
+        # lengths that are served, not the lengths that are allowed)
+        opened = min(32768, c.max_position_embeddings)
+        tps, _, _ = decode_run(model, torch, args.batch, args.context, min(args.steps, 64), 8, args.dtype, use_graphs,
+                               args.seed, opened)
+        points[f"decode_b{args.batch}_open{opened // 1024}k"] = round(tps, 1)
+        # prompts of 1,024 tokens, 512 generated (8 of them untimed): decoded tokens a second over the rest
+        for b in (1, 8, 64):
+            tps, _, _ = decode_run(model, torch, b, 1024 + 512, 504, 8, args.dtype, use_graphs, args.seed, opened)
+            points[f"gen512_b{b}"] = round(tps, 1)
+    ceiling = read_ceiling(torch, model.device)
 
     line = {
         "metric": f"decode tok/s @ batch {args.batch}, {shape_name} {'bf16' if args.dtype == 'bfloat16' else 'fp32'} "
@@ -258,7 +301,8 @@ def main():
         "prefill": {"value": round(t / (prefill_ms / 1000), 1), "tokens": t, "ms": round(prefill_ms, 3),
                     "frac": round(prefill_tflops / PEAK_TFLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "measured_read_ceiling": round(ceiling, 1),
+                     "frac_of_measured": round(achieved / ceiling, 4)},
         "points": points,
     }
     print(json.dumps(line))

@@ -33,3 +33,31 @@ extern "C" int tw_graph_launch(void* exec, hipStream_t stream) {
 }
 
 extern "C" int tw_graph_destroy(void* exec) { return (int)hipGraphExecDestroy((hipGraphExec_t)exec); }
+
+// ---- a yardstick, not part of any model: how fast can this device read memory at all? --------------------
+// Every wave streams 1 KB non-temporal loads, eight in flight, and adds them up; nothing is written unless
+// the sum takes one particular value (so the loads cannot be dropped). Benchmarks time it over gigabytes to
+// put a measured ceiling beside the nominal one.
+template <int U>
+__global__ __launch_bounds__(256) void probe_read_kernel(const f32x4* __restrict__ src, float* out, size_t vec_per_block) {
+  const f32x4* p = src + (size_t)blockIdx.x * vec_per_block + threadIdx.x;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (size_t i = 0; i < vec_per_block; i += 256 * U) {
+    f32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p + i + u * 256);
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc += v[u];
+  }
+  if (acc[0] + acc[1] + acc[2] + acc[3] == 12345.678f) out[0] = 1.f;
+}
+
+// Reads the first `blocks * floor(bytes / blocks / 32 KiB) * 32 KiB` bytes of src; returns that count in *read_bytes.
+extern "C" int tw_probe_read(const void* src, long bytes, float* out, int blocks, long* read_bytes, hipStream_t stream) {
+  TW_REQUIRE(src != nullptr && out != nullptr && blocks > 0 && (uintptr_t)src % 16 == 0);
+  const size_t per_block = (size_t)bytes / blocks / (256 * 8 * 16) * (256 * 8);      // in 16-byte vectors
+  TW_REQUIRE(per_block > 0);
+  if (read_bytes) *read_bytes = (long)(per_block * 16 * blocks);
+  probe_read_kernel<8><<<blocks, 256, 0, stream>>>((const f32x4*)src, out, per_block);
+  return TW_LAUNCH_RESULT();
+}

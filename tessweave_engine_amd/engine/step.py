@@ -10,8 +10,12 @@ packed on the host into a single int32 buffer, uploaded once, and every layer
 only reads it. Logits come back in float32 for exactly the rows asked for.
 
 Decode-only steps of a model whose parts are all graph-safe are captured once
-per batch size into a HIP graph and replayed; only the metadata upload differs
-between replays.
+per (batch size, length class) into a HIP graph and replayed; only the metadata
+upload differs between replays. The length class is the longest sequence of
+the step rounded up to a power of two: launch shapes that should follow the
+lengths (the number of key ranges of decode attention) follow the class, so an
+engine opened for 32,768 tokens that serves 2,000-token requests runs the
+launches of a 2,048-token engine.
 """
 from __future__ import annotations
 
@@ -37,6 +41,7 @@ def _round_up(v, m):
 
 
 GRAPH_SEGMENT_RUNS = 8       # layer runs per captured graph after the first
+MIN_LENGTH_CLASS = 512       # steps whose longest sequence is shorter share one captured graph
 
 
 class _Graph:
@@ -149,7 +154,7 @@ class Stepper:
         with torch.cuda.stream(self.stream):
             self.upload(ctx)
             if graphable:
-                logits = self._run_graphable(ctx, ctx.n_seqs)
+                logits = self._run_graphable(ctx, (ctx.n_seqs, ctx.kv_bound))
             else:
                 logits = self.model.forward(ctx)
         caller.wait_stream(self.stream)
@@ -263,6 +268,7 @@ class Stepper:
         ctx.max_q_len = int(q_lens[n_decode:].max()) if n_decode < n_seqs else 0
         ctx.max_kv_len = int(kv_len.max())
         ctx.kv_capacity = width * page
+        ctx.kv_bound = min(ctx.kv_capacity, max(MIN_LENGTH_CLASS, 1 << max(0, ctx.max_kv_len - 1).bit_length()))
         ctx.max_tokens = self.max_tokens
         ctx.cache, ctx.workspace = self.cache, self.workspace
         ctx.token_feed = self.token_feed
@@ -327,17 +333,18 @@ class Stepper:
             raise RuntimeError("a scratch buffer was allocated during graph capture")
         return _Graph(handles, logits, generation)
 
-    def _run_graphable(self, ctx, n_seqs):
-        graph = self._graphs.get(n_seqs)
+    def _run_graphable(self, ctx, key):
+        """KEY = (batch size, length class) names the captured graph this step can be replayed from."""
+        graph = self._graphs.get(key)
         if graph is not None and graph.generation != self.workspace.generation:
             self._drop_graphs()
             graph = None
         if graph is None:
-            if n_seqs not in self._warm:
-                # First time at this batch size: run eagerly so every scratch buffer exists.
-                self._warm.add(n_seqs)
+            if key not in self._warm:
+                # First time at this batch size and length class: run eagerly so every scratch buffer exists.
+                self._warm.add(key)
                 return self.model.forward(ctx)
-            graph = self._graphs[n_seqs] = self._capture(ctx)
+            graph = self._graphs[key] = self._capture(ctx)
         lib = library()
         for handle in graph.handles:
             check(lib.tw_graph_launch(handle, self.stream.cuda_stream), "graph launch")

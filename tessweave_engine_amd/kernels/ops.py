@@ -44,6 +44,17 @@ def dtype_id(dtype):
     return _DTYPE_ID[dtype]
 
 
+def probe_read(buffer, out, blocks=2048):
+    """Launch the plain streaming reader over BUFFER (any contiguous device tensor); returns the bytes it reads.
+    A yardstick for benchmarks: time it to get the device's own read ceiling."""
+    import ctypes
+    _need(buffer.is_contiguous(), "probe_read needs a contiguous buffer")
+    n = ctypes.c_long(0)
+    check(library().tw_probe_read(_dev(buffer), buffer.numel() * buffer.element_size(), _dev(out, torch.float32, "out"),
+                                  int(blocks), ctypes.byref(n), _stream()), "probe_read")
+    return int(n.value)
+
+
 def embed_gather(ids, table, out, feed=None):
     """out[n, :] = float32(table[ids[n], :]); an id -1 - k stands for feed[k] (int32, on the device)."""
     n = ids.numel()

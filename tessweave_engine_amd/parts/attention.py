@@ -76,14 +76,18 @@ class GroupedQueryAttention(Mixer):
         out = ctx.scratch("attn.out", (n, self.q_heads * self.head_dim))
         window = self.window or 0
         if ctx.n_decode:
-            # Under graph capture the split count may not depend on this step's lengths.
-            longest = ctx.kv_capacity if ctx.capturing else ctx.max_kv_len
+            # A captured step is replayed for other lengths: its split count follows the step's length
+            # class (the kernel itself cuts each sequence's own keys into that many ranges).
+            longest = ctx.kv_bound if ctx.capturing else ctx.max_kv_len
             if window:
                 longest = min(longest, window)
             splits = ops.attn_decode_splits(ctx.n_decode, self.q_heads, self.kv_heads, longest)
             ws = None
             if splits > 1:
-                floats = ops.attn_decode_workspace_floats(ctx.n_decode, self.q_heads, self.head_dim, splits)
+                # sized for the most splits any length class can ask for, so that it never grows under a capture
+                most = max(splits, ops.attn_decode_splits(ctx.n_decode, self.q_heads, self.kv_heads,
+                                                          min(ctx.kv_capacity, window) if window else ctx.kv_capacity))
+                floats = ops.attn_decode_workspace_floats(ctx.n_decode, self.q_heads, self.head_dim, most)
                 ws = ctx.workspace.get("attn.split", (floats,), torch.float32)
             ops.attn_decode(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode, out,
                             self.q_heads, self.kv_heads, self.head_dim, self.scale, window=window,

@@ -169,8 +169,10 @@ class StepContext:
         self.max_q_len = 0           # over the sequences after the first n_decode
         self.max_kv_len = 0
         self.kv_capacity = 0         # most keys a sequence can ever hold (block-table width * page size)
+        self.kv_bound = 0            # while capturing: the step's length class, an upper bound of every kv_len that
+                                     # a replay of this capture will see (a power of two, at most kv_capacity)
         self.token_feed = None       # int32 device tensor: a token id -1 - k in token_ids stands for token_feed[k]
-        self.capturing = False       # launches must not depend on this step's lengths
+        self.capturing = False       # launches may depend on kv_bound and capacities, not on this step's lengths
         self.segment_end = None      # while a step is captured: called with the index of each finished layer run
         self.max_tokens = 0          # row capacity of per-token scratch buffers
         self.cache = None            # cache.CacheManager

@@ -241,3 +241,33 @@ def test_a_2048_token_portion_in_one_step_then_decoding_past_4096_keys(wide_long
         assert worst_engine <= 4 * worst_plain + 1e-6, (worst_engine, worst_plain)
     cache.close(seq)
     stepper.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_across_a_length_class_takes_a_second_graph_and_changes_nothing(long_model, dtype):
+    """Captured decode steps are keyed by (batch size, length class): a request that grows from 500 to 530
+    tokens leaves the class of 512 for that of 1,024. Every logits row is compared, and both graphs replay."""
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.weights import load_model
+    page, vocab = long_model["page"], long_model["cfg"]["vocab_size"]
+    g = torch.Generator().manual_seed(512)
+    tokens = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (530, 60)]
+    want = [plain.forward(long_model["config"], long_model["weights"], t) for t in tokens]
+    model = load_model(long_model["folder"], dtype=dtype, device="cuda:0")
+    cache = CacheManager(model.cache_layout(), page, 64, 2, dtype=dtype, device=model.device, prefix_cache=False,
+                         max_request_tokens=8192)
+    stepper = Stepper(model, cache, max_step_tokens=512, max_step_seqs=2)
+    seqs = [cache.open("long"), cache.open("short")]
+    stepper.step([StepEntry(seqs[0], tokens[0][:500], []), StepEntry(seqs[1], tokens[1][:30], [])])
+    for s in range(30):
+        got = stepper.step([StepEntry(seqs[0], [tokens[0][500 + s]], [0]), StepEntry(seqs[1], [tokens[1][30 + s]], [0])]).cpu()
+        for r, (i, pos) in enumerate(((0, 500 + s), (1, 30 + s))):
+            w = want[i][pos]
+            if dtype == "float32":
+                assert torch.allclose(got[r], w, atol=5e-6, rtol=2e-5), (i, pos)
+            else:
+                assert float((got[r] - w).abs().max()) <= 0.02 * float(w.abs().max()), (i, pos)
+    assert sorted(stepper._graphs) == [(2, 512), (2, 1024)]
+    assert stepper.graph_replays == 30 - 4                 # one eager and one capturing step per class
+    stepper.close()
