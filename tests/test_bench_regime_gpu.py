@@ -269,5 +269,5 @@ def test_decoding_across_a_length_class_takes_a_second_graph_and_changes_nothing
             else:
                 assert float((got[r] - w).abs().max()) <= 0.02 * float(w.abs().max()), (i, pos)
     assert sorted(stepper._graphs) == [(2, 512), (2, 1024)]
-    assert stepper.graph_replays == 30 - 4                 # one eager and one capturing step per class
+    assert stepper.graph_replays == 30 - 2                 # the first step of each class runs eagerly, the next is captured
     stepper.close()
