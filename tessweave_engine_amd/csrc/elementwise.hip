@@ -266,8 +266,8 @@ extern "C" int tw_rope_table(const int* positions, const float* inv_freq, float*
 
 // ---- rotation of q and k, and the cache write ----------------------------------------------
 // qkv[n] = [q heads | k heads | v heads], head-major, `ld` elements per row.
-// Pair j of a head is (x[j], x[j + rot/2]) for j < rot/2 (rotate-half); elements
-// from `rot` on are not rotated. q is rotated in place. Rotated k goes to
+// Pair j of a head is (x[j], x[j + rot/2]) for j < rot/2 (rotate-half), or, with `adjacent`,
+// (x[2j], x[2j + 1]); elements from `rot` on are not rotated. q is rotated in place. Rotated k goes to
 //   keys  [page][kv_head][offset][d]      and raw v to
 //   values[page][kv_head][d][offset]      (transposed inside the page),
 // slot = page * page_size + offset; a negative slot writes nothing.
@@ -284,7 +284,8 @@ template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* __restrict__ cos_t,
                                      const float* __restrict__ sin_t, const int* __restrict__ slots,
                                      T* __restrict__ keys, T* __restrict__ values, int q_heads,
-                                     int kv_heads, int head_dim, int rot, int page_size, int write_cache) {
+                                     int kv_heads, int head_dim, int rot, int page_size, int write_cache,
+                                     int adjacent) {
   const int n = blockIdx.x;
   const int half = rot / 2;
   T* row = qkv + (size_t)n * ld;
@@ -298,18 +299,19 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* 
   for (int i = threadIdx.x; i < rot_heads * half; i += blockDim.x) {
     const int head = i / half, j = i % half;
     T* x = row + (size_t)head * head_dim;
-    const float lo = tw_to_float(x[j]), hi = tw_to_float(x[j + half]);
+    const int i_lo = adjacent ? 2 * j : j, i_hi = adjacent ? 2 * j + 1 : j + half;
+    const float lo = tw_to_float(x[i_lo]), hi = tw_to_float(x[i_hi]);
     float r_lo, r_hi;
     tw_rotate_pair(lo, hi, c[j], s[j], r_lo, r_hi);
     const T out_lo = tw_from_float<T>(r_lo), out_hi = tw_from_float<T>(r_hi);
     if (head < q_heads) {
-      x[j] = out_lo;
-      x[j + half] = out_hi;
+      x[i_lo] = out_lo;
+      x[i_hi] = out_hi;
     } else if (slot >= 0) {
       const int kh = head - q_heads;
       T* dst = keys + (((size_t)page * kv_heads + kh) * page_size + off) * head_dim;
-      dst[j] = out_lo;
-      dst[j + half] = out_hi;
+      dst[i_lo] = out_lo;
+      dst[i_hi] = out_hi;
     }
   }
   if (slot < 0) return;
@@ -337,7 +339,7 @@ __global__ void qkv_finish_kernel(T* __restrict__ qkv, long ld, const float* __r
                                   T* __restrict__ keys, T* __restrict__ values, int q_heads, int kv_heads,
                                   int head_dim, int rot, int page_size, int write_cache,
                                   const float* __restrict__ partial, int splits, size_t split_stride,
-                                  const float* __restrict__ bias) {
+                                  const float* __restrict__ bias, int adjacent) {
   const int head = blockIdx.x, n = blockIdx.y;
   const int width = (q_heads + 2 * kv_heads) * head_dim;
   const int half = rot / 2;
@@ -380,12 +382,13 @@ __global__ void qkv_finish_kernel(T* __restrict__ qkv, long ld, const float* __r
     T* dst = is_q ? row : keys + (((size_t)page * kv_heads + (head - q_heads)) * page_size + off) * head_dim;
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
       const float cj = cos_t[(size_t)n * half + j], sj = sin_t[(size_t)n * half + j];
+      const int i_lo = adjacent ? 2 * j : j, i_hi = adjacent ? 2 * j + 1 : j + half;
       float lo, hi;
-      values2(j, j + half, lo, hi);
+      values2(i_lo, i_hi, lo, hi);
       float r_lo, r_hi;
       tw_rotate_pair(lo, hi, cj, sj, r_lo, r_hi);
-      dst[j] = tw_from_float<T>(r_lo);
-      dst[j + half] = tw_from_float<T>(r_hi);
+      dst[i_lo] = tw_from_float<T>(r_lo);
+      dst[i_hi] = tw_from_float<T>(r_hi);
     }
     for (int d = rot + threadIdx.x; d < head_dim; d += 2 * blockDim.x) {      // the part that is not rotated
       const int d1 = d + blockDim.x < head_dim ? d + blockDim.x : d;
@@ -411,7 +414,8 @@ __global__ void qkv_finish_kernel(T* __restrict__ qkv, long ld, const float* __r
 extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_t, const float* sin_t,
                                 const int* slots, void* keys, void* values, int n, int q_heads,
                                 int kv_heads, int head_dim, int rot, int page_size, int write_cache,
-                                const float* partial, int splits, const float* bias, hipStream_t stream) {
+                                const float* partial, int splits, const float* bias, int adjacent,
+                                hipStream_t stream) {
   TW_REQUIRE(partial == nullptr || splits >= 1);
   const size_t split_stride = (size_t)n * (q_heads + 2 * kv_heads) * head_dim;
   TW_REQUIRE(n >= 0 && q_heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0);
@@ -426,11 +430,11 @@ extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_
     if (dtype == TW_DTYPE_F32)
       qkv_finish_kernel<float><<<grid, threads, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
                                                             (float*)values, q_heads, kv_heads, head_dim, rot,
-                                                            page_size, write_cache, partial, splits, split_stride, bias);
+                                                            page_size, write_cache, partial, splits, split_stride, bias, adjacent);
     else if (dtype == TW_DTYPE_BF16)
       qkv_finish_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots, (bf16_t*)keys,
                                                              (bf16_t*)values, q_heads, kv_heads, head_dim, rot,
-                                                             page_size, write_cache, partial, splits, split_stride, bias);
+                                                             page_size, write_cache, partial, splits, split_stride, bias, adjacent);
     else
       return TW_ERR_BAD_ARGUMENT;
     return TW_LAUNCH_RESULT();
@@ -438,11 +442,11 @@ extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_
   if (dtype == TW_DTYPE_F32)
     rope_kv_write_kernel<float><<<n, 256, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
                                                        (float*)values, q_heads, kv_heads, head_dim, rot,
-                                                       page_size, write_cache);
+                                                       page_size, write_cache, adjacent);
   else if (dtype == TW_DTYPE_BF16)
     rope_kv_write_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots,
                                                         (bf16_t*)keys, (bf16_t*)values, q_heads, kv_heads,
-                                                        head_dim, rot, page_size, write_cache);
+                                                        head_dim, rot, page_size, write_cache, adjacent);
   else
     return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();

@@ -62,6 +62,7 @@ class Stepper:
         self.workspace = Workspace(self.device)
         self.stream = torch.cuda.Stream(device=self.device)
         self.use_graphs = bool(use_graphs) and model.graph_safe_model
+        self._defer_sums = bool(getattr(model, "defers_sums", False))
         self.max_tokens = 0
         self.max_seqs = 0
         self._graphs = {}
@@ -272,6 +273,7 @@ class Stepper:
         ctx.max_tokens = self.max_tokens
         ctx.cache, ctx.workspace = self.cache, self.workspace
         ctx.token_feed = self.token_feed
+        ctx.defer_sums = self._defer_sums
 
         graphable = (self.use_graphs and n_decode == n_seqs and n_logits == n_seqs
                      and rows == list(range(n_seqs)))

@@ -21,7 +21,7 @@ _SIGNATURES = {
     "tw_embed_gather": (I, [I, P, P, P, I, I, I, P, I, P]),
     "tw_rmsnorm": (I, [I, P, P, P, P, I, I, F, P, I, L, P, P]),
     "tw_rope_table": (I, [P, P, P, P, I, I, P]),
-    "tw_rope_kv_write": (I, [I, P, L, P, P, P, P, P, I, I, I, I, I, I, I, P, I, P, P]),
+    "tw_rope_kv_write": (I, [I, P, L, P, P, P, P, P, I, I, I, I, I, I, I, P, I, P, I, P]),
     "tw_silu_mul": (I, [I, P, P, I, I, P]),
     "tw_linear_workspace_bytes": (L, [I, I, I, I]),
     "tw_linear_partial_splits": (I, [I, I, I]),

@@ -110,8 +110,10 @@ def rope_table(positions, inv_freq, cos, sin):
 
 
 def rope_kv_write(qkv, cos, sin, slots, keys, values, q_heads, kv_heads, head_dim, page_size,
-                  write_cache=True, partial=None, bias=None):
+                  write_cache=True, partial=None, bias=None, adjacent=False):
     """Rotate q (in place) and k of qkv[n] = [q | k | v]; write rotated k and v to the pages.
+
+    Pair j of a head is elements (j, j + rot/2), or with `adjacent` elements (2j, 2j + 1).
 
     keys [pages, kv_heads, page_size, head_dim]; values hold the same number of
     elements and are written as [pages, kv_heads, head_dim, page_size].
@@ -146,7 +148,7 @@ def rope_kv_write(qkv, cos, sin, slots, keys, values, q_heads, kv_heads, head_di
         _dev(partial, torch.float32, "partial") if partial is not None else None,
         partial.shape[0] if partial is not None else 0,
         _dev(bias, torch.float32, "bias") if (partial is not None and bias is not None) else None,
-        _stream()), "rope_kv_write")
+        1 if adjacent else 0, _stream()), "rope_kv_write")
 
 
 def silu_mul(gate_up, out):

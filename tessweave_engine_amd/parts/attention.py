@@ -61,6 +61,7 @@ class GroupedQueryAttention(Mixer):
         width = (self.q_heads + 2 * self.kv_heads) * self.head_dim
         qkv = ctx.scratch("attn.qkv", (n, width))
         cos, sin = self.position.tables(ctx)
+        adjacent = self.position.pairing == "adjacent"
         keys, values, g = ctx.cache.keys_values(run.cache_slot)
         group = ctx.groups[g]
         if self.qkv.deferrable(n):
@@ -68,11 +69,12 @@ class GroupedQueryAttention(Mixer):
             partial = self.qkv.forward_partials(ctx, h, "qkv")
             ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
                               self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache,
-                              partial=partial, bias=self.qkv.biases[0] if self.qkv.biases else None)
+                              partial=partial, bias=self.qkv.biases[0] if self.qkv.biases else None,
+                              adjacent=adjacent)
         else:
             self.qkv.forward(ctx, h, qkv)
             ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
-                              self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache)
+                              self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache, adjacent=adjacent)
         out = ctx.scratch("attn.out", (n, self.q_heads * self.head_dim))
         window = self.window or 0
         if ctx.n_decode:
@@ -103,7 +105,7 @@ class GroupedQueryAttention(Mixer):
             ops.attn_prefill(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode,
                              ctx.n_seqs - ctx.n_decode, ctx.max_q_len, out, self.q_heads, self.kv_heads,
                              self.head_dim, self.scale, window=window, split=split, workspace=ws)
-        if not self.o.biases and self.o.deferrable(n):
+        if ctx.defer_sums and not self.o.biases and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # the next norm adds them into x
         self.o.forward(ctx, out, x, residual=x)
         return None

@@ -49,11 +49,16 @@ class Part:
 
 
 class Norm(Part):
-    def forward(self, ctx, x, rows=None, add=None):
+    #: True if `forward` takes `add`: pending partial sums (float32 [splits, n, hidden]) that the part
+    #: before left to be added into x first (see `Mixer.forward`). A model defers such sums only if every
+    #: one of its norms says so; a norm that leaves this False is never handed any.
+    folds_pending = False
+
+    def forward(self, ctx, x, rows=None):
         """x float32 [n, hidden] -> normalised rows in the compute type.
 
-        add: pending partial sums (float32 [splits, n, hidden]) of the part before, to be
-        added into x first (see `Mixer.forward`). rows: int32 indices of the rows wanted.
+        rows: int32 indices (on the device) of the rows wanted; None: all of them.
+        Norms with `folds_pending` also take add=..., see above.
         """
         raise NotImplementedError
 
@@ -62,6 +67,9 @@ class PositionEncoding(Part):
     """Rotary-style encodings hand per-token (cos, sin) tables to the mixers that use them."""
 
     rotary_dim = 0
+    #: which two elements of a head turn together: "half" pairs element j with j + rotary_dim/2,
+    #: "adjacent" pairs element 2j with 2j + 1
+    pairing = "half"
 
     def tables(self, ctx):
         raise NotImplementedError
@@ -75,9 +83,10 @@ class Mixer(Part):
     def forward(self, ctx, run, h, x):
         """Add the mixer's output for normalised input H into the residual stream X (float32, in place).
 
-        Returns None, or PENDING partial sums (float32 [splits, n, hidden]) that are not yet in X:
-        whoever runs next (the following norm) adds them up and into X. This saves a kernel per
-        projection when a step has few rows.
+        Returns None, or, only if `ctx.defer_sums` allows it, PENDING partial sums (float32
+        [splits, n, hidden]) that are not yet in X: whoever runs next (the following norm) adds them up
+        and into X. This saves a kernel per projection when a step has few rows. A part that always
+        returns None is a complete part.
         """
         raise NotImplementedError
 
@@ -172,6 +181,7 @@ class StepContext:
         self.kv_bound = 0            # while capturing: the step's length class, an upper bound of every kv_len that
                                      # a replay of this capture will see (a power of two, at most kv_capacity)
         self.token_feed = None       # int32 device tensor: a token id -1 - k in token_ids stands for token_feed[k]
+        self.defer_sums = True       # may a mixer or feed-forward leave partial sums pending for the next norm?
         self.capturing = False       # launches may depend on kv_bound and capacities, not on this step's lengths
         self.segment_end = None      # while a step is captured: called with the index of each finished layer run
         self.max_tokens = 0          # row capacity of per-token scratch buffers

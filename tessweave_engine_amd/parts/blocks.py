@@ -4,7 +4,7 @@
 """
 from __future__ import annotations
 
-from .base import Block
+from .base import Block, fold_pending
 
 
 class PreNormBlock(Block):
@@ -22,7 +22,17 @@ class PreNormBlock(Block):
             p.bind(tensors, dtype, device)
 
     def forward(self, ctx, run, x, pending=None):
-        h = self.mixer_norm.forward(ctx, x, add=pending)
+        h = normalise(self.mixer_norm, ctx, x, pending)
         pending = self.mixer.forward(ctx, run, h, x)
-        h = self.ffn_norm.forward(ctx, x, add=pending)
+        h = normalise(self.ffn_norm, ctx, x, pending)
         return self.ffn.forward(ctx, h, x)
+
+
+def normalise(norm, ctx, x, pending=None, rows=None):
+    """NORM of X; PENDING partial sums go to a norm that folds them, and are folded here for one that does not
+    (which only happens when parts are driven by hand: a model defers sums only if all its norms fold them)."""
+    if pending is not None and not norm.folds_pending:
+        pending = fold_pending(x, pending)
+    if pending is not None:
+        return norm.forward(ctx, x, rows=rows, add=pending)
+    return norm.forward(ctx, x, rows=rows)

@@ -4,7 +4,8 @@ from __future__ import annotations
 import torch
 
 from ..cache.spec import CacheLayout
-from .base import LayerRun, Part
+from .base import LayerRun, Norm, Part
+from .blocks import normalise
 
 
 def walk(part):
@@ -40,6 +41,11 @@ class DecoderModel(Part):
     @property
     def graph_safe_model(self):
         return all(p.graph_safe for p in walk(self))
+
+    @property
+    def defers_sums(self):
+        """May mixers and feed-forwards leave split-K sums to the next norm? Only if every norm folds them."""
+        return all(p.folds_pending for p in walk(self) if isinstance(p, Norm))
 
     def tensor_specs(self):
         specs, seen = [], set()
@@ -105,5 +111,5 @@ class DecoderModel(Part):
                 ctx.segment_end(i)
         if ctx.n_logits == 0:
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=ctx.device)
-        h = self.final_norm.forward(ctx, x, rows=ctx.logit_rows, add=pending, tag="norm.final")
+        h = normalise(self.final_norm, ctx, x, pending, rows=ctx.logit_rows)
         return self.head.forward(ctx, h)

@@ -12,6 +12,8 @@ from .base import Norm
 
 
 class RMSNorm(Norm):
+    folds_pending = True
+
     def __init__(self, name, size, eps):
         self.name = name
         self.size = int(size)
@@ -24,7 +26,8 @@ class RMSNorm(Norm):
     def bind(self, tensors, dtype, device):
         self.weight = tensors.pop(self.name + ".weight").contiguous()
 
-    def forward(self, ctx, x, rows=None, add=None, tag="norm.out"):
+    def forward(self, ctx, x, rows=None, add=None):
+        tag = "norm.out" if rows is None else "norm.rows"        # a model's last norm (chosen rows) keeps its own buffer
         n_out = rows.numel() if rows is not None else x.shape[0]
         out = ctx.scratch(tag, (n_out, self.size))
         scratch = None

@@ -14,7 +14,10 @@ from .base import PositionEncoding
 
 
 class RotaryEmbedding(PositionEncoding):
-    def __init__(self, head_dim, theta, rotary_dim=None):
+    def __init__(self, head_dim, theta, rotary_dim=None, pairing="half"):
+        if pairing not in ("half", "adjacent"):
+            raise ValueError("pairing must be 'half' or 'adjacent'")
+        self.pairing = pairing
         self.head_dim = int(head_dim)
         self.theta = float(theta)
         self.rotary_dim = int(rotary_dim if rotary_dim is not None else head_dim)

@@ -317,7 +317,7 @@ def test_each_part_alone(tiny, dtype):
         torch.testing.assert_close(xb.cpu(), want_b, **(tight if dtype == "float32" else dict(atol=6e-2, rtol=6e-2)))
         # head on chosen rows
         rows = torch.tensor([0, n - 1], dtype=torch.int32, device="cuda")
-        hf = model.final_norm.forward(ctx, xd, rows=rows, tag="norm.final")
+        hf = model.final_norm.forward(ctx, xd, rows=rows)
         logits = model.head.forward(ctx, hf)
         head_w = w["model.embed_tokens.weight"] if s["tied"] else w["lm_head.weight"]
         want_l = plain.rms_norm(x0[[0, n - 1]], w["model.norm.weight"], s["eps"]) @ head_w.T
@@ -678,3 +678,115 @@ def test_toy_routed_feed_forward_scaled_partial_rotary_and_a_window(tmp_path, de
         stepper.close()
     finally:
         unregister_architecture("ToyRoutedForCausalLM")
+
+
+def test_a_norm_that_folds_nothing_and_a_rotation_of_adjacent_pairs(tmp_path, device):
+    """Two more toy parts, built outside the package: a norm that knows nothing of pending partial sums (the
+    model then never defers any) and a rotary encoding that turns elements (2j, 2j + 1) of the first 8 of 16.
+    Float32, a prompt in two portions and decoded tokens, against formulas written out here (the kernel behind
+    the pairing is compared in both precisions in test_kernels_gpu)."""
+    from dataclasses import dataclass
+    from safetensors.torch import save_file
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.config import register_architecture, unregister_architecture
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.parts import (DecoderModel, GroupedQueryAttention, Norm, OutputHead, PreNormBlock,
+                                            RotaryEmbedding, SwiGLU, TokenEmbedding)
+    from tessweave_engine_amd.weights import VECTOR, ONE_PLUS_NORMAL, TensorSpec, load_model, random_tensors
+
+    H, HEADS, KV, D, ROT, THETA, INTER, VOCAB = 32, 2, 1, 16, 8, 100.0, 48, 41
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str = "ToyCenteredForCausalLM"
+        vocab_size: int = VOCAB
+        max_position_embeddings: int = 128
+        eos_token_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return dict(architectures=[self.architecture], model_type="toy_centered", vocab_size=self.vocab_size)
+
+    class CenteredNorm(Norm):
+        """(x - mean) / sqrt(var + eps) * weight, written with torch operations; takes no pending sums."""
+        graph_safe = False
+
+        def __init__(self, name, size, eps):
+            self.name, self.size, self.eps = name, size, eps
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.size,), VECTOR, ONE_PLUS_NORMAL)]
+
+        def bind(self, tensors, dtype, device):
+            self.weight, self.dtype = tensors.pop(self.name + ".weight"), dtype
+
+        def forward(self, ctx, x, rows=None):
+            if rows is not None:
+                x = x[rows.long()]
+            c = x - x.mean(-1, keepdim=True)
+            return (c * torch.rsqrt(c.square().mean(-1, keepdim=True) + self.eps) * self.weight).to(self.dtype).contiguous()
+
+    def build_toy(c):
+        emb = TokenEmbedding("emb", c.vocab_size, H)
+        rotary = RotaryEmbedding(D, THETA, rotary_dim=ROT, pairing="adjacent")
+        blocks = [PreNormBlock(CenteredNorm(f"l{i}.n1", H, 1e-5),
+                               GroupedQueryAttention(f"l{i}.att.", H, HEADS, KV, D, rotary, qkv_bias=True),
+                               CenteredNorm(f"l{i}.n2", H, 1e-5), SwiGLU(f"l{i}.ff.", H, INTER)) for i in range(2)]
+        return DecoderModel(c, emb, blocks, CenteredNorm("final", H, 1e-5), OutputHead("head", c.vocab_size, H, tied_to=emb))
+
+    register_architecture("ToyCenteredForCausalLM", "toy_centered", ToyConfig, build_toy)
+    try:
+        cfg = ToyConfig()
+        (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+        tensors = random_tensors(build_toy(cfg).tensor_specs(), 9, std=0.3)
+        save_file(tensors, str(tmp_path / "model.safetensors"))
+        w = {k: v.float() for k, v in tensors.items()}
+
+        def norm(x, weight):
+            c = x - x.mean(-1, keepdim=True)
+            return c / torch.sqrt((c * c).mean(-1, keepdim=True) + 1e-5) * weight
+
+        def rotate(t, pos):
+            inv = THETA ** (-torch.arange(0, ROT, 2, dtype=torch.float32) / ROT)
+            angle = pos.float()[:, None] * inv[None, :]
+            cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+            out = t.clone()
+            even, odd = t[..., 0:ROT:2], t[..., 1:ROT:2]
+            out[..., 0:ROT:2], out[..., 1:ROT:2] = even * cos - odd * sin, odd * cos + even * sin
+            return out
+
+        def plain_toy(tokens):
+            x = w["emb.weight"][torch.tensor(tokens)]
+            t, pos = len(tokens), torch.arange(len(tokens))
+            for i in range(2):
+                p = f"l{i}."
+                hn = norm(x, w[p + "n1.weight"])
+                q, k, v = (hn @ w[p + f"att.{n}_proj.weight"].T + w[p + f"att.{n}_proj.bias"] for n in "qkv")
+                att = plain.attention(rotate(q.reshape(t, HEADS, D), pos), rotate(k.reshape(t, KV, D), pos),
+                                      v.reshape(t, KV, D), pos)
+                x = x + att.reshape(t, HEADS * D) @ w[p + "att.o_proj.weight"].T
+                hn = norm(x, w[p + "n2.weight"])
+                x = x + plain.swiglu(hn, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+            return norm(x, w["final.weight"]) @ w["emb.weight"].T
+
+        tokens = torch.randint(0, VOCAB, (40,), generator=torch.Generator().manual_seed(4)).tolist()
+        want = plain_toy(tokens)
+        for dtype in ("float32",):
+            model = load_model(tmp_path, dtype=dtype, device="cuda:0")
+            assert not model.defers_sums and not model.graph_safe_model
+            cache = CacheManager(model.cache_layout(), 8, 8, 1, dtype=dtype, device=model.device, prefix_cache=False,
+                                 max_request_tokens=48)
+            stepper = Stepper(model, cache, max_step_tokens=32)
+            seq = cache.open("r")
+            got = [stepper.step([StepEntry(seq, tokens[:19], list(range(19)))]).cpu().clone(),
+                   stepper.step([StepEntry(seq, tokens[19:30], list(range(11)))]).cpu().clone()]
+            got += [stepper.step([StepEntry(seq, [t], [0])]).cpu().clone() for t in tokens[30:]]
+            got = torch.cat(got)
+            torch.testing.assert_close(got, want, atol=3e-5, rtol=3e-5)
+            cache.close(seq)
+            stepper.close()
+    finally:
+        unregister_architecture("ToyCenteredForCausalLM")

@@ -135,6 +135,53 @@ def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, p
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("head_dim,rot", [(16, 16), (32, 12), (48, 48)])
+def test_rope_with_adjacent_pairs(ops, device, dtype, head_dim, rot):
+    """Pairs (2j, 2j + 1) instead of (j, j + rot/2): the same rotation applied to the de-interleaved head."""
+    n, q_heads, kv_heads, page, pages, theta = 6, 3, 1, 4, 5, 1e4
+    width = (q_heads + 2 * kv_heads) * head_dim
+    qkv = rand((n, width), dtype, device)
+    positions = torch.tensor([0, 1, 7, 300, 301, 2], dtype=torch.int32, device=device)
+    inv = (theta ** (-torch.arange(0, rot, 2, dtype=torch.float32) / rot)).to(device)
+    cos, sin = torch.empty(n, rot // 2, device=device), torch.empty(n, rot // 2, device=device)
+    ops.rope_table(positions, inv, cos, sin)
+    slots = torch.tensor([4, 5, 0, 19, 9, 13], dtype=torch.int32, device=device)
+    src = qkv.float().cpu()
+
+    def want(block, heads):
+        x = block.reshape(n, heads, head_dim)
+        head = x[..., :rot]
+        halves = torch.cat((head[..., 0::2], head[..., 1::2]), -1)              # (2j, 2j + 1) -> (j, j + rot/2)
+        turned = plain.rope(halves, positions.cpu(), theta)
+        back = torch.empty_like(head)
+        back[..., 0::2], back[..., 1::2] = turned[..., :rot // 2], turned[..., rot // 2:]
+        return torch.cat((back, x[..., rot:]), -1)
+    q_want = want(src[:, :q_heads * head_dim], q_heads)
+    k_want = want(src[:, q_heads * head_dim:(q_heads + kv_heads) * head_dim], kv_heads)
+    t = tol(dtype, (2e-6, 2e-6), (1e-2, 1e-2))
+    bias = rand((width,), torch.float32, device, 0.3, seed=9)
+    for from_partials in (False, True):
+        keys = torch.zeros((pages, kv_heads, page, head_dim), dtype=dtype, device=device)
+        values = torch.zeros_like(keys)
+        if from_partials:                       # the same from split-K sums (no bias here: zeros)
+            parts = torch.stack([qkv.float() * 0.25, qkv.float() * 0.75])
+            got = torch.full((n, width), float("nan"), dtype=dtype, device=device)
+            ops.rope_kv_write(got, cos, sin, slots, keys, values, q_heads, kv_heads, head_dim, page, partial=parts,
+                              bias=torch.zeros_like(bias), adjacent=True)
+        else:
+            got = qkv.clone()
+            ops.rope_kv_write(got, cos, sin, slots, keys, values, q_heads, kv_heads, head_dim, page, adjacent=True)
+        torch.testing.assert_close(got[:, :q_heads * head_dim].float().cpu().reshape(n, q_heads, head_dim), q_want, **t)
+        kc = keys.float().cpu()
+        for i, slot in enumerate(slots.tolist()):
+            torch.testing.assert_close(kc[slot // page, :, slot % page, :], k_want[i], **t)
+    half_form = qkv.clone()
+    ops.rope_kv_write(half_form, cos, sin, slots, torch.zeros_like(keys), torch.zeros_like(values), q_heads, kv_heads,
+                      head_dim, page)
+    assert not torch.allclose(half_form[:, :q_heads * head_dim].float().cpu().reshape(n, q_heads, head_dim), q_want, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_silu_mul(ops, device, dtype):
     gu = rand((5, 2 * 70), dtype, device, 2.0)
     out = torch.empty(5, 70, dtype=dtype, device=device)
