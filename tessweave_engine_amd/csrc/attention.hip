@@ -1148,16 +1148,14 @@ static int decode_launch(AttnArgs a, int n_seqs, int generic, hipStream_t stream
   else
     attn_decode_kernel<T, 16><<<grid, 256, 0, stream>>>(a);
   int err = TW_LAUNCH_RESULT();
-  if (err || a.splits == 1 || a.out == nullptr) return err;       // no output: the caller merges the partial results
+  if (err || a.splits == 1) return err;
   attn_decode_reduce_kernel<T><<<dim3(a.q_heads, n_seqs), TW_REDUCE_THREADS, 0, stream>>>(
       a.part_o, a.part_ml, a.q_start, a.seq0, (T*)a.out, a.ldo, a.q_heads, a.head_dim, a.splits);
   return TW_LAUNCH_RESULT();
 }
 
 // Sequences seq0 .. seq0 + n_seqs - 1 must each have exactly one token in this step.
-// `workspace` holds tw_attn_decode_workspace_floats floats when splits > 1. With splits > 1, `out` may be
-// null: the partial results then stay in the workspace, part_o [n_seqs][q_heads][splits][head_dim]
-// followed by part_ml [n_seqs][q_heads][splits][2] (max, sum), for a caller that merges them itself.
+// `workspace` holds tw_attn_decode_workspace_floats floats when splits > 1.
 // generic != 0 forces the kernel that takes every type and page size.
 extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* keys, const void* values,
                               const int* block_table, int table_stride, const int* q_start,
@@ -1177,7 +1175,6 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
   int err = check_common(a);
   if (err) return err;
   TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && splits >= 1 && splits <= 64 && n_seqs <= 65535);
-  TW_REQUIRE(out != nullptr || splits > 1);
   if (n_seqs == 0) return 0;
   if (splits > 1) {
     TW_REQUIRE(workspace != nullptr);

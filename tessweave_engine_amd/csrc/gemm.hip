@@ -211,123 +211,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const T* __
 }
 
 // =====================================================================================
-// The skinny kernel for the output projection of a decode step, reading decode attention's split-KV
-// partial results itself. Row r of A (at most 16 rows) is token r's attention output; head h's dims are
-//   (sum_s w_s po[r][h][s][:]) / (sum_s w_s l_s),   w_s = exp(m_s - max_s m_s),
-// exactly what attn_decode_reduce_kernel would write, rounded to T as it would be. Each workgroup merges
-// only its own K range (a few heads) into LDS while its first weights are on their way, so the merge
-// kernel and its launch go; the activations then never leave LDS, and the waves meet at no further
-// barrier. Always writes float32 partial sums partial[split][M][N] (the caller's next kernel adds them).
-// =====================================================================================
-#define TW_MERGED_STEPS 32                   /* most MFMA steps (64 bytes of a row each) of a workgroup's K range */
-
-template <typename T, int U>
-__global__ __launch_bounds__(256) void gemm_skinny_merged_kernel(const float* __restrict__ part_o,
-                                                                  const float* __restrict__ part_ml, int heads,
-                                                                  int head_dim, int att_splits,
-                                                                  const T* __restrict__ W, long ldw,
-                                                                  float* __restrict__ partial, int M, int N, int K,
-                                                                  int n_groups, int splits) {
-  typedef typename Elem<T>::Frag Frag;
-  constexpr int EPF = Elem<T>::kPerFrag;
-  constexpr int XROW = TW_MERGED_STEPS * 64 + 16;        // bytes per row in LDS, padded
-  __shared__ __attribute__((aligned(16))) char xm[16 * XROW];
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int group = blockIdx.x % n_groups, split = blockIdx.x / n_groups;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = group * 64 + wave * 16;
-
-  const int chunks = K / EPF;
-  const int steps = (chunks + 3) / 4;
-  const int steps_per_split = (steps + splits - 1) / splits;
-  const int step_begin = split * steps_per_split;
-  const int step_end = min(steps, step_begin + steps_per_split);
-  const int n_stages = step_end > step_begin ? (step_end - step_begin + U - 1) / U : 0;
-
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  const T* w_row = W + ((size_t)min(n0 / 16, (N + 15) / 16 - 1) * ldw * 64 + lane) * EPF;
-  Frag wf[2][U];
-  auto load_w = [&](const int buf, int s0) {             // clamped, never predicated (the layout is zero padded)
-#pragma unroll
-    for (int u = 0; u < U; ++u) wf[buf][u] = tw_load_frag_stream(w_row + (size_t)min(s0 + u, steps - 1) * 64 * EPF);
-  };
-  if (n_stages > 0) load_w(0, step_begin);
-  if (n_stages > 1) load_w(1, step_begin + U);
-
-  // ---- this workgroup's K range of the merged attention output, into LDS ---------------------------
-  const int k_begin = step_begin * 4 * EPF;
-  const int k_end = min(step_end * 4 * EPF, K);
-  const int quads = n_stages * U * EPF;                  // groups of 4 elements per row (zeros from k_end on)
-  for (int item = tid; item < 16 * quads; item += 256) {
-    const int row = item / quads, e = (item - row * quads) * 4, k = k_begin + e;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (row < M && k < k_end) {
-      const int head = k / head_dim, d = k - head * head_dim;
-      const size_t base = ((size_t)row * heads + head) * att_splits;
-      const float* ml = part_ml + base * 2;
-      const float* po = part_o + base * head_dim + d;
-      float m = -INFINITY;
-      for (int s = 0; s < att_splits; ++s) m = fmaxf(m, ml[2 * s]);
-      const float m_use = m == -INFINITY ? 0.f : m;
-      float l = 0.f;
-      f32x4 total = {0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; s0 < att_splits; s0 += 8) {       // eight splits' loads in flight, added in split order
-        f32x4 p[8];
-        float ms[8], ls[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int s = min(s0 + i, att_splits - 1);
-          p[i] = *reinterpret_cast<const f32x4*>(po + (size_t)s * head_dim);
-          ms[i] = ml[2 * s];
-          ls[i] = ml[2 * s + 1];
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (s0 + i < att_splits) {
-            const float w = expf(ms[i] - m_use);
-            l += ls[i] * w;
-            total = total + p[i] * w;
-          }
-      }
-      if (l > 0.f) v = f32x4{total[0] / l, total[1] / l, total[2] / l, total[3] / l};
-    }
-    T packed[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) packed[i] = tw_from_float<T>(v[i]);
-    char* dst = xm + row * XROW + e * sizeof(T);
-    if (sizeof(T) == 2)
-      *reinterpret_cast<uint64_t*>(dst) = *reinterpret_cast<const uint64_t*>(packed);
-    else
-      *reinterpret_cast<f32x4*>(dst) = *reinterpret_cast<const f32x4*>(packed);
-  }
-  __syncthreads();
-
-  auto multiply = [&](const int buf, int stage) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const Frag xf = *reinterpret_cast<const Frag*>(xm + r * XROW + ((stage * U + u) * 4 + g) * 16);
-      tw_mma16(acc, wf[buf][u], xf);
-    }
-  };
-  for (int i = 0; i < n_stages; i += 2) {
-    multiply(0, i);
-    if (i + 2 < n_stages) load_w(0, step_begin + (i + 2) * U);
-    if (i + 1 < n_stages) {
-      multiply(1, i + 1);
-      if (i + 3 < n_stages) load_w(1, step_begin + (i + 3) * U);
-    }
-  }
-  // acc[j] = sum_k W[n0 + 4g + j][k] * A[r][k]
-  if (r >= M) return;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int col = n0 + 4 * g + j;
-    if (col < N) partial[((size_t)split * M + r) * N + col] = acc[j];
-  }
-}
-
-// =====================================================================================
 // Generic kernel: any K. One thread per output element, float32 accumulation.
 // =====================================================================================
 template <typename T>
@@ -549,40 +432,6 @@ static int partials_layout(int shuffled, const T* A, long lda, const T* W, long 
   if (shuffled)
     return launch_skinny_lds_m<T, float, true, true, false>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
   return launch_skinny_lds_m<T, float, true, false, false>(A, lda, W, ldw, nullptr, nullptr, 0, (float*)nullptr, N, partial, partial_bytes, M, N, K, stream);
-}
-
-// Can tw_linear_partials_merged take this shape? (at most 16 rows, a shuffled weight, heads whose size is a
-// multiple of 4, and K ranges short enough for a workgroup's LDS)
-extern "C" int tw_linear_merged_ok(int dtype, int M, int N, int K, int head_dim) {
-  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
-  if (M < 1 || M > 16 || N < 1 || K < 1 || K % epf || head_dim < 4 || head_dim % 4 || K % head_dim) return 0;
-  const int splits = skinny_lds_splits(N, K, epf);
-  const int steps = tw_div_up(K / epf, 4), per_split = tw_div_up(steps, splits);
-  return tw_div_up(per_split, 8) * 8 <= TW_MERGED_STEPS ? 1 : 0;
-}
-
-// tw_linear_partials with A given as decode attention's split-KV partial results (the workspace
-// tw_attn_decode leaves when it is called without an output): part_o [M][heads][att_splits][head_dim],
-// part_ml [M][heads][att_splits][2], K = heads * head_dim. W must be in the shuffled layout.
-extern "C" int tw_linear_partials_merged(int dtype, const float* part_o, const float* part_ml, int heads,
-                                         int head_dim, int att_splits, const void* W, long ldw, float* partial,
-                                         long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  TW_REQUIRE(part_o != nullptr && part_ml != nullptr && att_splits >= 1 && att_splits <= 64);
-  TW_REQUIRE(heads > 0 && (long)heads * head_dim == K && tw_linear_merged_ok(dtype, M, N, K, head_dim));
-  TW_REQUIRE((uintptr_t)part_o % 16 == 0 && (uintptr_t)W % 16 == 0 && weight_layout_ok(dtype, 1, ldw, K));
-  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
-  const int splits = skinny_lds_splits(N, K, epf);
-  TW_REQUIRE(partial != nullptr && partial_bytes >= (long)splits * M * N * 4);
-  const int groups = tw_div_up(N, 64);
-  if (dtype == TW_DTYPE_F32)
-    gemm_skinny_merged_kernel<float, 8><<<groups * splits, 256, 0, stream>>>(
-        part_o, part_ml, heads, head_dim, att_splits, (const float*)W, ldw, partial, M, N, K, groups, splits);
-  else if (dtype == TW_DTYPE_BF16)
-    gemm_skinny_merged_kernel<bf16_t, 8><<<groups * splits, 256, 0, stream>>>(
-        part_o, part_ml, heads, head_dim, att_splits, (const bf16_t*)W, ldw, partial, M, N, K, groups, splits);
-  else
-    return TW_ERR_BAD_ARGUMENT;
-  return TW_LAUNCH_RESULT();
 }
 
 // partial[split][M][N] (float32) = A[:, K range of split] W[:, same]^T for every split; the caller's

@@ -26,8 +26,6 @@ _SIGNATURES = {
     "tw_linear_workspace_bytes": (L, [I, I, I, I]),
     "tw_linear_partial_splits": (I, [I, I, I]),
     "tw_linear_partials": (I, [I, P, L, P, L, I, P, L, I, I, I, P]),
-    "tw_linear_merged_ok": (I, [I, I, I, I, I]),
-    "tw_linear_partials_merged": (I, [I, P, P, I, I, I, P, L, P, L, I, I, I, P]),
     "tw_linear_glu": (I, [I, P, L, P, L, I, P, P, L, I, I, I, I, P]),
     "tw_linear": (I, [I, I, P, L, P, L, I, P, P, L, P, L, P, L, I, I, I, I, P]),
     "tw_attn_decode_splits": (I, [I, I, I, I]),

@@ -244,39 +244,6 @@ def linear_partials(x, weight, partial):
     return partial
 
 
-def linear_merged_ok(dtype, m, n, k, head_dim):
-    """Can `linear_partials_merged` take m rows of an [n, k] weight over heads of head_dim?"""
-    return bool(library().tw_linear_merged_ok(dtype_id(dtype), int(m), int(n), int(k), int(head_dim)))
-
-
-def attn_decode_partials(workspace, n_seqs, q_heads, head_dim, splits):
-    """(part_o [n_seqs, q_heads, splits, head_dim], part_ml [n_seqs, q_heads, splits, 2]): the views of what
-    `attn_decode(..., out=None, splits=splits, workspace=workspace)` leaves in its workspace."""
-    n_o = n_seqs * q_heads * splits * head_dim
-    return (workspace[:n_o].view(n_seqs, q_heads, splits, head_dim),
-            workspace[n_o:n_o + n_seqs * q_heads * splits * 2].view(n_seqs, q_heads, splits, 2))
-
-
-def linear_partials_merged(part_o, part_ml, weight, partial):
-    """`linear_partials` whose input rows are decode attention's split-KV partial results, merged on the way
-    (row r, head h: sum_s w_s part_o[r, h, s] / sum_s w_s l_s with w_s = exp(m_s - max m), (m, l) = part_ml[r, h, s]),
-    rounded to the weight's type as the separate merge kernel would. At most 16 rows; a ShuffledWeight."""
-    _need(isinstance(weight, ShuffledWeight), "linear_partials_merged takes a shuffled weight")
-    m, heads, att_splits, head_dim = part_o.shape
-    _need(part_o.is_contiguous() and part_ml.is_contiguous() and tuple(part_ml.shape) == (m, heads, att_splits, 2),
-          "attention partial results must be contiguous [rows, heads, splits, head_dim] and [rows, heads, splits, 2]")
-    n, k = weight.n, weight.k
-    _need(k == heads * head_dim and linear_merged_ok(weight.dtype, m, n, k, head_dim),
-          "linear_partials_merged does not take this shape")
-    splits = linear_partial_splits(weight.dtype, n, k)
-    _need(partial.is_contiguous() and tuple(partial.shape) == (splits, m, n), f"partial must be [{splits}, {m}, {n}]")
-    check(library().tw_linear_partials_merged(dtype_id(weight.dtype), _dev(part_o, torch.float32, "part_o"),
-                                              _dev(part_ml, torch.float32, "part_ml"), heads, head_dim, att_splits,
-                                              _dev(weight.data), weight.k_steps, _dev(partial, torch.float32, "partial"),
-                                              partial.numel() * 4, m, n, k, _stream()), "linear_partials_merged")
-    return partial
-
-
 def interleave_glu_rows(gate, up):
     """[2n, k] with the rows of gate and up [n, k] alternating in blocks of 16 (n a multiple of 16).
 
@@ -348,11 +315,10 @@ def attn_decode_workspace_floats(n_seqs, q_heads, head_dim, splits):
 
 
 def _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim):
-    """OUT may be None (decode attention that keeps its partial results)."""
     nq, wq, ldq = _rows(q, "q")
-    no, wo, ldo = _rows(out, "out") if out is not None else (nq, q_heads * head_dim, q_heads * head_dim)
+    no, wo, ldo = _rows(out, "out")
     _need(wq >= q_heads * head_dim and wo == q_heads * head_dim and no == nq, "attention q/out shapes do not agree")
-    _need((out is None or out.dtype == q.dtype) and q.dtype == keys.dtype == values.dtype, "attention operand types differ")
+    _need(out.dtype == q.dtype == keys.dtype == values.dtype, "attention operand types differ")
     _need(keys.dim() == 4 and keys.is_contiguous() and values.is_contiguous() and values.numel() == keys.numel(),
           "keys must be contiguous [pages, kv_heads, page_size, head_dim] and values the same size")
     _need(keys.shape[1] == kv_heads and keys.shape[3] == head_dim, "cache shape does not match the head sizes")
@@ -370,11 +336,7 @@ def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out
 
     generic=True forces the kernel that takes every type and page size (bfloat16 with
     pages of a multiple of 8 keys otherwise runs a faster kernel of its own).
-    out=None (splits > 1 only): the partial results of the splits are left in the workspace, unmerged
-    (see `attn_decode_partials`).
     """
-    keep_partials = out is None
-    _need(not keep_partials or splits > 1, "decode attention without an output needs splits > 1")
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
     ws_ptr, ws_floats = None, 0
@@ -384,8 +346,7 @@ def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out
     check(library().tw_attn_decode(dtype_id(q.dtype), _dev(q), ldq, _dev(keys), _dev(values),
                                    _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
                                    _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
-                                   seq0, n_seqs, None if keep_partials else _dev(out), ldo, ws_ptr, ws_floats,
-                                   q_heads, kv_heads, head_dim,
+                                   seq0, n_seqs, _dev(out), ldo, ws_ptr, ws_floats, q_heads, kv_heads, head_dim,
                                    keys.shape[2], int(window or 0), float(scale), int(splits), 1 if generic else 0,
                                    _stream()),
           "attn_decode")

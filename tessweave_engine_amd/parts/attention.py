@@ -77,7 +77,6 @@ class GroupedQueryAttention(Mixer):
                               self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache, adjacent=adjacent)
         out = ctx.scratch("attn.out", (n, self.q_heads * self.head_dim))
         window = self.window or 0
-        merged = None           # decode attention's partial results, if the output projection merges them itself
         if ctx.n_decode:
             # A captured step is replayed for other lengths: its split count follows the step's length
             # class (the kernel itself cuts each sequence's own keys into that many ranges).
@@ -92,15 +91,9 @@ class GroupedQueryAttention(Mixer):
                                                           min(ctx.kv_capacity, window) if window else ctx.kv_capacity))
                 floats = ops.attn_decode_workspace_floats(ctx.n_decode, self.q_heads, self.head_dim, most)
                 ws = ctx.workspace.get("attn.split", (floats,), torch.float32)
-            # A step of a few single tokens and nothing else: the merge of the splits is left to the output
-            # projection, whose workgroups each merge their own K range (one kernel and its launch fewer).
-            keep = (splits > 1 and n == ctx.n_decode and ctx.defer_sums and not self.o.biases
-                    and self.o.mergeable(n, self.head_dim))
-            ops.attn_decode(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode,
-                            None if keep else out, self.q_heads, self.kv_heads, self.head_dim, self.scale,
-                            window=window, splits=splits, workspace=ws)
-            if keep:
-                merged = ops.attn_decode_partials(ws, n, self.q_heads, self.head_dim, splits)
+            ops.attn_decode(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode, out,
+                            self.q_heads, self.kv_heads, self.head_dim, self.scale, window=window,
+                            splits=splits, workspace=ws)
         if ctx.n_seqs > ctx.n_decode:
             # long key ranges are cut into chunks for separate workgroups when there are few tiles of rows
             longest = min(ctx.max_kv_len, window + ctx.max_q_len) if window else ctx.max_kv_len
@@ -112,8 +105,6 @@ class GroupedQueryAttention(Mixer):
             ops.attn_prefill(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode,
                              ctx.n_seqs - ctx.n_decode, ctx.max_q_len, out, self.q_heads, self.kv_heads,
                              self.head_dim, self.scale, window=window, split=split, workspace=ws)
-        if merged is not None:
-            return self.o.forward_partials_merged(ctx, *merged, "o")
         if ctx.defer_sums and not self.o.biases and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # the next norm adds them into x
         self.o.forward(ctx, out, x, residual=x)

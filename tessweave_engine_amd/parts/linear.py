@@ -140,24 +140,6 @@ class Linear(Part):
             self._ws_floats["splits"] = ops.linear_partial_splits(w.dtype, w.shape[0], w.shape[1])
         return self._ws_floats["splits"] > 0
 
-    def mergeable(self, n_rows, head_dim):
-        """Can `forward_partials_merged` run for N_ROWS rows of decode attention's partial results?"""
-        if not self.deferrable(n_rows) or not isinstance(self.weights[0], ops.ShuffledWeight):
-            return False
-        key = ("merged", min(n_rows, 16) == n_rows, head_dim)
-        if key not in self._ws_floats:
-            w = self.weights[0]
-            self._ws_floats[key] = ops.linear_merged_ok(w.dtype, n_rows, w.shape[0], w.shape[1], head_dim)
-        return self._ws_floats[key]
-
-    def forward_partials_merged(self, ctx, part_o, part_ml, tag):
-        """`forward_partials` of decode attention's output, given as its unmerged split-KV partial results."""
-        w = self.weights[0]
-        splits, n = self._ws_floats["splits"], part_o.shape[0]
-        buf = ctx.workspace.get("linear.partial." + tag, (splits, 64, w.shape[0]), torch.float32)
-        partial = buf.view(-1)[:splits * n * w.shape[0]].view(splits, n, w.shape[0])
-        return ops.linear_partials_merged(part_o, part_ml, w, partial)
-
     def forward_partials(self, ctx, x, tag):
         """float32 [splits, n, out] partial sums of x @ W.T (bias NOT added); see ops.linear_partials."""
         w = self.weights[0]

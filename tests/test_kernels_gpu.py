@@ -288,50 +288,6 @@ def test_linear_partials(ops, device, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,heads,head_dim,n,att_splits", [(1, 28, 128, 3584, 16), (8, 28, 128, 3584, 8), (16, 4, 16, 64, 2),
-                                                          (3, 6, 32, 200, 5), (5, 40, 128, 5120, 33), (2, 2, 256, 100, 64),
-                                                          (7, 3, 48, 389, 3)])
-def test_linear_partials_merged_reads_the_attention_splits_itself(ops, device, dtype, m, heads, head_dim, n, att_splits):
-    """The output projection of a decode step merging decode attention's split-KV partial results on the way:
-    against the merge written out in float64 and against the two separate kernels."""
-    k = heads * head_dim
-    g = torch.Generator().manual_seed(m * 1000 + att_splits)
-    part_o = torch.randn(m, heads, att_splits, head_dim, generator=g)
-    part_ml = torch.stack([torch.randn(m, heads, att_splits, generator=g) * 3,                # running maxima
-                           torch.rand(m, heads, att_splits, generator=g) * 5 + 0.1], -1)     # sums
-    part_ml[0, 0, 1:, 0], part_ml[0, 0, 1:, 1] = float("-inf"), 0.0                           # empty splits: (-inf, 0)
-    part_o[0, 0, 1:] = 0.0
-    if m > 1:
-        part_ml[1, heads - 1, :, 0], part_ml[1, heads - 1, :, 1] = float("-inf"), 0.0         # a row with no key at all
-    w = rand((n, k), dtype, device, 0.05, seed=2)
-    assert not ops.linear_merged_ok(dtype, 17, n, k, head_dim)
-    if not ops.linear_merged_ok(dtype, m, n, k, head_dim):
-        # a K range longer than a workgroup's LDS holds (float32 at this width): refused, and the caller merges first
-        assert (m, k, dtype) == (5, 5120, torch.float32)
-        with pytest.raises(ValueError, match="does not take this shape"):
-            ops.linear_partials_merged(part_o.to(device), part_ml.to(device), ops.shuffle_weight(w),
-                                       torch.empty(ops.linear_partial_splits(dtype, n, k), m, n, device=device))
-        return
-    mx = part_ml[..., 0].max(-1, keepdim=True).values
-    wts = torch.exp(part_ml[..., 0].double() - torch.where(torch.isinf(mx), torch.zeros_like(mx), mx).double())
-    l = (wts * part_ml[..., 1].double()).sum(-1)
-    total = (wts[..., None] * part_o.double()).sum(2)
-    merged = torch.where(l[..., None] > 0, total / l[..., None].clamp_min(1e-300), torch.zeros_like(total))
-    a = merged.reshape(m, k).to(dtype)                                         # what the merge kernel would store
-    want = a.double() @ w.double().cpu().T
-    splits = ops.linear_partial_splits(dtype, n, k)
-    partial = torch.full((splits, m, n), float("nan"), device=device)
-    ops.linear_partials_merged(part_o.to(device), part_ml.to(device), ops.shuffle_weight(w), partial)
-    scale = math.sqrt(k) * 0.05
-    t = dict(atol=3e-5 * scale, rtol=1e-5) if dtype == torch.float32 else dict(atol=1e-2 * scale, rtol=1e-2)
-    torch.testing.assert_close(partial.double().sum(0).cpu(), want, **t)
-    # the two kernels it replaces: the merge into a matrix of the weight's type, then the projection of that
-    two = torch.full((splits, m, n), float("nan"), device=device)
-    ops.linear_partials(a.to(device), ops.shuffle_weight(w), two)
-    torch.testing.assert_close(partial.sum(0), two.sum(0), **t)
-
-
-@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 64), (8, 208, 320), (17, 48, 1032), (64, 1040, 256), (65, 80, 64),
                                        (200, 400, 320), (130, 16, 101), (520, 272, 200), (520, 272, 320),
                                        (8, 9472, 64), (3, 9488, 96)])     # so many columns that few rows run in workgroups of two waves
