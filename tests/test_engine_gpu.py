@@ -246,6 +246,31 @@ def test_prefix_pages_are_reused_on_the_gpu(tiny):
     assert len(e.cache.pools[0].free) == e.cache.pools[0].capacity
 
 
+def test_requests_that_run_together_share_the_blocks_of_a_common_prompt(tiny):
+    """The full blocks of a prompt enter the prefix index as soon as their step has been issued: a request
+    that arrives while the first one is still in its prompt or decoding takes them (its own step runs later
+    on the same stream), in both ways of reading tokens, and generates what the plain implementation does."""
+    shared = prompts_for(tiny, [64], seed=8)[0]
+    p1, p2, p3 = shared + [3, 4, 5], shared + [9, 1], shared[:32] + [7, 7, 7]
+    want = [plain.greedy(tiny["config"], tiny["weights"], p, 8) for p in (p1, p2, p3)]
+    for look in (True, False):
+        e = engine(tiny, no_prefix_cache=False, no_lookahead=not look, prefill_chunk=32)
+        a = e.submit(p1, 8, ignore_eos=True)
+        e.step()                                         # a's first 32 prompt tokens are on the device
+        b = e.submit(p2, 8, ignore_eos=True)
+        e.step()                                         # b is admitted: it shares what a has issued so far
+        e.step()
+        c = e.submit(p3, 8, ignore_eos=True)
+        e.drain()
+        e.flush()
+        assert a.cached == 0 and b.cached == 32 and c.cached == 32, (a.cached, b.cached, c.cached)
+        assert [a.output, b.output, c.output] == want
+        assert e.stats()["prefix_hit_tokens"] == 64
+        e.close()
+        e.cache.check()
+        assert len(e.cache.pools[0].free) == e.cache.pools[0].capacity
+
+
 # ---- each part alone --------------------------------------------------------------------------------
 class PartHarness:
     """A cache, a step context and the GPU stream for running single parts on given sequences."""

@@ -618,3 +618,18 @@ def test_a_head_of_queue_that_does_not_fit_earns_no_hits_and_costs_no_index_entr
     assert again.output == first.output and long_.status == "length"
     e.close()
     e.cache.check()
+
+
+def test_prompt_blocks_are_shared_early_under_lookahead_too():
+    e, s = make_lookahead(max_active=2, prefill_chunk=8, max_step_tokens=8)
+    prompt = [2, 3, 4, 5, 6, 7, 8, 9, 10]
+    a = e.submit(prompt, 6)
+    e.step()
+    b = e.submit(prompt, 6)
+    e.step()
+    assert b.status == "active" and b.cached == 8 and a.status == "active"
+    drain(e)
+    assert a.output == b.output == expected(prompt, 6)
+    e.close()
+    e.cache.check()
+    assert len(e.cache.pools[0].free) == 32
