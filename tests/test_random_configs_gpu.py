@@ -3,7 +3,9 @@
 Each seed draws every size and option (head sizes in steps of 16 up to 256, odd counts of heads and
 groups, feed-forward widths and vocabularies that are multiples of nothing, number of layers, eps, theta,
 tied or untied head, page sizes from 4 to 64) and replays four requests whole, with the last 32 tokens one
-by one, and mixed with few pages, in both precisions, with the bars of test_replay_gpu. Head sizes that
+by one, and mixed with few pages, in both precisions: bfloat16 with the bar of test_replay_gpu, float32 with
+its calibrated bar (against the plain implementation in float64, at most four times the plain float32's own
+error: widths from 16 to 2,064 round very differently). Head sizes that
 are even but no multiple of 16 (18, 24, 72, 2, 250) replay the same way; above 256 the model is refused.
 """
 import random
@@ -48,7 +50,9 @@ def replay_three_ways(cfg, page, lengths, seed, tmp_path):
     g = torch.Generator().manual_seed(seed)
     requests = {f"r{i}": torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for i, n in enumerate(lengths)}
     want = {rid: plain.forward(config, weights, toks).numpy() for rid, toks in requests.items()}
-    model = dict(name=f"seed {seed}: {cfg}", folder=folder, page=page, cfg=cfg, requests=requests, want=want)
+    weights64 = {k: v.double() for k, v in weights.items()}
+    exact = {rid: plain.forward(config, weights64, toks).numpy() for rid, toks in requests.items()}    # summed in float64
+    model = dict(name=f"seed {seed}: {cfg}", folder=folder, page=page, cfg=cfg, requests=requests, want=want, exact=exact)
     biggest = max(replay_tests.round64(len(t)) for t in requests.values())
     for dtype in ("float32", "bfloat16"):
         steps, starts = replay_tests.sequential(model, lambda t: [t])

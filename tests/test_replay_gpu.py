@@ -63,7 +63,35 @@ def run_trace(tiny, dtype, steps, max_tokens, out_dir, extra=()):
 
 
 def compare(tiny, dtype, steps, got, starts):
-    """STARTS[(step, request id)] = position of the entry's first token."""
+    """STARTS[(step, request id)] = position of the entry's first token.
+
+    A model that also brings "exact" (the plain implementation's logits in float64) gets a calibrated float32
+    bar instead of the fixed one: the absolute part is four times what the plain implementation in float32
+    ("want") is off from float64 at worst, plus 1e-6; the relative part is the reference's own 2e-5
+    (tests/test_engine.py:65). Sums over a few thousand terms round differently in every order; how much
+    depends on the widths, which random configurations vary a hundredfold, and a tied head gives a token's
+    own logit a size of tens, where a chain of 32-bit additions is off by several units in the last place.
+    """
+    if dtype == "float32" and "exact" in tiny:
+        rows = []
+        for s in steps:
+            row = 0
+            for e in s["entries"]:
+                base = starts[(s["step"], e["id"])]
+                for w in e["want"]:
+                    rows.append((e["id"], base + w, s["step"], got[s["step"]][row]))
+                    row += 1
+        worst_plain = max(float(np.abs(tiny["want"][rid][pos] - tiny["exact"][rid][pos]).max()) for rid, pos, _, _ in rows)
+        atol = 4 * worst_plain + 1e-6
+        worst_engine = 0.0
+        for rid, pos, step, have in rows:
+            exact = tiny["exact"][rid][pos]
+            err = np.abs(have - exact)
+            worst_engine = max(worst_engine, float(err.max()))
+            assert (err <= atol + 2e-5 * np.abs(exact)).all(), (
+                f"{tiny['name']} float32: request {rid} position {pos} (step {step}): off from float64 by "
+                f"{err.max():.3e}; plain float32 is off by at most {worst_plain:.3e}, largest logit {np.abs(exact).max():.3f}")
+        return worst_engine
     worst = 0.0
     for s in steps:
         row = 0
