@@ -5,7 +5,8 @@ import pytest
 import torch
 from safetensors.torch import save_file
 
-from tessweave_engine_amd.config import (ConfigError, EngineConfig, Qwen2Config, build_model, config_from_dict,
+from tessweave_engine_amd.models.qwen2 import Qwen2Config
+from tessweave_engine_amd.config import (ConfigError, EngineConfig, build_model, config_from_dict,
                                          read_model_config, register_architecture, registered_architectures,
                                          unregister_architecture)
 from tessweave_engine_amd.weights import (WeightError, random_tensors, read_tensors, write_model_folder)
