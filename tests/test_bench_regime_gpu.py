@@ -271,3 +271,52 @@ def test_decoding_across_a_length_class_takes_a_second_graph_and_changes_nothing
     assert sorted(stepper._graphs) == [(2, 512), (2, 1024)]
     assert stepper.graph_replays == 30 - 2                 # the first step of each class runs eagerly, the next is captured
     stepper.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_request_of_33000_tokens_through_the_engine(long_model, dtype, device):
+    """Positions up to 33,000 (rotation angles of thousands of turns), block tables two thousand pages wide,
+    prompt portions of 2,048 tokens behind a long history (their keys are cut into chunks for separate
+    workgroups), then single tokens over 33,000 keys in as many ranges as the launcher picks. The plain
+    implementation runs on the device for this (a 33,000 x 33,000 score matrix per head)."""
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.weights import load_model
+    page, vocab = long_model["page"], long_model["cfg"]["vocab_size"]
+    n, n_decode = 33000, 4
+    import json
+    cfg = dict(long_model["cfg"], max_position_embeddings=40000)
+    (long_model["folder"] / "config.json").write_text(json.dumps(cfg))
+    g = torch.Generator().manual_seed(33)
+    tokens = torch.randint(0, vocab, (n + n_decode,), generator=g).tolist()
+    rows = [0, 2047, 2048, 20479, 20480, n - 1] + list(range(n, n + n_decode))
+    w = {k: t.to(device) for k, t in long_model["weights"].items()}
+    with torch.device(device):
+        want = plain.forward(long_model["config"], w, tokens)[rows].cpu()
+    del w
+    torch.cuda.empty_cache()
+    model = load_model(long_model["folder"], dtype=dtype, device="cuda:0")
+    cache = CacheManager(model.cache_layout(), page, (n + n_decode) // page + 2, 1, dtype=dtype, device=model.device,
+                         prefix_cache=False, max_request_tokens=n + n_decode + page)
+    stepper = Stepper(model, cache, max_step_tokens=2048, max_step_seqs=1)
+    seq = cache.open("far")
+    got = {}
+    for a in range(0, n, 2048):
+        b = min(n, a + 2048)
+        wanted = [r - a for r in rows if a <= r < b]
+        out = stepper.step([StepEntry(seq, tokens[a:b], wanted)]).cpu()
+        for j, r in enumerate(wanted):
+            got[r + a] = out[j].clone()
+    for p in range(n, n + n_decode):
+        got[p] = stepper.step([StepEntry(seq, [tokens[p]], [0])]).cpu()[0].clone()
+    worst = 0.0
+    for j, r in enumerate(rows):
+        err = float((got[r] - want[j]).abs().max())
+        worst = max(worst, err)
+        if dtype == "float32":
+            assert torch.allclose(got[r], want[j], atol=5e-6, rtol=2e-5), (r, err)
+        else:
+            assert err <= 0.02 * float(want[j].abs().max()), (r, err)
+    print(f"33,000 tokens, {dtype}: worst difference {worst:.3e}")
+    cache.close(seq)
+    stepper.close()

@@ -134,6 +134,20 @@ def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, p
     torch.testing.assert_close(qkv3[:, :q_heads * head_dim], ref[:, :q_heads * head_dim], atol=0, rtol=0)
 
 
+@pytest.mark.parametrize("theta", [1e4, 1e6])
+def test_rope_tables_at_far_positions(ops, device, theta):
+    """cos and sin of float32(position) * inv_freq at positions up to 131,071: the angle is formed in float32 as
+    the reference forms it (flow_engine/model.py:28-29), and the fast pairs turn tens of thousands of times."""
+    positions = torch.tensor([0, 1, 4095, 4096, 31999, 32767, 32768, 100003, 131071], dtype=torch.int32)
+    inv = theta ** (-torch.arange(0, 128, 2, dtype=torch.float32) / 128)
+    cos = torch.empty(len(positions), 64, device=device)
+    sin = torch.empty_like(cos)
+    ops.rope_table(positions.to(device), inv.to(device), cos, sin)
+    angle = positions.float()[:, None] * inv[None, :]                       # float32, as the kernel
+    torch.testing.assert_close(cos.cpu(), angle.double().cos().float(), atol=3e-7, rtol=0)
+    torch.testing.assert_close(sin.cpu(), angle.double().sin().float(), atol=3e-7, rtol=0)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("head_dim,rot", [(16, 16), (32, 12), (48, 48)])
 def test_rope_with_adjacent_pairs(ops, device, dtype, head_dim, rot):
