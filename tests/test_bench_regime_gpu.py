@@ -101,7 +101,7 @@ def test_decode_attention_at_the_benchmarks_lengths_with_the_launchers_own_range
     assert hits >= 20
 
 
-# ---- the engine opened for thousands of tokens, a decode batch of 48 from graphs ----------------------------
+# ---- the engine opened for thousands of tokens, decode batches of 40 and 64 from graphs ----------------------------
 @pytest.fixture(scope="module")
 def long_model(tmp_path_factory, device):
     folder = tmp_path_factory.mktemp("longA")
@@ -114,15 +114,17 @@ def long_model(tmp_path_factory, device):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_decode_batch_of_48_requests_short_and_long_from_graphs(long_model, dtype):
-    """An engine opened for 4,224 tokens a request: the captured decode step sizes its key ranges by that, and
-    the batch holds requests of 3 to 4,100 tokens. Six decode steps (one eager, one captured, four replayed) of
-    48 requests, every logits row against the plain implementation."""
+@pytest.mark.parametrize("n_req", [40, 64])
+def test_a_decode_batch_of_40_and_of_64_requests_short_and_long_from_graphs(long_model, dtype, n_req):
+    """An engine opened for 4,224 tokens a request: the captured decode step sizes its key ranges by the
+    length class, and the batch holds requests of 3 to 4,100 tokens. Six decode steps (one eager, one captured,
+    four replayed) of 40 requests (the streaming matrix kernel's 48-row form) and of 64 (its 64-row form, the
+    benchmark's), every logits row against the plain implementation."""
     from tessweave_engine_amd.cache import CacheManager
     from tessweave_engine_amd.engine import StepEntry, Stepper
     from tessweave_engine_amd.weights import load_model
     page, vocab = long_model["page"], long_model["cfg"]["vocab_size"]
-    n_req, n_decode, capacity = 48, 6, 4224
+    n_decode, capacity = 6, 4224
     g = torch.Generator().manual_seed(48)
     prompt_lens = [4100, 1500, 3, 700] + torch.randint(1, 200, (n_req - 4,), generator=g).tolist()
     tokens = [torch.randint(0, vocab, (n + n_decode,), generator=g).tolist() for n in prompt_lens]
@@ -156,12 +158,12 @@ def test_a_decode_batch_of_48_requests_short_and_long_from_graphs(long_model, dt
         batch = rest[a:a + 8]
         got = stepper.step([StepEntry(seqs[i], tokens[i][:prompt_lens[i]], [prompt_lens[i] - 1]) for i in batch]).cpu()
         check(got, [(i, prompt_lens[i] - 1) for i in batch])
-    # decode: all 48 in every step
+    # decode: all of them in every step
     for s in range(n_decode):
         got = stepper.step([StepEntry(seqs[i], [tokens[i][prompt_lens[i] + s]], [0]) for i in range(n_req)]).cpu()
         check(got, [(i, prompt_lens[i] + s) for i in range(n_req)])
     assert stepper.graph_replays >= n_decode - 2
-    print(f"48 requests, {dtype}: worst difference {worst:.3e}")
+    print(f"{n_req} requests, {dtype}: worst difference {worst:.3e}")
     for seq in seqs:
         cache.close(seq)
     cache.check()
