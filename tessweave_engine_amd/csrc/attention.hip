@@ -363,12 +363,12 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
       const bf16_t* k_row = keys + ((size_t)page_of(k_pi[tile]) * a.kv_heads + kvh) * head_stride + pb * D + k_off[tile];
 #pragma unroll
       for (int st = 0; st < NSMAX; ++st)
-        L.k[tile][st] = (EXACT || st * 4 + g < chunks) ? tw_load_frag(k_row + st * 32) : Elem<bf16_t>::zero();
+        L.k[tile][st] = (EXACT || st * 4 + g < chunks) ? tw_load_frag_stream(k_row + st * 32) : Elem<bf16_t>::zero();
     }
     const bf16_t* v_base = values + ((size_t)page_of(v_pi) * a.kv_heads + kvh) * head_stride + pb + v_off;
 #pragma unroll
     for (int dt = 0; dt < DTMAX; ++dt)
-      if (EXACT || dt < dts) L.v[dt] = tw_load_frag(v_base + (size_t)(dt * 16) * P);
+      if (EXACT || dt < dts) L.v[dt] = tw_load_frag_stream(v_base + (size_t)(dt * 16) * P);
   };
 
   auto compute_as = [&](int blk, KVBlock<DTMAX>& L, auto edge_tag) {

@@ -27,12 +27,6 @@ __device__ __forceinline__ size_t tw_shuffled_chunk(int n, int c, int k_steps, i
   return ((size_t)((size_t)(n >> 4) * k_steps + (c >> 2)) * 64 + (c & 3) * 16 + (n & 15)) * epf;
 }
 
-template <typename T>
-__device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p) {
-  // weights are read once per step: do not keep them in the caches
-  return __builtin_nontemporal_load(reinterpret_cast<const typename Elem<T>::Frag*>(p));
-}
-
 // =====================================================================================
 // Skinny kernel (M <= 16*MT rows), workgroup-cooperative. The WAVES (4, or 2) waves of a workgroup own
 // neighbouring tiles of 16 output columns and the SAME K range. Per stage of U

@@ -62,6 +62,13 @@ __device__ __forceinline__ typename Elem<T>::Frag tw_load_frag(const T* p) {
   return *reinterpret_cast<const typename Elem<T>::Frag*>(p);
 }
 
+// For data that a kernel reads once (weights of a decode step, the cache in decode attention): the
+// caches are told not to keep it.
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::Frag tw_load_frag_stream(const T* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const typename Elem<T>::Frag*>(p));
+}
+
 // ---- MFMA: 16x16 tiles --------------------------------------------------------
 // Lane l = 16*g + r (g = l / 16, r = l % 16).
 //   A operand: row r of the 16-row tile, the fragment chosen by g.
