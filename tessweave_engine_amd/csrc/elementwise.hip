@@ -148,22 +148,58 @@ __global__ void rmsnorm_vec4_kernel(float* __restrict__ x, const float* __restri
   }
 }
 
-// Many rows, nothing to add: one WAVE per row (4 rows per workgroup), a row of up to 256 * NG elements
-// in registers as up to NG groups of 4, every load issued at once, and no barrier: the sum of squares
-// is a wave reduction. (With one workgroup of 896 threads per row, 2,048 rows of 3,584 took 15 us.)
-template <typename T, int NG>
-__global__ __launch_bounds__(256) void rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                           T* __restrict__ out, int n_rows, int hidden, float eps) {
+// Many rows: one WAVE per row (4 rows per workgroup), a row of up to 256 * NG elements in registers as
+// up to NG groups of 4, every load of a pass issued at once, and no barrier: the sum of squares is a wave
+// reduction. (With one workgroup of 896 threads per row, 2,048 rows of 3,584 took 15 us.) With ADD the
+// row is (sum_s add[s]) + x, added in that order as everywhere, and written back to x.
+template <typename T, int NG, bool ADD>
+__global__ __launch_bounds__(256) void rmsnorm_wave_kernel(float* __restrict__ x, const float* __restrict__ w,
+                                                           T* __restrict__ out, int n_rows, int hidden, float eps,
+                                                           const float* __restrict__ add, int add_splits,
+                                                           size_t add_stride) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= n_rows) return;
-  const float* src = x + (size_t)row * hidden;
+  float* src = x + (size_t)row * hidden;
   f32x4 v[NG];
   float ss = 0.f;
+  if (ADD) {
+    // CH groups at a time (a whole row of up to 4,096 elements, half of a longer one): the row's own
+    // values and one split's sums are in flight together
+    constexpr int CH = NG <= 16 ? NG : 16;
+    const float* p = add + (size_t)row * hidden;
 #pragma unroll
-  for (int i = 0; i < NG; ++i) {
-    const int h = (i * 64 + lane) * 4;
-    v[i] = h < hidden ? *reinterpret_cast<const f32x4*>(src + h) : f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < NG; c += CH) {
+      f32x4 xv[CH], acc[CH];
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        const int h = ((c + j) * 64 + lane) * 4;
+        xv[j] = h < hidden ? *reinterpret_cast<const f32x4*>(src + h) : f32x4{0.f, 0.f, 0.f, 0.f};
+        acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+      for (int s = 0; s < add_splits; ++s) {
+        f32x4 a[CH];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+          const int h = ((c + j) * 64 + lane) * 4;
+          a[j] = h < hidden ? *reinterpret_cast<const f32x4*>(p + s * add_stride + h) : f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < CH; ++j) acc[j] = acc[j] + a[j];
+      }
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        const int h = ((c + j) * 64 + lane) * 4;
+        v[c + j] = acc[j] + xv[j];
+        if (h < hidden) *reinterpret_cast<f32x4*>(src + h) = v[c + j];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const int h = (i * 64 + lane) * 4;
+      v[i] = h < hidden ? *reinterpret_cast<const f32x4*>(src + h) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
   }
 #pragma unroll
   for (int i = 0; i < NG; ++i) ss += ((v[i][0] * v[i][0] + v[i][1] * v[i][1]) + v[i][2] * v[i][2]) + v[i][3] * v[i][3];
@@ -198,12 +234,16 @@ static void launch_rmsnorm_vec4(int groups_per_thread, int n_out, int threads, h
 }
 
 template <typename T>
-static void launch_rmsnorm_wave(int n_out, hipStream_t stream, const float* x, const float* w, T* out, int hidden,
-                                float eps) {
-  if (hidden <= 4096)
-    rmsnorm_wave_kernel<T, 16><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, out, n_out, hidden, eps);
-  else
-    rmsnorm_wave_kernel<T, 32><<<(n_out + 3) / 4, 256, 0, stream>>>(x, w, out, n_out, hidden, eps);
+static void launch_rmsnorm_wave(int n_out, hipStream_t stream, float* x, const float* w, T* out, int hidden,
+                                float eps, const float* add, int add_splits, size_t add_stride) {
+  const int grid = (n_out + 3) / 4;
+  if (hidden <= 4096) {
+    if (add) rmsnorm_wave_kernel<T, 16, true><<<grid, 256, 0, stream>>>(x, w, out, n_out, hidden, eps, add, add_splits, add_stride);
+    else rmsnorm_wave_kernel<T, 16, false><<<grid, 256, 0, stream>>>(x, w, out, n_out, hidden, eps, nullptr, 0, 0);
+  } else {
+    if (add) rmsnorm_wave_kernel<T, 32, true><<<grid, 256, 0, stream>>>(x, w, out, n_out, hidden, eps, add, add_splits, add_stride);
+    else rmsnorm_wave_kernel<T, 32, false><<<grid, 256, 0, stream>>>(x, w, out, n_out, hidden, eps, nullptr, 0, 0);
+  }
 }
 
 extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, const int* rows,
@@ -213,12 +253,13 @@ extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, co
   TW_REQUIRE(add == nullptr || (add_splits > 0 && (rows == nullptr || row_scratch != nullptr)));
   if (n_out == 0) return 0;
   if (out_dtype != TW_DTYPE_F32 && out_dtype != TW_DTYPE_BF16) return TW_ERR_BAD_ARGUMENT;
-  if (add == nullptr && rows == nullptr && n_out >= 256 && hidden % 4 == 0 && hidden <= 8192 &&
-      (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0) {
+  if (rows == nullptr && n_out >= 256 && hidden % 4 == 0 && hidden <= 8192 &&
+      (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+      (add == nullptr || ((uintptr_t)add % 16 == 0 && add_stride % 4 == 0))) {
     if (out_dtype == TW_DTYPE_F32)
-      launch_rmsnorm_wave<float>(n_out, stream, x, w, (float*)out, hidden, eps);
+      launch_rmsnorm_wave<float>(n_out, stream, x, w, (float*)out, hidden, eps, add, add_splits, (size_t)add_stride);
     else
-      launch_rmsnorm_wave<bf16_t>(n_out, stream, x, w, (bf16_t*)out, hidden, eps);
+      launch_rmsnorm_wave<bf16_t>(n_out, stream, x, w, (bf16_t*)out, hidden, eps, add, add_splits, (size_t)add_stride);
     return TW_LAUNCH_RESULT();
   }
   // rows of up to 16384 elements: one, two or four groups of 4 elements per thread, everything in registers

@@ -420,6 +420,16 @@ extern "C" int tw_linear_partial_splits(int dtype, int N, int K) {
   return skinny_lds_splits(N, K, epf);
 }
 
+// The same for M rows: up to 64 rows the streaming kernel's ranges; above, those of the tiled kernels
+// (0 where they would not split K: the product with its epilogue is then the better call).
+extern "C" int tw_linear_partial_splits_rows(int dtype, int shuffled, int M, int N, int K) {
+  if (M <= 64) return tw_linear_partial_splits(dtype, N, K);
+  const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
+  if (K % epf) return 0;
+  const int splits = tw_tiled_partial_splits(dtype, shuffled, K, M, N, K);
+  return splits > 1 ? splits : 0;
+}
+
 template <typename T>
 static int partials_layout(int shuffled, const T* A, long lda, const T* W, long ldw, float* partial,
                            long partial_bytes, int M, int N, int K, hipStream_t stream) {
@@ -429,13 +439,23 @@ static int partials_layout(int shuffled, const T* A, long lda, const T* W, long 
 }
 
 // partial[split][M][N] (float32) = A[:, K range of split] W[:, same]^T for every split; the caller's
-// next kernel adds the splits up (with bias, residual, norm or rotation as it needs).
+// next kernel adds the splits up (with bias, residual, norm or rotation as it needs). Up to 64 rows the
+// streaming kernel runs, above that the tiled kernels.
 extern "C" int tw_linear_partials(int dtype, const void* A, long lda, const void* W, long ldw, int shuffled,
                                   float* partial, long partial_bytes, int M, int N, int K, hipStream_t stream) {
-  TW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && lda >= K);
+  TW_REQUIRE(M >= 1 && N > 0 && K > 0 && lda >= K);
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
   TW_REQUIRE(K % epf == 0 && lda % epf == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0);
   TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K) && (shuffled || ldw % epf == 0));
+  if (M > 64) {
+    // the caller sized `partial` for the ranges tw_linear_partial_splits_rows named: they must be the ones used
+    const int expect = tw_tiled_partial_splits(dtype, shuffled, lda, M, N, K);
+    TW_REQUIRE(expect >= 1 && partial_bytes == (long)expect * M * N * 4);
+    int used = 0;
+    const int err = tw_tiled_partials(dtype, shuffled, A, lda, W, ldw, partial, partial_bytes, M, N, K, &used, stream);
+    if (err) return err;
+    return used == expect ? 0 : TW_ERR_BAD_ARGUMENT;
+  }
   if (dtype == TW_DTYPE_F32)
     return partials_layout<float>(shuffled, (const float*)A, lda, (const float*)W, ldw, partial, partial_bytes, M, N, K, stream);
   if (dtype == TW_DTYPE_BF16)

@@ -77,5 +77,10 @@ static inline int launch_splitk_reduce(const float* partial, int splits, const f
 int tw_tiled_linear(int dtype, int out_f32, int shuffled, int glu, int shape, const void* A, long lda,
                     const void* W, long ldw, const float* bias, const float* residual, long ldr, void* C,
                     long ldc, float* partial, long partial_bytes, int M, int N, int K, hipStream_t stream);
+// The tiled kernels with the sums of their K ranges left in partial[s][M][N] (no reduction kernel), and
+// the number of ranges they would use (1: none; then partial[0] is the product).
+int tw_tiled_partial_splits(int dtype, int shuffled, long lda, int M, int N, int K);
+int tw_tiled_partials(int dtype, int shuffled, const void* A, long lda, const void* W, long ldw, float* partial,
+                      long partial_bytes, int M, int N, int K, int* splits_used, hipStream_t stream);
 // Bytes of split-K scratch the tiled kernels can use for `rows` rows of an [N, K] weight (0: none).
 long tw_tiled_workspace_bytes(int dtype, int rows, int N, int K);

@@ -502,6 +502,15 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
 // How many K ranges the tiled kernel uses: with fewer tiles than the chip has room for (a prompt
 // portion of a few hundred rows against a square or tall matrix) the k-tiles of a tile are dealt
 // to several workgroups. Depends on the shape only.
+// How a launch may deviate from "compute C": `leave` keeps the float32 sums of the K ranges in `partial`
+// for the caller's next kernel (no reduction kernel; the caller passes C = partial as float32 without
+// bias or residual, so that with a single range the product itself is partial[0]); `dry` launches
+// nothing and only reports, in `splits`, the number of K ranges the launch would use.
+struct TiledMode {
+  bool leave = false, dry = false;
+  int splits = 0;
+};
+
 static int tiled_splits(int M, int N, int K, int epf, int bm, int bn) {
   const long tiles = (long)tw_div_up(M, bm) * tw_div_up(N, bn);
   if (tiles >= 192) return 1;
@@ -517,12 +526,18 @@ static int tiled_splits(int M, int N, int K, int epf, int bm, int bn) {
 template <typename T, typename OutT, int WM, int WN, bool SHUF, bool GLU>
 static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float* bias,
                         const float* residual, long ldr, OutT* C, long ldc, float* partial,
-                        long partial_bytes, int M, int N, int K, int want_splits, hipStream_t stream) {
+                        long partial_bytes, int M, int N, int K, int want_splits, hipStream_t stream,
+                        TiledMode* mode = nullptr) {
   constexpr int BM = 64 * WM, BN = 64 * WN, KCH = 8;
   constexpr int EPF = Elem<T>::kPerFrag;
   const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
   int splits = GLU ? 1 : (want_splits > 0 ? want_splits : tiled_splits(M, N, K, EPF, BM, BN));
+  if (mode && mode->dry) {
+    mode->splits = splits;
+    return 0;
+  }
   if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4 || (uintptr_t)partial % 16 != 0)) splits = 1;
+  if (mode) mode->splits = splits;
   const long n_blocks = (long)tiles_m * tiles_n * splits;
   TW_REQUIRE(n_blocks < (1L << 30));
   // per-tile offsets are 32-bit
@@ -543,7 +558,7 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
   kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m,
                                            (int)n_blocks, splits, partial);
   int err = TW_LAUNCH_RESULT();
-  if (err || splits == 1) return err;
+  if (err || splits == 1 || (mode && mode->leave)) return err;
   return launch_splitk_reduce<OutT>(partial, splits, bias, residual, ldr, C, ldc, M, N, stream);
 }
 
@@ -551,12 +566,17 @@ static int launch_tiled(const T* A, long lda, const T* W, long ldw, const float*
 template <typename OutT, int WM, int WN, bool GLU>
 static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias,
                       const float* residual, long ldr, OutT* C, long ldc, float* partial, long partial_bytes,
-                      int M, int N, int K, int want_splits, hipStream_t stream) {
+                      int M, int N, int K, int want_splits, hipStream_t stream, TiledMode* mode = nullptr) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   TW_REQUIRE(K % 32 == 0 && K >= 32 && lda % 8 == 0);
   const int tiles_m = tw_div_up(M, BM), tiles_n = tw_div_up(N, BN);
   int splits = GLU ? 1 : (want_splits > 0 ? want_splits : tiled_splits(M, N, K, 8, BM, BN));
+  if (mode && mode->dry) {
+    mode->splits = splits;
+    return 0;
+  }
   if (splits > 1 && (partial == nullptr || partial_bytes < (long)splits * M * N * 4 || (uintptr_t)partial % 16 != 0)) splits = 1;
+  if (mode) mode->splits = splits;
   const long n_blocks = (long)tiles_m * tiles_n * splits;
   TW_REQUIRE(n_blocks < (1L << 30));
   const int grid = (int)((n_blocks + 7) / 8 * 8);
@@ -574,7 +594,7 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
   kernel<<<grid, 256, lds_bytes, stream>>>(A, lda, W, ldw, bias, residual, ldr, C, ldc, M, N, K, tiles_m,
                                            (int)n_blocks, splits, partial);
   int err = TW_LAUNCH_RESULT();
-  if (err || splits == 1) return err;
+  if (err || splits == 1 || (mode && mode->leave)) return err;
   return launch_splitk_reduce<OutT>(partial, splits, bias, residual, ldr, C, ldc, M, N, stream);
 }
 
@@ -645,7 +665,7 @@ static TilePlan choose_plan(bool big_ok, bool glu, int M, int N, int K, int epf)
 template <typename T, typename OutT, bool SHUF, bool GLU>
 static int tiled_by_shape(int shape, const T* A, long lda, const T* W, long ldw, const float* bias,
                           const float* residual, long ldr, OutT* C, long ldc, float* partial,
-                          long partial_bytes, int M, int N, int K, hipStream_t stream) {
+                          long partial_bytes, int M, int N, int K, hipStream_t stream, TiledMode* mode = nullptr) {
   constexpr bool BIG = sizeof(T) == 2 && SHUF;
   int splits = 0;                                   // a forced shape keeps the launcher's own rule
   if (shape == 0) {
@@ -656,39 +676,40 @@ static int tiled_by_shape(int shape, const T* A, long lda, const T* W, long ldw,
   if constexpr (BIG) {
     // bfloat16 and shuffled weights: the kernels that copy straight into LDS, if K allows
     if (K % 32 == 0 && K >= 32 && lda % 8 == 0) {
-      if (shape == 4) return launch_dma<OutT, 4, 3, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
+      if (shape == 4) return launch_dma<OutT, 4, 3, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream, mode);
       if constexpr ((TW_DMA_SHAPES & 8) != 0)
-        if (shape == 3) return launch_dma<OutT, 4, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
+        if (shape == 3) return launch_dma<OutT, 4, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream, mode);
       if constexpr ((TW_DMA_SHAPES & 4) != 0)
-        if (shape == 2) return launch_dma<OutT, 2, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
+        if (shape == 2) return launch_dma<OutT, 2, 4, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream, mode);
       if constexpr ((TW_DMA_SHAPES & 2) != 0)
-        if (shape == 1) return launch_dma<OutT, 2, 2, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
+        if (shape == 1) return launch_dma<OutT, 2, 2, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream, mode);
     }
     if (shape == 3 || shape == 4)             // (K no multiple of 32: the register-staged 256x256 tile for both)
-      return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
+      return launch_tiled<T, OutT, 4, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream, mode);
   }
   if (shape == 3 || shape == 4) return TW_ERR_BAD_ARGUMENT;
   if (shape == 2)
-    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
-  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream);
+    return launch_tiled<T, OutT, 2, 4, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream, mode);
+  return launch_tiled<T, OutT, 2, 2, SHUF, GLU>(A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, splits, stream, mode);
 }
 
 template <typename T, typename OutT>
 static int tiled_by_layout(int shuffled, int glu, int shape, const void* A, long lda, const void* W, long ldw,
                            const float* bias, const float* residual, long ldr, void* C, long ldc, float* partial,
-                           long partial_bytes, int M, int N, int K, hipStream_t stream) {
+                           long partial_bytes, int M, int N, int K, hipStream_t stream,
+                           TiledMode* mode = nullptr) {
   const T* a = (const T*)A;
   const T* w = (const T*)W;
   OutT* c = (OutT*)C;
   if (glu) {
     if constexpr (sizeof(T) == sizeof(OutT)) {
-      if (shuffled) return tiled_by_shape<T, OutT, true, true>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream);
-      return tiled_by_shape<T, OutT, false, true>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream);
+      if (shuffled) return tiled_by_shape<T, OutT, true, true>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream, mode);
+      return tiled_by_shape<T, OutT, false, true>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream, mode);
     }
     return TW_ERR_BAD_ARGUMENT;          // the GLU form writes the input type
   }
-  if (shuffled) return tiled_by_shape<T, OutT, true, false>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream);
-  return tiled_by_shape<T, OutT, false, false>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream);
+  if (shuffled) return tiled_by_shape<T, OutT, true, false>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream, mode);
+  return tiled_by_shape<T, OutT, false, false>(shape, a, lda, w, ldw, bias, residual, ldr, c, ldc, partial, partial_bytes, M, N, K, stream, mode);
 }
 
 int tw_tiled_linear(int dtype, int out_f32, int shuffled, int glu, int shape, const void* A, long lda,
@@ -701,6 +722,38 @@ int tw_tiled_linear(int dtype, int out_f32, int shuffled, int glu, int shape, co
   if (out_f32)
     return tiled_by_layout<bf16_t, float>(shuffled, glu, shape, A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
   return tiled_by_layout<bf16_t, bf16_t>(shuffled, glu, shape, A, lda, W, ldw, bias, residual, ldr, C, ldc, partial, partial_bytes, M, N, K, stream);
+}
+
+// K ranges the tiled kernels would use for this product (1: no split).
+int tw_tiled_partial_splits(int dtype, int shuffled, long lda, int M, int N, int K) {
+  TiledMode mode;
+  mode.dry = true;
+  int err;
+  if (dtype == TW_DTYPE_F32)
+    err = tiled_by_layout<float, float>(shuffled, 0, 0, nullptr, lda, nullptr, K, nullptr, nullptr, 0, nullptr, N, nullptr, 0, M, N, K, nullptr, &mode);
+  else if (dtype == TW_DTYPE_BF16)
+    err = tiled_by_layout<bf16_t, float>(shuffled, 0, 0, nullptr, lda, nullptr, K, nullptr, nullptr, 0, nullptr, N, nullptr, 0, M, N, K, nullptr, &mode);
+  else
+    return 0;
+  return err ? 0 : mode.splits;
+}
+
+// partial[s][M][N] (float32) = A[:, K range s] W[:, K range s]^T for the ranges the tiled kernels choose;
+// no reduction. *splits_used tells how many ranges there are (1: partial[0] is the product itself).
+int tw_tiled_partials(int dtype, int shuffled, const void* A, long lda, const void* W, long ldw, float* partial,
+                      long partial_bytes, int M, int N, int K, int* splits_used, hipStream_t stream) {
+  TW_REQUIRE(partial != nullptr && (uintptr_t)partial % 16 == 0 && partial_bytes >= (long)M * N * 4);
+  TiledMode mode;
+  mode.leave = true;
+  int err;
+  if (dtype == TW_DTYPE_F32)
+    err = tiled_by_layout<float, float>(shuffled, 0, 0, A, lda, W, ldw, nullptr, nullptr, 0, partial, N, partial, partial_bytes, M, N, K, stream, &mode);
+  else if (dtype == TW_DTYPE_BF16)
+    err = tiled_by_layout<bf16_t, float>(shuffled, 0, 0, A, lda, W, ldw, nullptr, nullptr, 0, partial, N, partial, partial_bytes, M, N, K, stream, &mode);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  if (splits_used) *splits_used = mode.splits;
+  return err;
 }
 
 long tw_tiled_workspace_bytes(int dtype, int rows, int N, int K) {

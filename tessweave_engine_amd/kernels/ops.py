@@ -226,17 +226,25 @@ def linear_partial_splits(dtype, n, k):
     return int(library().tw_linear_partial_splits(dtype_id(dtype), int(n), int(k)))
 
 
+def linear_partial_splits_rows(weight, rows):
+    """K ranges `linear_partials` uses for ROWS rows against WEIGHT; 0 where it cannot or would not split
+    (above 64 rows the tiled kernels decide, and split only where whole tiles would leave CUs idle)."""
+    n, k, _, _, shuffled, w_dtype = _weight_args(weight)
+    return int(library().tw_linear_partial_splits_rows(dtype_id(w_dtype), shuffled, int(rows), n, k))
+
+
 def linear_partials(x, weight, partial):
-    """partial[s] = x[:, K range s] @ weight[:, K range s].T in float32, for at most 64 rows.
+    """partial[s] = x[:, K range s] @ weight[:, K range s].T in float32, for the K ranges
+    `linear_partial_splits_rows` names for these rows.
 
     The caller's next kernel adds the splits up.
     """
     m, kx, lda = _rows(x, "x")
     n, k, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
     _need(kx == k, "linear_partials shapes do not agree")
-    _need(x.dtype == w_dtype and 1 <= m <= 64, "linear_partials takes 1..64 rows of the weight's type")
-    splits = linear_partial_splits(w_dtype, n, k)
-    _need(splits > 0, "linear_partials needs K to be a multiple of 16 bytes")
+    _need(x.dtype == w_dtype and m >= 1, "linear_partials takes rows of the weight's type")
+    splits = linear_partial_splits_rows(weight, m)
+    _need(splits > 0, "linear_partials: K must be a multiple of 16 bytes, and above 64 rows the shape must be one the tiled kernels split")
     _need(partial.is_contiguous() and tuple(partial.shape) == (splits, m, n), f"partial must be [{splits}, {m}, {n}]")
     check(library().tw_linear_partials(dtype_id(x.dtype), _dev(x), lda, w_ptr, ldw, shuffled,
                                        _dev(partial, torch.float32, "partial"), partial.numel() * 4, m, n, k,

@@ -64,7 +64,7 @@ class GroupedQueryAttention(Mixer):
         adjacent = self.position.pairing == "adjacent"
         keys, values, g = ctx.cache.keys_values(run.cache_slot)
         group = ctx.groups[g]
-        if self.qkv.deferrable(n):
+        if n <= 64 and self.qkv.deferrable(n):
             # few rows: the projection leaves split-K sums; bias, rotation and cache write finish them
             partial = self.qkv.forward_partials(ctx, h, "qkv")
             ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,

@@ -33,8 +33,8 @@ class SwiGLU(FeedForward):
             gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
             self.gate_up.forward(ctx, h, gu)
             ops.silu_mul(gu, act)
-        if ctx.defer_sums and self.down.deferrable(n):
-            # few rows: the down projection's split-K sums are left to the next norm
+        if ctx.defer_sums and not self.down.biases and self.down.deferrable(n):
+            # where the down projection splits K (few rows; many rows against its long K), the sums are left to the next norm
             return self.down.forward_partials(ctx, act, "down")
         self.down.forward(ctx, act, x, residual=x)
         return None

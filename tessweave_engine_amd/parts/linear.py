@@ -130,20 +130,31 @@ class Linear(Part):
             col += rows
         return out
 
-    # ---- few rows: leave the split-K sums to the next kernel --------------------------------
+    # ---- leave the split-K sums to the next kernel -------------------------------------------
+    def _partial_splits(self, n_rows):
+        """K ranges of `forward_partials` for N_ROWS rows (0: none). Up to 64 rows the streaming kernel's
+        ranges depend on the matrix alone; above, the tiled kernels choose them per row count."""
+        key = ("splits", 64 if n_rows <= 64 else n_rows)
+        if key not in self._ws_floats:
+            self._ws_floats[key] = ops.linear_partial_splits_rows(self.weights[0], n_rows)
+        return self._ws_floats[key]
+
     def deferrable(self, n_rows):
-        """Can `forward_partials` run for N_ROWS rows? (one packed matrix, no bias of its own to add)"""
-        if len(self.weights) != 1 or not 1 <= n_rows <= 64:
+        """Can `forward_partials` run for N_ROWS rows, and is it worth it? (one packed matrix and a kernel
+        that splits K for these rows anyway; a bias is NOT added to the partial sums: the caller's next
+        kernel has to, or the caller must not defer)"""
+        if len(self.weights) != 1 or n_rows < 1:
             return False
-        w = self.weights[0]
-        if "splits" not in self._ws_floats:
-            self._ws_floats["splits"] = ops.linear_partial_splits(w.dtype, w.shape[0], w.shape[1])
-        return self._ws_floats["splits"] > 0
+        return self._partial_splits(n_rows) > 0
 
     def forward_partials(self, ctx, x, tag):
         """float32 [splits, n, out] partial sums of x @ W.T (bias NOT added); see ops.linear_partials."""
         w = self.weights[0]
-        splits = self._ws_floats["splits"]
-        buf = ctx.workspace.get("linear.partial." + tag, (splits, 64, w.shape[0]), torch.float32)
-        partial = buf.view(-1)[:splits * x.shape[0] * w.shape[0]].view(splits, x.shape[0], w.shape[0])
+        n = x.shape[0]
+        splits = self._partial_splits(n)
+        if n <= 64:     # sized once for the largest such batch, so that it never regrows under a captured graph
+            buf = ctx.workspace.get("linear.partial." + tag, (splits, 64, w.shape[0]), torch.float32)
+        else:
+            buf = ctx.workspace.get("linear.partial.rows." + tag, (splits, n, w.shape[0]), torch.float32)
+        partial = buf.view(-1)[:splits * n * w.shape[0]].view(splits, n, w.shape[0])
         return ops.linear_partials(x, w, partial)

@@ -66,6 +66,16 @@ def test_rmsnorm(ops, device, dtype, hidden, eps):
     torch.testing.assert_close(x2.cpu(), total.float(), atol=1e-5, rtol=1e-6)
     want3 = plain.rms_norm(total, w.cpu().double(), eps).float()
     torch.testing.assert_close(out3.float().cpu(), want3, **tol(dtype, (3e-6, 3e-6), (1e-2, 1e-2)))
+    # many rows with partial sums (the wave-per-row kernel's own form of it)
+    addm = rand((2, 261, hidden), torch.float32, device, 1.0, seed=6)
+    xm2 = xm.clone()
+    outm2 = torch.full((261, hidden), float("nan"), dtype=dtype, device=device)
+    ops.rmsnorm(xm2, w, eps, outm2, add=addm)
+    totalm = xm.cpu().double() + addm.cpu().double().sum(0)
+    torch.testing.assert_close(xm2.cpu(), totalm.float(), atol=1e-5, rtol=1e-6)
+    torch.testing.assert_close(xm2, (addm[0] + addm[1]) + xm, atol=0, rtol=0)          # in that order, to the bit
+    torch.testing.assert_close(outm2.float().cpu(), plain.rms_norm(totalm, w.cpu().double(), eps).float(),
+                               **tol(dtype, (3e-6, 3e-6), (1e-2, 1e-2)))
     # gathered rows AND partial sums (a row may be named twice): x itself stays as it was
     rows2 = torch.tensor([6, 0, 6], dtype=torch.int32, device=device)
     x3 = x.clone()
@@ -299,6 +309,34 @@ def test_linear_partials(ops, device, dtype, m, n, k):
     part.fill_(float("nan"))
     ops.linear_partials(x, w, part)
     torch.testing.assert_close(part.sum(0), rows_sum, atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(300, 256, 4096), (1024, 512, 8192), (2048, 896, 9472), (520, 130, 2056),
+                                   (2048, 4096, 512)])
+def test_linear_partials_of_many_rows(ops, device, dtype, m, n, k):
+    """Above 64 rows the tiled kernels leave the sums of their K ranges; where they would not split K
+    the call is refused (the product with its epilogue is then the better one)."""
+    x = rand((m, k), dtype, device, 1.0, seed=1)
+    w = rand((n, k), dtype, device, 0.05, seed=2)
+    want = (x.double() @ w.double().T).cpu()
+    scale = math.sqrt(k) * 0.05
+    seen = 0
+    for weight in (w, ops.shuffle_weight(w)):
+        splits = ops.linear_partial_splits_rows(weight, m)
+        if splits == 0:
+            with pytest.raises(ValueError, match="linear_partials"):
+                ops.linear_partials(x, weight, torch.empty(1, m, n, device=device))
+            continue
+        assert splits >= 2
+        seen += 1
+        part = torch.full((splits, m, n), float("nan"), device=device)
+        ops.linear_partials(x, weight, part)
+        torch.testing.assert_close(part.double().sum(0).cpu(), want, atol=3e-5 * scale, rtol=1e-5)
+        assert part.abs().amax(dim=(1, 2)).min() > 0             # every range did its share
+        with pytest.raises(ValueError, match="partial must be"):
+            ops.linear_partials(x, weight, torch.empty(splits + 1, m, n, device=device))
+    assert seen or (m, n, k) == (2048, 4096, 512)                # (many tiles, short K: nothing to split)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
