@@ -25,7 +25,9 @@ int tw_sample_rows(const float* logits, long ld, int rows, int vocab, const floa
 // no routine that does. More than TW_SAMPLE_STATIC_MAX_ROWS rows are refused with TW_ERR_TOO_LARGE.
 // All calls on one GPU share that array: two calls whose kernels overlap there (other streams, other
 // threads) race; calls on one stream are ordered and safe. Nothing in the array has to start at zero:
-// every entry a call reads it has written first.
+// every entry a call reads it has written first. The first call on a device looks the array's address
+// up there (hipGetSymbolAddress, no allocation) and keeps it: a caller that captures graphs makes one
+// call on the device before its first capture.
 #define TW_SAMPLE_STATIC_MAX_ROWS 256
 int tw_sample_rows_static(const float* logits, long ld, int rows, int vocab, const float* temperature,
                           const uint64_t* seeds, const int* counters, int* out, hipStream_t stream);
