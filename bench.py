@@ -12,8 +12,9 @@ request. One JSON line is printed: decoded tokens a second, a 2,048-token
 prefill, the decode step's HBM roofline (against the nominal 8 TB/s and against
 what a plain streaming reader reaches on this device, measured in the same run),
 and further points: decode at batch 1 and 64 at the same context; the same batch
-of 8 with the engine opened for 32,768 tokens a request (`decode_b8_open32k`);
-and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
+of 8 with the engine opened for 32,768 tokens a request (`decode_b8_open32k`)
+and with requests of that length (`decode_b8_ctx32k`: the cache is then as large
+as the weights); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
 (`gen512_b*`, decoded tokens a second over the generated part).
 
 Other sizes of the architecture: --shape 14b|32b. --serve measures continuous
@@ -61,7 +62,7 @@ def parse():
     p.add_argument("--max-context", type=int, default=0,
                    help="tokens a request may hold, which the engine is opened for (0: the context + 1)")
     p.add_argument("--no-extra-points", action="store_true",
-                   help="skip decode_b8_open32k and the gen512_b* points (1,024-token prompts + 512 generated)")
+                   help="skip decode_b8_open32k, decode_b8_ctx32k and the gen512_b* points (1,024-token prompts + 512 generated)")
     p.add_argument("--no-graphs", action="store_true")
     p.add_argument("--prefill-only", action="store_true", help="measure only the prefill (profiling runs)")
     p.add_argument("--seed", type=int, default=0)
@@ -282,6 +283,9 @@ def main():
         for b in (1, 8, 64):
             tps, _, _ = decode_run(model, torch, b, 1024 + 512, 504, 8, args.dtype, use_graphs, args.seed, opened)
             points[f"gen512_b{b}"] = round(tps, 1)
+        # and with requests that really are that long: the cache is then as large as the weights
+        tps, _, _ = decode_run(model, torch, args.batch, opened - 16, 32, 8, args.dtype, use_graphs, args.seed, opened)
+        points[f"decode_b{args.batch}_ctx{opened // 1024}k"] = round(tps, 1)
     ceiling = read_ceiling(torch, model.device)
 
     line = {
