@@ -14,7 +14,8 @@ what a plain streaming reader reaches on this device, measured in the same run),
 and further points: decode at batch 1 and 64 at the same context; the same batch
 of 8 with the engine opened for 32,768 tokens a request (`decode_b8_open32k`)
 and with requests of that length (`decode_b8_ctx32k`: the cache is then as large
-as the weights); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
+as the weights; `prefill_32k_prompts`: tokens a second over those prompts, which
+go through in portions of 2,048); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
 (`gen512_b*`, decoded tokens a second over the generated part).
 
 Other sizes of the architecture: --shape 14b|32b. --serve measures continuous
@@ -97,9 +98,13 @@ def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, s
     from tessweave_engine_amd.engine import StepEntry
     engine._admit()
     assert len(engine.active) == batch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
     for r in requests:
         for i in range(0, prompt_len - 1, chunk):
             engine.stepper.step([StepEntry(r.seq, r.prompt[i:min(prompt_len - 1, i + chunk)], [])])
+    torch.cuda.synchronize()
+    decode_run.prompt_tokens_per_s = batch * (prompt_len - 1) / (time.perf_counter() - t0)
     for _ in range(warmup):
         engine.step()
     engine.flush()
@@ -286,6 +291,8 @@ def main():
         # and with requests that really are that long: the cache is then as large as the weights
         tps, _, _ = decode_run(model, torch, args.batch, opened - 16, 32, 8, args.dtype, use_graphs, args.seed, opened)
         points[f"decode_b{args.batch}_ctx{opened // 1024}k"] = round(tps, 1)
+        # what that run's prompts took: portions of 2,048 tokens, most of their keys from the cache
+        points[f"prefill_{opened // 1024}k_prompts"] = round(decode_run.prompt_tokens_per_s, 1)
     ceiling = read_ceiling(torch, model.device)
 
     line = {
