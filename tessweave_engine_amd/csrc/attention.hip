@@ -634,6 +634,9 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   constexpr int KPIECES = (32 * DTMAX * 2 + 255) / 256;  // 16-byte pieces per thread per block
   constexpr int VPIECES = (DTMAX * 16 * 4 + 255) / 256;
   constexpr int CH = DTMAX * 2;                          // 16-byte chunks per key row of this size class
+  // every thread's every piece is part of the block (then the copies to LDS carry no lane mask, which costs
+  // a dozen scalar instructions a piece)
+  constexpr bool ALL_USED = EXACT && (32 * CH) % 256 == 0 && (DTMAX * 16 * 4) % 256 == 0;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   char* lds_k = lds;
   char* lds_v = lds + 2 * KSTAGE;
@@ -788,19 +791,27 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       for (int i = 0; i < VPIECES; ++i) v_pg[i] = entry[held(v_slot[i])];
     }
   };
-  const size_t head_off = (size_t)kvh * head_stride;
-  const size_t page_stride = (size_t)a.kv_heads * head_stride;
+  // Where this lane's pieces lie in page 0 of its kv head: an address is that plus page * (bytes of a page)
+  // plus where the block starts inside its page, one 32 x 32 -> 64 bit multiply-add and one 64-bit add a
+  // piece (the launcher checks that a page's bytes fit 32 bits; page numbers are not negative).
+  const unsigned page_bytes = (unsigned)a.kv_heads * head_stride * 2u;
+  const char* k_at[KPIECES];
+  const char* v_at[VPIECES];
+#pragma unroll
+  for (int i = 0; i < KPIECES; ++i) k_at[i] = (const char*)keys + ((size_t)kvh * head_stride + k_goff[i]) * 2;
+#pragma unroll
+  for (int i = 0; i < VPIECES; ++i) v_at[i] = (const char*)values + ((size_t)kvh * head_stride + v_goff[i]) * 2;
   auto fetch = [&](int blk_v) {                              // (after lookup of the same block)
     const int blk = __builtin_amdgcn_readfirstlane(blk_v);
     const int p0 = blk * 32;
-    const int in_page = P >= 32 ? (p0 & pmask) : 0;          // where the block starts inside its page
-    const size_t k_in = head_off + (size_t)in_page * D, v_in = head_off + in_page;
+    const unsigned in_page = P >= 32 ? (unsigned)(p0 & pmask) : 0u;   // where the block starts inside its page
+    const unsigned k_in = in_page * (unsigned)D * 2u, v_in = in_page * 2u;
 #pragma unroll
     for (int i = 0; i < KPIECES; ++i)
-      kreg[i] = tw_load_frag(keys + ((size_t)k_pg[i] * page_stride + k_in + k_goff[i]));
+      kreg[i] = tw_load_frag((const bf16_t*)(k_at[i] + ((uint64_t)(unsigned)k_pg[i] * page_bytes + k_in)));
 #pragma unroll
     for (int i = 0; i < VPIECES; ++i)
-      vreg[i] = tw_load_frag(values + ((size_t)v_pg[i] * page_stride + v_in + v_goff[i]));
+      vreg[i] = tw_load_frag((const bf16_t*)(v_at[i] + ((uint64_t)(unsigned)v_pg[i] * page_bytes + v_in)));
     if (p0 + 32 > kv_len || p0 < lo) {
 #pragma unroll
       for (int i = 0; i < VPIECES; ++i) {
@@ -814,10 +825,10 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   auto stash = [&](int buf) {                                // registers -> LDS
 #pragma unroll
     for (int i = 0; i < KPIECES; ++i)
-      if (k_use[i]) *reinterpret_cast<bf16x8*>(lds_k + buf * KSTAGE + k_loff[i]) = kreg[i];
+      if (ALL_USED || k_use[i]) *reinterpret_cast<bf16x8*>(lds_k + buf * KSTAGE + k_loff[i]) = kreg[i];
 #pragma unroll
     for (int i = 0; i < VPIECES; ++i)
-      if (v_use[i]) *reinterpret_cast<bf16x8*>(lds_v + buf * VSTAGE + v_loff[i]) = vreg[i];
+      if (ALL_USED || v_use[i]) *reinterpret_cast<bf16x8*>(lds_v + buf * VSTAGE + v_loff[i]) = vreg[i];
   };
 
   // LDS addresses of this lane's fragments in stage 0
@@ -1069,6 +1080,7 @@ static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_
   a.max_tiles = (int)tw_div_up(rows, a.tile_rows);
   const long total = (long)a.max_tiles * a.kv_heads * n_seqs * a.max_chunks;
   TW_REQUIRE(total < (1L << 30));
+  TW_REQUIRE((long)a.kv_heads * a.page_size * a.head_dim * 2 < (1L << 31));      // a page's bytes: 32-bit in the kernel
   dim3 grid((unsigned)total);
   const size_t lds_bytes = 2 * 32 * (DTMAX * 32 + 16) + 2 * DTMAX * 16 * TW_PF_VROW;
   static bool attribute_set = false;
