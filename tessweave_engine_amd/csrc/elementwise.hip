@@ -374,6 +374,74 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* 
 // The same work from split-K partial sums, one workgroup per (token, head): the
 // head's values are round_T(sum_s partial[s][n][col] + bias[col]); q heads are
 // rotated into qkv, k heads are rotated into the pages, v heads go to the pages.
+// The common case of rope_kv_write_kernel (the whole head rotated as pairs (j, j + half), every row and
+// pointer 16-byte aligned): a thread moves 16 bytes of each half of a head at a time, and finds its head
+// with one division instead of one per element. Every element goes through the same arithmetic, so the
+// two kernels give the same bits. (2,048 tokens of 36 heads of 128, cold: the rotation alone 12.5 -> 7.7 us;
+// with the cache written 18.4 -> 16.2 us: the values' transposed pages still take one 2-byte store an
+// element, which is now most of the kernel's time.)
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(T* __restrict__ qkv, long ld,
+                                                                const float* __restrict__ cos_t,
+                                                                const float* __restrict__ sin_t,
+                                                                const int* __restrict__ slots, T* __restrict__ keys,
+                                                                T* __restrict__ values, int q_heads, int kv_heads,
+                                                                int head_dim, int page_size, int write_cache) {
+  typedef typename Elem<T>::Frag Frag;
+  constexpr int V = Elem<T>::kPerFrag;
+  const int n = blockIdx.x;
+  const int half = head_dim / 2, cpb = half / V;             // 16-byte chunks per half head
+  T* row = qkv + (size_t)n * ld;
+  const float* c = cos_t + (size_t)n * half;
+  const float* s = sin_t + (size_t)n * half;
+  const int slot = write_cache ? slots[n] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  const int rot_heads = q_heads + kv_heads;
+  for (int item = threadIdx.x; item < rot_heads * cpb; item += blockDim.x) {
+    const int head = item / cpb, j0 = (item - head * cpb) * V;
+    T* x = row + (size_t)head * head_dim;
+    T* dst = x;
+    if (head >= q_heads) {
+      if (slot < 0) continue;
+      dst = keys + (((size_t)page * kv_heads + (head - q_heads)) * page_size + off) * head_dim;
+    }
+    const Frag lo = tw_load_frag(x + j0), hi = tw_load_frag(x + half + j0);
+    float cj[V], sj[V];
+#pragma unroll
+    for (int q = 0; q < V / 4; ++q) {
+      const f32x4 cq = *reinterpret_cast<const f32x4*>(c + j0 + 4 * q);
+      const f32x4 sq = *reinterpret_cast<const f32x4*>(s + j0 + 4 * q);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        cj[4 * q + e] = cq[e];
+        sj[4 * q + e] = sq[e];
+      }
+    }
+    Frag out_lo, out_hi;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      float r_lo, r_hi;
+      tw_rotate_pair(tw_to_float(lo[e]), tw_to_float(hi[e]), cj[e], sj[e], r_lo, r_hi);
+      out_lo[e] = tw_from_float<T>(r_lo);
+      out_hi[e] = tw_from_float<T>(r_hi);
+    }
+    *reinterpret_cast<Frag*>(dst + j0) = out_lo;
+    *reinterpret_cast<Frag*>(dst + half + j0) = out_hi;
+  }
+  if (slot < 0) return;
+  // values, transposed inside the page
+  const T* v = row + (size_t)rot_heads * head_dim;
+  const int vpb = head_dim / V;
+  for (int item = threadIdx.x; item < kv_heads * vpb; item += blockDim.x) {
+    const int kh = item / vpb, d0 = (item - kh * vpb) * V;
+    const Frag val = tw_load_frag(v + (size_t)kh * head_dim + d0);
+    T* dst = values + (((size_t)page * kv_heads + kh) * head_dim + d0) * page_size + off;
+#pragma unroll
+    for (int e = 0; e < V; ++e) dst[(size_t)e * page_size] = val[e];
+  }
+}
+
 template <typename T>
 __global__ void qkv_finish_kernel(T* __restrict__ qkv, long ld, const float* __restrict__ cos_t,
                                   const float* __restrict__ sin_t, const int* __restrict__ slots,
@@ -476,6 +544,23 @@ extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_
       qkv_finish_kernel<bf16_t><<<grid, threads, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots, (bf16_t*)keys,
                                                              (bf16_t*)values, q_heads, kv_heads, head_dim, rot,
                                                              page_size, write_cache, partial, splits, split_stride, bias, adjacent);
+    else
+      return TW_ERR_BAD_ARGUMENT;
+    return TW_LAUNCH_RESULT();
+  }
+  // the whole head rotated in halves, everything 16-byte aligned: the vector form
+  const int per16 = dtype == TW_DTYPE_F32 ? 4 : 8;
+  if (rot == head_dim && !adjacent && head_dim % (2 * per16) == 0 && ld % per16 == 0 &&
+      (uintptr_t)qkv % 16 == 0 && (uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0 &&
+      (!write_cache || (uintptr_t)keys % 16 == 0)) {
+    if (dtype == TW_DTYPE_F32)
+      rope_kv_write_vec_kernel<float><<<n, 256, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
+                                                             (float*)values, q_heads, kv_heads, head_dim,
+                                                             page_size, write_cache);
+    else if (dtype == TW_DTYPE_BF16)
+      rope_kv_write_vec_kernel<bf16_t><<<n, 256, 0, stream>>>((bf16_t*)qkv, ld, cos_t, sin_t, slots, (bf16_t*)keys,
+                                                              (bf16_t*)values, q_heads, kv_heads, head_dim,
+                                                              page_size, write_cache);
     else
       return TW_ERR_BAD_ARGUMENT;
     return TW_LAUNCH_RESULT();

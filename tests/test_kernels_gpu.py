@@ -87,7 +87,8 @@ def test_rmsnorm(ops, device, dtype, hidden, eps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("q_heads,kv_heads,head_dim,page,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 8, 1e6), (5, 5, 48, 4, 5e5)])
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,page,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 8, 1e6), (5, 5, 48, 4, 5e5),
+                                                                 (3, 1, 20, 8, 1e4), (28, 4, 128, 16, 1e6)])
 def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, page, theta):
     n, pages = 9, 7
     width = (q_heads + 2 * kv_heads) * head_dim
@@ -128,6 +129,15 @@ def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, p
     assert torch.isnan(kflat[~written]).all()
     vflat = vc.permute(0, 3, 1, 2).reshape(pages * page, -1)
     assert torch.isnan(vflat[~written]).all()
+    # rows that are not 16-byte aligned take the kernel that moves one element at a time: identical bits
+    wide = torch.zeros(n, width + 1, dtype=dtype, device=device)
+    odd = wide[:, :width]
+    odd.copy_(before)
+    keys1, values1 = torch.full_like(keys, float("nan")), torch.full_like(values, float("nan"))
+    ops.rope_kv_write(odd, cos, sin, slots, keys1, values1, q_heads, kv_heads, head_dim, page)
+    torch.testing.assert_close(odd, qkv, atol=0, rtol=0)
+    torch.testing.assert_close(keys1, keys, atol=0, rtol=0, equal_nan=True)
+    torch.testing.assert_close(values1, values, atol=0, rtol=0, equal_nan=True)
     # the same from split-K partial sums plus bias: identical bits
     bias = rand((width,), torch.float32, device, 0.3, seed=9)
     parts = rand((3, n, width), torch.float32, device, 1.0, seed=10)
