@@ -378,8 +378,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long ld, const float* 
 // pointer 16-byte aligned): a thread moves 16 bytes of each half of a head at a time, and finds its head
 // with one division instead of one per element. Every element goes through the same arithmetic, so the
 // two kernels give the same bits. (2,048 tokens of 36 heads of 128, cold: the rotation alone 12.5 -> 7.7 us;
-// with the cache written 18.4 -> 16.2 us: the values' transposed pages still take one 2-byte store an
-// element, which is now most of the kernel's time.)
+// with the cache written 18.4 -> 14.9 us, of which the grouped stores of the values, below, are 1.3.)
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(T* __restrict__ qkv, long ld,
                                                                 const float* __restrict__ cos_t,
@@ -430,9 +429,40 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(T* __restrict__ 
     *reinterpret_cast<Frag*>(dst + half + j0) = out_hi;
   }
   if (slot < 0) return;
-  // values, transposed inside the page
-  const T* v = row + (size_t)rot_heads * head_dim;
+  // Values, transposed inside the page: element (head, d) of this token goes to [d][off], so a token alone
+  // writes one element at a time. Where V tokens in a row of the batch hold V consecutive slots that start
+  // at a multiple of V (a prompt portion: 16 bytes of one [d] row of the page), the first of them writes
+  // for all and the others write nothing: each thread reads 16 bytes of each token's row and stores V
+  // vectors of V tokens. Every token of such a group sees the same slots and decides alike.
   const int vpb = head_dim / V;
+  const int lead = n - off % V;
+  bool grouped = page_size % V == 0 && lead >= 0 && lead + V <= (int)gridDim.x;
+  if (grouped) {
+    const int first = slots[lead];
+    grouped = first >= 0 && first == slot - off % V;
+#pragma unroll
+    for (int i = 1; i < V; ++i) grouped = grouped && slots[lead + i] == first + i;
+  }
+  if (grouped) {
+    if (n != lead) return;
+    const T* v0 = row + (size_t)rot_heads * head_dim;                  // this (the first) token's values
+    for (int item = threadIdx.x; item < kv_heads * vpb; item += blockDim.x) {
+      const int kh = item / vpb, d0 = (item - kh * vpb) * V;
+      Frag val[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) val[i] = tw_load_frag(v0 + (size_t)i * ld + (size_t)kh * head_dim + d0);
+      T* dst = values + (((size_t)page * kv_heads + kh) * head_dim + d0) * page_size + off;
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        Frag column;
+#pragma unroll
+        for (int i = 0; i < V; ++i) column[i] = val[i][e];
+        *reinterpret_cast<Frag*>(dst + (size_t)e * page_size) = column;
+      }
+    }
+    return;
+  }
+  const T* v = row + (size_t)rot_heads * head_dim;
   for (int item = threadIdx.x; item < kv_heads * vpb; item += blockDim.x) {
     const int kh = item / vpb, d0 = (item - kh * vpb) * V;
     const Frag val = tw_load_frag(v + (size_t)kh * head_dim + d0);
@@ -552,7 +582,7 @@ extern "C" int tw_rope_kv_write(int dtype, void* qkv, long ld, const float* cos_
   const int per16 = dtype == TW_DTYPE_F32 ? 4 : 8;
   if (rot == head_dim && !adjacent && head_dim % (2 * per16) == 0 && ld % per16 == 0 &&
       (uintptr_t)qkv % 16 == 0 && (uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0 &&
-      (!write_cache || (uintptr_t)keys % 16 == 0)) {
+      (!write_cache || ((uintptr_t)keys % 16 == 0 && (uintptr_t)values % 16 == 0))) {
     if (dtype == TW_DTYPE_F32)
       rope_kv_write_vec_kernel<float><<<n, 256, 0, stream>>>((float*)qkv, ld, cos_t, sin_t, slots, (float*)keys,
                                                              (float*)values, q_heads, kv_heads, head_dim,

@@ -154,6 +154,48 @@ def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, p
     torch.testing.assert_close(qkv3[:, :q_heads * head_dim], ref[:, :q_heads * head_dim], atol=0, rtol=0)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kv_heads,head_dim,page", [(2, 32, 16), (4, 128, 16), (1, 64, 8), (3, 48, 32), (2, 32, 4)])
+def test_cache_write_of_tokens_with_consecutive_slots(ops, device, dtype, kv_heads, head_dim, page):
+    """A prompt portion holds consecutive slots: aligned groups of them write the transposed value pages
+    together. Runs that start and end anywhere, a gap, a row that writes nothing and rows in other pages
+    must leave exactly what the element-wise kernel leaves."""
+    q_heads = 2 * kv_heads
+    width = (q_heads + 2 * kv_heads) * head_dim
+    pages = 40
+    runs = [(3, 45), (72, 16), (97, 3)]                              # (first slot, tokens)
+    slots = [s for first, count in runs for s in range(first, first + count)]
+    slots[20] = -1                                                   # a row in the middle of a run writes nothing
+    slots += [130, 120, 122]                                         # single tokens elsewhere
+    n = len(slots)
+    slots_t = torch.tensor(slots, dtype=torch.int32, device=device)
+    qkv = rand((n, width), dtype, device)
+    half = head_dim // 2
+    positions = torch.arange(n, dtype=torch.int32, device=device)
+    inv = (1e4 ** (-torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim)).to(device)
+    cos, sin = torch.empty(n, half, device=device), torch.empty(n, half, device=device)
+    ops.rope_table(positions, inv, cos, sin)
+    results = []
+    for pad in (0, 1):                                               # rows of odd length take the element-wise kernel
+        buf = torch.zeros(n, width + pad, dtype=dtype, device=device)
+        rows = buf[:, :width]
+        rows.copy_(qkv)
+        keys = torch.full((pages, kv_heads, page, head_dim), float("nan"), dtype=dtype, device=device)
+        values = torch.full_like(keys, float("nan"))
+        ops.rope_kv_write(rows, cos, sin, slots_t, keys, values, q_heads, kv_heads, head_dim, page)
+        results.append((rows.clone(), keys, values))
+    for a, b in zip(*results):
+        torch.testing.assert_close(a, b, atol=0, rtol=0, equal_nan=True)
+    values = results[0][2].float().cpu().reshape(pages, kv_heads, head_dim, page)
+    v_src = qkv[:, (q_heads + kv_heads) * head_dim:].float().cpu().reshape(n, kv_heads, head_dim)
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for i, slot in enumerate(slots):
+        if slot >= 0:
+            written[slot] = True
+            torch.testing.assert_close(values[slot // page, :, :, slot % page], v_src[i], atol=0, rtol=0)
+    assert torch.isnan(values.permute(0, 3, 1, 2).reshape(pages * page, -1)[~written]).all()
+
+
 @pytest.mark.parametrize("theta", [1e4, 1e6])
 def test_rope_tables_at_far_positions(ops, device, theta):
     """cos and sin of float32(position) * inv_freq at positions up to 131,071: the angle is formed in float32 as
