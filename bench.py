@@ -76,7 +76,8 @@ def parse():
 
 
 def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, seed, max_context=0):
-    """Tokens/s and ms/step of STEPS decode steps at BATCH, ending at CONTEXT keys per request."""
+    """Tokens/s and ms/step of STEPS decode steps at BATCH, ending at CONTEXT keys per request; the graph
+    replays; and the tokens a second at which the prompts went through beforehand (untimed for the former)."""
     from tessweave_engine_amd.config import EngineConfig
     from tessweave_engine_amd.engine import Engine
 
@@ -104,7 +105,7 @@ def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, s
         for i in range(0, prompt_len - 1, chunk):
             engine.stepper.step([StepEntry(r.seq, r.prompt[i:min(prompt_len - 1, i + chunk)], [])])
     torch.cuda.synchronize()
-    decode_run.prompt_tokens_per_s = batch * (prompt_len - 1) / (time.perf_counter() - t0)
+    prompt_tokens_per_s = batch * (prompt_len - 1) / (time.perf_counter() - t0)
     for _ in range(warmup):
         engine.step()
     engine.flush()
@@ -120,7 +121,7 @@ def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, s
     engine.close()
     del engine
     torch.cuda.empty_cache()
-    return batch * steps / elapsed, elapsed / steps * 1000, replays
+    return batch * steps / elapsed, elapsed / steps * 1000, replays, prompt_tokens_per_s
 
 
 def serve_run(model, torch, args):
@@ -251,7 +252,7 @@ def main():
         print(json.dumps({"prefill_ms": round(ms, 3), "tokens": args.prefill_tokens,
                           "tokens_per_s": round(args.prefill_tokens / (ms / 1000), 1)}))
         return 0
-    value, ms_per_step, replays = decode_run(model, torch, args.batch, args.context, args.steps, args.warmup,
+    value, ms_per_step, replays, _ = decode_run(model, torch, args.batch, args.context, args.steps, args.warmup,
                                              args.dtype, use_graphs, args.seed, args.max_context)
     element = 2 if args.dtype == "bfloat16" else 4
     layer_weights = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
@@ -274,25 +275,25 @@ def main():
     points = {}
     for b in [int(v) for v in args.points.split(",") if v]:
         steps = min(args.steps, 64)
-        tps, _, _ = decode_run(model, torch, b, args.context, steps, 8, args.dtype, use_graphs, args.seed,
+        tps, _, _, _ = decode_run(model, torch, b, args.context, steps, 8, args.dtype, use_graphs, args.seed,
                                args.max_context)
         points[f"decode_b{b}"] = round(tps, 1)
     if not args.no_extra_points:
         # the same batch with the engine opened for 32,768 tokens a request (launch shapes must follow the
         # lengths that are served, not the lengths that are allowed)
         opened = min(32768, c.max_position_embeddings)
-        tps, _, _ = decode_run(model, torch, args.batch, args.context, min(args.steps, 64), 8, args.dtype, use_graphs,
+        tps, _, _, _ = decode_run(model, torch, args.batch, args.context, min(args.steps, 64), 8, args.dtype, use_graphs,
                                args.seed, opened)
         points[f"decode_b{args.batch}_open{opened // 1024}k"] = round(tps, 1)
         # prompts of 1,024 tokens, 512 generated (8 of them untimed): decoded tokens a second over the rest
         for b in (1, 8, 64):
-            tps, _, _ = decode_run(model, torch, b, 1024 + 512, 504, 8, args.dtype, use_graphs, args.seed, opened)
+            tps, _, _, _ = decode_run(model, torch, b, 1024 + 512, 504, 8, args.dtype, use_graphs, args.seed, opened)
             points[f"gen512_b{b}"] = round(tps, 1)
         # and with requests that really are that long: the cache is then as large as the weights
-        tps, _, _ = decode_run(model, torch, args.batch, opened - 16, 32, 8, args.dtype, use_graphs, args.seed, opened)
+        tps, _, _, prompts_tps = decode_run(model, torch, args.batch, opened - 16, 32, 8, args.dtype, use_graphs, args.seed, opened)
         points[f"decode_b{args.batch}_ctx{opened // 1024}k"] = round(tps, 1)
         # what that run's prompts took: portions of 2,048 tokens, most of their keys from the cache
-        points[f"prefill_{opened // 1024}k_prompts"] = round(decode_run.prompt_tokens_per_s, 1)
+        points[f"prefill_{opened // 1024}k_prompts"] = round(prompts_tps, 1)
     ceiling = read_ceiling(torch, model.device)
 
     line = {
