@@ -400,7 +400,8 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
       sum += pe;
       pb[e] = (bf16_t)pe;
     }
-    sum = tw_rows_sum(sum);
+    // (l is this lane's sum over its 8 keys of every block; the four lane groups of a row are added up
+    // once, after the loop: the maximum, and with it every rescaling, is the row's)
     // the running maximum of a row rarely moves after the first blocks: rescale only then
     if (__any(m_new > m)) {
       const float alpha = __expf(m - m_use);
@@ -453,6 +454,7 @@ __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
     }
   }
 
+  l = tw_rows_sum(l);
   // ---- merge the 4 waves (fixed order: wave 0 absorbs 1, 2, 3) -------------------
   if (wave > 0) {
 #pragma unroll
@@ -899,10 +901,11 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float pe = __builtin_amdgcn_exp2f(fmaf(s[rt][e >> 2][e & 3], c2, -m_use));
-        sum += pe;
+        sum = e == 0 ? pe : sum + pe;
         pb[rt][e] = (bf16_t)pe;
       }
-      sum = tw_rows_sum(sum);
+      // l is this LANE's sum (its 8 keys of every block); the four lane groups of a row are added up
+      // once, after the loop
       l[rt] = l[rt] * alpha[rt] + sum;
       m[rt] = m_new;
     }
@@ -946,6 +949,8 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     __syncthreads();
   }
   compute_if_seen(blk, (blk - blk_begin) & 1);                // the last block (blk_end > blk_begin always)
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) l[rt] = tw_rows_sum(l[rt]);   // (the running maximum, and so every rescaling, was the row's: the same for the four)
 
   if (n_chunks > 1) {
 #pragma unroll
