@@ -643,7 +643,8 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   char* lds_k = lds;
   char* lds_v = lds + 2 * KSTAGE;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // the same for the wave's lanes: what follows from it stays scalar
   const int r = lane & 15, g = lane >> 4;
   const int G = a.q_heads / a.kv_heads;
   // Which tile this workgroup takes. Tiles are ranked by the keys they see (most first: rank =
