@@ -15,7 +15,7 @@ import math
 
 import numpy as np
 
-from .pages import CapacityError, PagePool
+from .pages import CapacityError, PagePool, block_keys
 from .spec import CacheLayout
 
 _STATE_DTYPES = {"float32": "float32", "bfloat16": "bfloat16", "int32": "int32"}
@@ -24,7 +24,8 @@ _STATE_DTYPES = {"float32": "float32", "bfloat16": "bfloat16", "int32": "int32"}
 class Sequence:
     """What the cache holds for one live request."""
 
-    __slots__ = ("id", "state_slot", "tables", "computed", "cached", "promised", "budget", "closed")
+    __slots__ = ("id", "state_slot", "tables", "computed", "cached", "promised", "budget", "closed",
+                 "block_keys", "key_namespace")
 
     def __init__(self, seq_id, state_slot, n_groups):
         self.id = seq_id
@@ -35,6 +36,8 @@ class Sequence:
         self.promised = [0] * n_groups                 # pages promised to this request and not yet taken
         self.budget = [0] * n_groups                   # pages reserved at admission (0: grows on demand)
         self.closed = False
+        self.block_keys = []                           # prefix-index keys of the first full blocks of its tokens, as far
+        self.key_namespace = None                      # as they have been hashed (a request's tokens only grow)
 
     def held(self, group):
         return sum(1 for page in self.tables[group] if page >= 0)
@@ -161,7 +164,7 @@ class CacheManager:
         if not self.prefix_cache or seq.computed or seq.tables[0]:
             return 0
         pool = self.pools[0]
-        shared = pool.acquire_prefix(prompt, namespace)
+        shared = pool.acquire_prefix(prompt, namespace, keys=self._keys(seq, prompt, len(prompt) - 1, namespace))
         seq.tables[0] = list(shared)
         self.table_rows[0][seq.state_slot, :len(shared)] = shared
         seq.computed = seq.cached = len(shared) * self.page_size
@@ -187,8 +190,19 @@ class CacheManager:
         """Offer the full blocks of TOKENS that SEQ holds keys and values for (its first COMPUTED tokens,
         by default everything it has computed) to the prefix index."""
         if self.prefix_cache:
-            upto = seq.computed if computed is None else min(int(computed), seq.computed)
-            self.pools[0].publish(tokens, upto, seq.tables[0], namespace)
+            upto = min(seq.computed if computed is None else min(int(computed), seq.computed), len(tokens))
+            self.pools[0].publish(tokens, upto, seq.tables[0], namespace, keys=self._keys(seq, tokens, upto, namespace))
+
+    def _keys(self, seq, tokens, upto, namespace):
+        """Prefix-index keys of the full blocks of TOKENS[:UPTO]. A request's tokens only grow, so the keys
+        hashed for it before stay valid and only the blocks after them are hashed now: a prompt published
+        portion by portion is hashed once over, not once per portion."""
+        if seq.key_namespace != namespace:
+            seq.block_keys, seq.key_namespace = [], namespace
+        blocks = max(0, int(upto)) // self.page_size
+        if blocks > len(seq.block_keys):
+            seq.block_keys = block_keys(tokens[:blocks * self.page_size], self.page_size, namespace, known=seq.block_keys)
+        return seq.block_keys[:blocks]
 
     def first_needed_block(self, group, computed):
         """First logical block of GROUP that a query at position >= COMPUTED can see."""

@@ -23,25 +23,32 @@ behalf of a request that then still does not fit. Here a request for pages is
 first checked against what eviction COULD free; only then are entries dropped,
 oldest first, and only entries whose page nobody else uses. Within one prefix
 chain deeper blocks are kept older than their parents, so a chain is eaten from
-its tail and what stays is still reachable from the root.
+its tail and what stays is still reachable from the root. Both a lookup and a
+publication re-age the whole chain they walk, root last: a chain that enters
+the index portion by portion (its root first) keeps that order too.
 """
 from __future__ import annotations
 
 from collections import OrderedDict
 import hashlib
+import struct
 
 
 class CapacityError(RuntimeError):
     """Not enough free pages (or state slots); the caller waits or refuses."""
 
 
-def block_keys(tokens, page_size, namespace):
-    """Keys of the full blocks of TOKENS, root first."""
-    key = hashlib.sha256(namespace.encode()).digest()
-    keys = []
-    for end in range(page_size, len(tokens) + 1, page_size):
-        packed = b"".join(int(t).to_bytes(8, "little", signed=True) for t in tokens[end - page_size:end])
-        key = hashlib.sha256(key + packed).digest()
+def block_keys(tokens, page_size, namespace, known=()):
+    """Keys of the full blocks of TOKENS, root first.
+
+    KNOWN: the keys of the first len(KNOWN) blocks, if the caller already has them (a key names its
+    whole prefix, so hashing goes on from the last of them and touches only the blocks after it).
+    """
+    keys = list(known[:len(tokens) // page_size])
+    key = keys[-1] if keys else hashlib.sha256(namespace.encode()).digest()
+    pack = struct.Struct("<%dq" % page_size).pack
+    for end in range((len(keys) + 1) * page_size, len(tokens) + 1, page_size):
+        key = hashlib.sha256(key + pack(*tokens[end - page_size:end])).digest()
         keys.append(key)
     return keys
 
@@ -128,13 +135,16 @@ class PagePool:
         self.promised -= count
 
     # ---- prefix index -------------------------------------------------------------------
-    def acquire_prefix(self, tokens, namespace="local"):
-        """Pages of the longest indexed prefix of TOKENS, each with one more use; never the last token's block."""
+    def acquire_prefix(self, tokens, namespace="local", keys=None):
+        """Pages of the longest indexed prefix of TOKENS, each with one more use; never the last token's block.
+        KEYS: the block keys of TOKENS, if the caller has them."""
         if not self.prefix_cache:
             return []
-        usable = (len(tokens) - 1) // self.page_size * self.page_size
+        usable = (len(tokens) - 1) // self.page_size
+        if keys is None:
+            keys = block_keys(tokens[:usable * self.page_size], self.page_size, namespace)
         found = []
-        for key in block_keys(tokens[:usable], self.page_size, namespace):
+        for key in keys[:usable]:
             page = self.prefixes.get(key)
             if page is None:
                 break
@@ -144,15 +154,26 @@ class PagePool:
             self._use(page)
         return [page for _, page in found]
 
-    def publish(self, tokens, computed, table, namespace="local"):
-        """Enter the full blocks of TOKENS[:COMPUTED] (pages TABLE[i]) that the index does not know yet."""
+    def publish(self, tokens, computed, table, namespace="local", keys=None):
+        """Enter the full blocks of TOKENS[:COMPUTED] (pages TABLE[i]) that the index does not know yet.
+        KEYS: the block keys of TOKENS[:COMPUTED], if the caller has them.
+
+        The whole chain is re-aged, deepest block first and root last, whether its blocks are new to the
+        index or not: a prompt that is published portion by portion would otherwise leave its root the
+        oldest entry, and one eviction would cut every deeper block off.
+        """
         if not self.prefix_cache:
             return
-        fresh = [(key, table[i]) for i, key in enumerate(block_keys(tokens[:computed], self.page_size, namespace))
-                 if key not in self.prefixes and table[i] >= 0]
-        for key, page in reversed(fresh):
-            self.prefixes[key] = page
-            self._use(page)
+        blocks = int(computed) // self.page_size
+        if keys is None:
+            keys = block_keys(tokens[:blocks * self.page_size], self.page_size, namespace)
+        for i in range(min(blocks, len(keys)) - 1, -1, -1):
+            key = keys[i]
+            if key in self.prefixes:
+                self.prefixes.move_to_end(key)
+            elif table[i] >= 0:
+                self.prefixes[key] = table[i]
+                self._use(table[i])
 
     def clear_prefixes(self):
         while self.prefixes:

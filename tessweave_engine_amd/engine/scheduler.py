@@ -308,7 +308,7 @@ class Engine:
                 continue
             whole = min(r.computed, len(r.prompt)) // page * page
             if whole > r.published:
-                self.cache.publish(r.seq, r.prompt[:whole], r.namespace, computed=whole)
+                self.cache.publish(r.seq, r.prompt, r.namespace, computed=whole)    # hashes only the new blocks
                 r.published = whole
 
     def _sampling_stream(self):

@@ -5,6 +5,7 @@ import pytest
 
 from tessweave_engine_amd.cache import (CacheLayout, CacheManager, CacheNeed, CapacityError, FixedState, PagedKV,
                                         PagePool)
+from tessweave_engine_amd.cache.pages import block_keys
 
 
 def full_layout(layers=2):
@@ -48,6 +49,73 @@ def test_prefix_keys_full_blocks_namespaces_and_last_token():
     t2 = off.allocate(3)
     off.publish(tokens, 9, t2)
     assert off.acquire_prefix(tokens) == [] and not off.prefixes
+
+
+def test_a_chain_published_portion_by_portion_is_still_eaten_from_its_tail():
+    """The scheduler offers a prompt's blocks as its portions are issued, root first. The root must not
+    be left the oldest entry: one eviction would then cut off every deeper block while they still hold pages."""
+    tokens = [1, 2, 3, 4, 5, 6]
+    p = PagePool(5, 2)
+    a = p.allocate(3)
+    for upto in (2, 4, 6):
+        p.publish(tokens, upto, a)
+    p.release(a)
+    assert list(p.prefixes.values()) == [a[2], a[1], a[0]]          # deepest oldest, root youngest
+    got = p.allocate(3)                                             # two pages are free, one must be evicted
+    assert p.evictions == 1 and a[2] in got
+    assert p.acquire_prefix(tokens + [7]) == a[:2]                  # what is left is reachable from the root
+    # a block that a second request publishes again (same tokens) re-ages the chain, it does not duplicate it
+    q = PagePool(6, 2)
+    a = q.allocate(3)
+    q.publish(tokens, 6, a)
+    b = q.allocate(1)
+    q.publish([9, 9], 2, b)
+    q.publish(tokens, 4, a)                                         # the chain's first two blocks are young again
+    q.release(a + b)
+    assert list(q.prefixes.values()) == [a[2], b[0], a[1], a[0]]
+    q.check()
+
+
+def test_block_keys_go_on_from_known_keys_and_keep_the_format():
+    import hashlib, struct
+    tokens = list(range(100, 123))
+    whole = block_keys(tokens, 4, "ns")
+    assert len(whole) == 5
+    root = hashlib.sha256(b"ns").digest()                           # flow_engine/cache.py:60-65
+    first = hashlib.sha256(root + struct.pack("<4q", *tokens[:4])).digest()
+    assert whole[0] == first
+    assert whole[1] == hashlib.sha256(first + struct.pack("<4q", *tokens[4:8])).digest()
+    assert block_keys(tokens, 4, "ns", known=whole[:2]) == whole
+    assert block_keys(tokens[:9], 4, "ns", known=whole) == whole[:2]      # more known than asked for
+    assert block_keys(tokens, 4, "other") != whole
+    assert block_keys([-1, 5, 2 ** 40, 0], 4, "ns")[0] == hashlib.sha256(root + struct.pack("<4q", -1, 5, 2 ** 40, 0)).digest()
+
+
+def test_manager_hashes_each_block_of_a_request_once(monkeypatch):
+    import tessweave_engine_amd.cache.manager as manager_module
+    hashed = []
+    real = manager_module.block_keys
+
+    def counting(tokens, page_size, namespace, known=()):
+        hashed.append(len(tokens) // page_size - min(len(known), len(tokens) // page_size))
+        return real(tokens, page_size, namespace, known)
+
+    monkeypatch.setattr(manager_module, "block_keys", counting)
+    m = CacheManager(full_layout(), page_size=4, pages=16, max_requests=2, max_request_tokens=64)
+    prompt = list(range(40))
+    a = m.open("a")
+    assert m.acquire_prefix(a, prompt) == 0                         # hashes the 9 blocks a lookup may use
+    for upto in (8, 16, 24, 40):
+        m.ensure(a, upto)
+        m.advance(a, upto)
+        m.publish(a, prompt, computed=upto)
+    m.publish(a, prompt + [1, 2, 3, 4], computed=40)                # the finished sequence: nothing new below 40
+    assert sum(hashed) == 10                                        # 40 tokens, 10 blocks, each hashed once
+    b = m.open("b")
+    assert m.acquire_prefix(b, prompt) == 36
+    assert m.acquire_prefix(b, prompt) == 0                         # a request that holds pages takes no more
+    m.close(a), m.close(b)
+    m.check()
 
 
 def test_eviction_takes_unused_entries_oldest_first_and_a_chain_from_its_tail():
