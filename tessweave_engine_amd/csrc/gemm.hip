@@ -420,13 +420,14 @@ extern "C" int tw_linear_partial_splits(int dtype, int N, int K) {
   return skinny_lds_splits(N, K, epf);
 }
 
-// The same for M rows: up to 64 rows the streaming kernel's ranges; above, those of the tiled kernels
-// (0 where they would not split K: the product with its epilogue is then the better call).
-extern "C" int tw_linear_partial_splits_rows(int dtype, int shuffled, int M, int N, int K) {
+// The same for M rows whose stride is LDA elements: up to 64 rows the streaming kernel's ranges; above,
+// those of the tiled kernels (0 where they would not split K: the product with its epilogue is then the
+// better call). Which tiled kernel runs, and so how it splits, depends on the rows' stride too.
+extern "C" int tw_linear_partial_splits_rows(int dtype, int shuffled, int M, int N, int K, long lda) {
   if (M <= 64) return tw_linear_partial_splits(dtype, N, K);
   const int epf = dtype == TW_DTYPE_F32 ? 4 : 8;
-  if (K % epf) return 0;
-  const int splits = tw_tiled_partial_splits(dtype, shuffled, K, M, N, K);
+  if (K % epf || lda < K) return 0;
+  const int splits = tw_tiled_partial_splits(dtype, shuffled, lda, M, N, K);
   return splits > 1 ? splits : 0;
 }
 

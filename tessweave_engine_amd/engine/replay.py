@@ -33,9 +33,19 @@ def parse_args(argv=None):
     p.add_argument("--out", required=True, help="folder for <step>.f32 files")
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at once (each rounded up to a multiple of 64)")
-    p.add_argument("--page-size", type=int, default=PAGE_SIZE, help="tokens per cache page (divides 64)")
+    p.add_argument("--page-size", type=int, default=PAGE_SIZE,
+                   help="tokens per cache page: any size the engine takes (a multiple of 4)")
     p.add_argument("--no-graphs", action="store_true", help="never replay decode steps from HIP graphs")
     return p.parse_args(argv)
+
+
+def pool_pages(max_tokens, page_size):
+    """Pages that hold MAX_TOKENS tokens of live requests, each request's count rounded up to a multiple of 64
+    (of the page size, if that is larger): every 64 tokens of a request lie in at most ceil(64 / page) pages of
+    its own, whatever the page size, so a page size that does not divide 64 gets the few pages more it needs."""
+    if page_size >= 64:
+        return math.ceil(max_tokens / page_size)
+    return math.ceil(max_tokens / 64) * math.ceil(64 / page_size)
 
 
 def run(args, lines, out=sys.stdout):
@@ -45,14 +55,14 @@ def run(args, lines, out=sys.stdout):
     from ..weights import load_model
     from .step import StepEntry, Stepper
 
-    if args.max_tokens <= 0 or args.page_size <= 0 or 64 % args.page_size:
-        raise SystemExit("--max-tokens must be positive and --page-size must divide 64")
+    if args.max_tokens <= 0 or args.page_size <= 0 or args.page_size % 4:
+        raise SystemExit("--max-tokens must be positive and --page-size a positive multiple of 4")
     if not torch.cuda.is_available():
         raise SystemExit("trace_run needs a GPU: there is no CPU path")
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
     model = load_model(args.model, dtype=args.dtype, device="cuda:0")
-    pages = math.ceil(args.max_tokens / args.page_size)
+    pages = pool_pages(args.max_tokens, args.page_size)
     cache = CacheManager(model.cache_layout(), args.page_size, pages, MAX_LIVE_REQUESTS, dtype=args.dtype,
                          device=model.device, prefix_cache=False,
                          max_request_tokens=pages * args.page_size)

@@ -19,6 +19,7 @@ launches of a 2,048-token engine.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 import ctypes
 from dataclasses import dataclass, field
 
@@ -42,17 +43,23 @@ def _round_up(v, m):
 
 GRAPH_SEGMENT_RUNS = 8       # layer runs per captured graph after the first
 MIN_LENGTH_CLASS = 512       # steps whose longest sequence is shorter share one captured graph
+MAX_GRAPHS = 96              # captured steps kept (one per batch size and length class met); the least recently
+                             # replayed one goes first
 
 
 class _Graph:
-    """A captured decode step: several graphs launched one after the other (see Stepper._capture)."""
+    """A captured decode step: several graphs launched one after the other (see Stepper._capture).
 
-    def __init__(self, handles, logits, generation):
-        self.handles, self.logits, self.generation = handles, logits, generation
+    BUFFERS names the scratch buffers whose addresses the capture holds, each with its version at the
+    time: the capture stays good until one of THOSE is allocated anew (a larger prompt portion growing a
+    buffer that only prompt portions use leaves every captured decode step alone)."""
+
+    def __init__(self, handles, logits, generation, buffers):
+        self.handles, self.logits, self.generation, self.buffers = handles, logits, generation, buffers
 
 
 class Stepper:
-    def __init__(self, model, cache, max_step_tokens=256, max_step_seqs=None, use_graphs=True):
+    def __init__(self, model, cache, max_step_tokens=256, max_step_seqs=None, use_graphs=True, max_graphs=MAX_GRAPHS):
         if model.device is None or model.device.type != "cuda":
             raise RuntimeError("the model's weights must be on a GPU: there is no CPU path")
         self.model = model
@@ -65,8 +72,9 @@ class Stepper:
         self._defer_sums = bool(getattr(model, "defers_sums", False))
         self.max_tokens = 0
         self.max_seqs = 0
-        self._graphs = {}
+        self._graphs = OrderedDict()     # (batch size, length class) -> _Graph, least recently replayed first
         self._warm = set()
+        self.max_graphs = max(1, int(max_graphs))
         self.token_feed = None
         self.segment_graphs = True
         self._staging = []
@@ -117,8 +125,16 @@ class Stepper:
             for graph in self._graphs.values():
                 for handle in graph.handles:
                     lib.tw_graph_destroy(handle)
-        self._graphs = {}
+        self._graphs = OrderedDict()
         self._warm = set()
+
+    def _drop_graph(self, key):
+        """Destroy one captured step (it may still be running: wait for the step's stream first)."""
+        graph = self._graphs.pop(key)
+        self.stream.synchronize()
+        lib = library()
+        for handle in graph.handles:
+            lib.tw_graph_destroy(handle)
 
     def close(self):
         self._drop_graphs()
@@ -319,6 +335,7 @@ class Stepper:
 
         check(lib.tw_graph_begin(stream), "graph capture begin")
         ctx.segment_end = segment_end
+        self.workspace.touched = touched = set()
         try:
             logits = self.model.forward(ctx)
         except BaseException:
@@ -328,25 +345,34 @@ class Stepper:
             raise
         finally:
             ctx.segment_end = None
+            self.workspace.touched = None
         check(end_segment(), "graph capture end")
         if self.workspace.generation != generation:
             for handle in handles:
                 lib.tw_graph_destroy(handle)
             raise RuntimeError("a scratch buffer was allocated during graph capture")
-        return _Graph(handles, logits, generation)
+        return _Graph(handles, logits, generation, {key: self.workspace.versions[key] for key in touched})
 
     def _run_graphable(self, ctx, key):
         """KEY = (batch size, length class) names the captured graph this step can be replayed from."""
         graph = self._graphs.get(key)
         if graph is not None and graph.generation != self.workspace.generation:
-            self._drop_graphs()
-            graph = None
+            # some scratch buffer was allocated since: only a capture that holds THAT buffer's address is stale
+            if self.workspace.holds(graph.buffers):
+                graph.generation = self.workspace.generation
+            else:
+                self._drop_graph(key)
+                graph = None
         if graph is None:
             if key not in self._warm:
                 # First time at this batch size and length class: run eagerly so every scratch buffer exists.
                 self._warm.add(key)
                 return self.model.forward(ctx)
             graph = self._graphs[key] = self._capture(ctx)
+            while len(self._graphs) > self.max_graphs:
+                self._drop_graph(next(iter(self._graphs)))
+        else:
+            self._graphs.move_to_end(key)
         lib = library()
         for handle in graph.handles:
             check(lib.tw_graph_launch(handle, self.stream.cuda_stream), "graph launch")

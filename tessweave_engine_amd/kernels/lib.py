@@ -25,7 +25,7 @@ _SIGNATURES = {
     "tw_silu_mul": (I, [I, P, P, I, I, P]),
     "tw_linear_workspace_bytes": (L, [I, I, I, I]),
     "tw_linear_partial_splits": (I, [I, I, I]),
-    "tw_linear_partial_splits_rows": (I, [I, I, I, I, I]),
+    "tw_linear_partial_splits_rows": (I, [I, I, I, I, I, L]),
     "tw_linear_partials": (I, [I, P, L, P, L, I, P, L, I, I, I, P]),
     "tw_linear_glu": (I, [I, P, L, P, L, I, P, P, L, I, I, I, I, P]),
     "tw_linear": (I, [I, I, P, L, P, L, I, P, P, L, P, L, P, L, I, I, I, I, P]),

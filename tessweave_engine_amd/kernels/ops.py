@@ -226,11 +226,13 @@ def linear_partial_splits(dtype, n, k):
     return int(library().tw_linear_partial_splits(dtype_id(dtype), int(n), int(k)))
 
 
-def linear_partial_splits_rows(weight, rows):
-    """K ranges `linear_partials` uses for ROWS rows against WEIGHT; 0 where it cannot or would not split
-    (above 64 rows the tiled kernels decide, and split only where whole tiles would leave CUs idle)."""
+def linear_partial_splits_rows(weight, rows, lda=None):
+    """K ranges `linear_partials` uses for ROWS rows (LDA elements apart, default: contiguous) against WEIGHT;
+    0 where it cannot or would not split (above 64 rows the tiled kernels decide, and split only where whole
+    tiles would leave CUs idle; which of them runs depends on the rows' stride too)."""
     n, k, _, _, shuffled, w_dtype = _weight_args(weight)
-    return int(library().tw_linear_partial_splits_rows(dtype_id(w_dtype), shuffled, int(rows), n, k))
+    return int(library().tw_linear_partial_splits_rows(dtype_id(w_dtype), shuffled, int(rows), n, k,
+                                                       int(lda if lda is not None else k)))
 
 
 def linear_partials(x, weight, partial):
@@ -243,7 +245,7 @@ def linear_partials(x, weight, partial):
     n, k, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
     _need(kx == k, "linear_partials shapes do not agree")
     _need(x.dtype == w_dtype and m >= 1, "linear_partials takes rows of the weight's type")
-    splits = linear_partial_splits_rows(weight, m)
+    splits = linear_partial_splits_rows(weight, m, lda)
     _need(splits > 0, "linear_partials: K must be a multiple of 16 bytes, and above 64 rows the shape must be one the tiled kernels split")
     _need(partial.is_contiguous() and tuple(partial.shape) == (splits, m, n), f"partial must be [{splits}, {m}, {n}]")
     check(library().tw_linear_partials(dtype_id(x.dtype), _dev(x), lda, w_ptr, ldw, shuffled,

@@ -120,7 +120,9 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self.buffers = {}
-        self.generation = 0          # changes whenever a buffer is (re)allocated
+        self.generation = 0          # changes whenever any buffer is (re)allocated
+        self.versions = {}           # per buffer: how often it has been (re)allocated
+        self.touched = None          # while a set: the buffers asked for (a graph capture notes whose addresses it holds)
 
     def get(self, tag, shape, dtype, capacity=None):
         """A tensor of SHAPE; the buffer behind it holds CAPACITY rows (default: shape[0])."""
@@ -129,12 +131,19 @@ class Workspace:
         per_row = math.prod(shape[1:]) if shape else 1
         want = max(numel, per_row * max(capacity or 0, shape[0] if shape else 1), 1)
         key = (tag, dtype)
+        if self.touched is not None:
+            self.touched.add(key)
         buf = self.buffers.get(key)
         if buf is None or buf.numel() < numel:
             buf = torch.empty(want, dtype=dtype, device=self.device)
             self.buffers[key] = buf
+            self.versions[key] = self.versions.get(key, 0) + 1
             self.generation += 1
         return buf[:numel].view(shape)
+
+    def holds(self, versions):
+        """Are the buffers named in VERSIONS ({key: version}) still the allocations they were then?"""
+        return all(self.versions.get(key) == version for key, version in versions.items())
 
     def bytes(self):
         return sum(b.numel() * b.element_size() for b in self.buffers.values())

@@ -123,20 +123,23 @@ class Linear(Part):
             else:
                 # few tiles for the chip (a few hundred rows, or large tiles against a matrix with few
                 # columns and a long K): the tiled kernel splits K too
+                # (a buffer of its own: growing with a prompt portion, it must not move the one captured decode steps hold)
                 floats = ops.linear_workspace_bytes(w.dtype, x.shape[0], rows, w.shape[1]) // 4
                 if floats:
-                    ws = ctx.workspace.get("linear.splitk", (floats,), torch.float32)
+                    ws = ctx.workspace.get("linear.splitk.rows", (floats,), torch.float32)
             ops.linear(x, w, target, bias=self.biases[i] if self.biases else None, residual=res, workspace=ws)
             col += rows
         return out
 
     # ---- leave the split-K sums to the next kernel -------------------------------------------
-    def _partial_splits(self, n_rows):
-        """K ranges of `forward_partials` for N_ROWS rows (0: none). Up to 64 rows the streaming kernel's
-        ranges depend on the matrix alone; above, the tiled kernels choose them per row count."""
-        key = ("splits", 64 if n_rows <= 64 else n_rows)
+    def _partial_splits(self, n_rows, lda=None):
+        """K ranges of `forward_partials` for N_ROWS rows, LDA elements apart (default: contiguous); 0: none.
+        Up to 64 rows the streaming kernel's ranges depend on the matrix alone; above, the tiled kernels
+        choose them per row count and stride."""
+        lda = self.weights[0].shape[1] if lda is None else int(lda)
+        key = ("splits", 64 if n_rows <= 64 else n_rows, lda)
         if key not in self._ws_floats:
-            self._ws_floats[key] = ops.linear_partial_splits_rows(self.weights[0], n_rows)
+            self._ws_floats[key] = ops.linear_partial_splits_rows(self.weights[0], n_rows, lda)
         return self._ws_floats[key]
 
     def deferrable(self, n_rows):
@@ -151,7 +154,7 @@ class Linear(Part):
         """float32 [splits, n, out] partial sums of x @ W.T (bias NOT added); see ops.linear_partials."""
         w = self.weights[0]
         n = x.shape[0]
-        splits = self._partial_splits(n)
+        splits = self._partial_splits(n, x.stride(0) if n > 1 else None)
         if n <= 64:     # sized once for the largest such batch, so that it never regrows under a captured graph
             buf = ctx.workspace.get("linear.partial." + tag, (splits, 64, w.shape[0]), torch.float32)
         else:

@@ -114,12 +114,14 @@ def long_model(tmp_path_factory, device):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n_req", [40, 64])
-def test_a_decode_batch_of_40_and_of_64_requests_short_and_long_from_graphs(long_model, dtype, n_req):
+@pytest.mark.parametrize("n_req", [40, 64, 65, 128])
+def test_decode_batches_of_40_to_128_requests_short_and_long_from_graphs(long_model, dtype, n_req):
     """An engine opened for 4,224 tokens a request: the captured decode step sizes its key ranges by the
     length class, and the batch holds requests of 3 to 4,100 tokens. Six decode steps (one eager, one captured,
-    four replayed) of 40 requests (the streaming matrix kernel's 48-row form) and of 64 (its 64-row form, the
-    benchmark's), every logits row against the plain implementation."""
+    four replayed) of 40 requests (the streaming matrix kernel's 48-row form), of 64 (its 64-row form, the
+    benchmark's), and of 65 and 128 (single tokens through the tiled matrix kernels, which take over above 64
+    rows, where the projections also stop leaving their sums to the next kernel), every logits row against the
+    plain implementation."""
     from tessweave_engine_amd.cache import CacheManager
     from tessweave_engine_amd.engine import StepEntry, Stepper
     from tessweave_engine_amd.weights import load_model
@@ -272,6 +274,65 @@ def test_decoding_across_a_length_class_takes_a_second_graph_and_changes_nothing
                 assert float((got[r] - w).abs().max()) <= 0.02 * float(w.abs().max()), (i, pos)
     assert sorted(stepper._graphs) == [(2, 512), (2, 1024)]
     assert stepper.graph_replays == 30 - 2                 # the first step of each class runs eagerly, the next is captured
+    stepper.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_steps_are_bounded_and_outlive_a_larger_prompt_portion(long_model, dtype):
+    """The table of captured decode steps keeps at most `max_graphs` entries (the least recently replayed one
+    goes first and is captured again when its batch size returns), and a prompt portion that grows a scratch
+    buffer which only portions use leaves the captured decode steps alone. Every decode row is compared."""
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.weights import load_model
+    page, vocab = long_model["page"], long_model["cfg"]["vocab_size"]
+    g = torch.Generator().manual_seed(96)
+    tokens = [torch.randint(0, vocab, (n,), generator=g).tolist() for n in (70, 45, 52, 400)]
+    want = [plain.forward(long_model["config"], long_model["weights"], t) for t in tokens]
+    model = load_model(long_model["folder"], dtype=dtype, device="cuda:0")
+    cache = CacheManager(model.cache_layout(), page, 64, 4, dtype=dtype, device=model.device, prefix_cache=False,
+                         max_request_tokens=1024)
+    stepper = Stepper(model, cache, max_step_tokens=512, max_step_seqs=4, max_graphs=2)
+    seqs = [cache.open(i) for i in range(4)]
+    at = [30, 20, 25]
+    stepper.step([StepEntry(seqs[i], tokens[i][:at[i]], []) for i in range(3)])
+
+    def decode(live):
+        got = stepper.step([StepEntry(seqs[i], [tokens[i][at[i]]], [0]) for i in live]).cpu()
+        for r, i in enumerate(live):
+            w = want[i][at[i]]
+            if dtype == "float32":
+                assert torch.allclose(got[r], w, atol=5e-6, rtol=2e-5), (live, i, at[i])
+            else:
+                assert float((got[r] - w).abs().max()) <= 0.02 * float(w.abs().max()), (live, i, at[i])
+            at[i] += 1
+
+    for live in ([0, 1, 2], [0, 1], [2]):                       # three batch sizes, room for two captures
+        for _ in range(3):
+            decode(live)
+    assert list(stepper._graphs) == [(2, 512), (1, 512)]
+    kept = stepper._graphs[(1, 512)]
+    # a prompt portion larger than any before: scratch buffers of its own may grow, the captured steps stay
+    generation = stepper.workspace.generation
+    got = stepper.step([StepEntry(seqs[3], tokens[3][:333], [332])]).cpu()
+    assert float((got[0] - want[3][332]).abs().max()) <= (1e-4 if dtype == "float32" else 0.02 * float(want[3][332].abs().max()))
+    stepper.workspace.get("a buffer no captured step holds", (1 << 16,), torch.float32)
+    assert stepper.workspace.generation != generation
+    replays = stepper.graph_replays
+    decode([2])
+    assert stepper._graphs[(1, 512)] is kept and stepper.graph_replays == replays + 1
+    # a buffer that the captured step does hold is allocated anew: that capture is stale and is made again
+    (tag, buffer_dtype), _ = next(iter(kept.buffers.items()))
+    stepper.workspace.get(tag, (stepper.workspace.buffers[tag, buffer_dtype].numel() + 64,), buffer_dtype)
+    decode([2])
+    assert stepper._graphs[(1, 512)] is not kept and list(stepper._graphs) == [(2, 512), (1, 512)]
+    decode([2])
+    for _ in range(3):
+        decode([0, 1, 2])                                       # evicted before: warm already, so captured at once
+    assert list(stepper._graphs) == [(1, 512), (3, 512)]
+    decode([0, 1])
+    decode([0, 1])
+    assert list(stepper._graphs) == [(3, 512), (2, 512)]
     stepper.close()
 
 

@@ -88,7 +88,8 @@ def test_rmsnorm(ops, device, dtype, hidden, eps):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("q_heads,kv_heads,head_dim,page,theta", [(4, 2, 16, 16, 1e4), (6, 1, 32, 8, 1e6), (5, 5, 48, 4, 5e5),
-                                                                 (3, 1, 20, 8, 1e4), (28, 4, 128, 16, 1e6)])
+                                                                 (3, 1, 20, 8, 1e4), (28, 4, 128, 16, 1e6),
+                                                                 (4, 2, 32, 12, 1e4), (2, 1, 64, 24, 1e6), (3, 3, 16, 48, 1e4)])
 def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, page, theta):
     n, pages = 9, 7
     width = (q_heads + 2 * kv_heads) * head_dim
@@ -155,7 +156,8 @@ def test_rope_and_cache_write(ops, device, dtype, q_heads, kv_heads, head_dim, p
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("kv_heads,head_dim,page", [(2, 32, 16), (4, 128, 16), (1, 64, 8), (3, 48, 32), (2, 32, 4)])
+@pytest.mark.parametrize("kv_heads,head_dim,page", [(2, 32, 16), (4, 128, 16), (1, 64, 8), (3, 48, 32), (2, 32, 4),
+                                                    (2, 32, 12), (1, 64, 24), (2, 16, 48), (1, 128, 20)])
 def test_cache_write_of_tokens_with_consecutive_slots(ops, device, dtype, kv_heads, head_dim, page):
     """A prompt portion holds consecutive slots: aligned groups of them write the transposed value pages
     together. Runs that start and end anywhere, a gap, a row that writes nothing and rows in other pages
@@ -374,20 +376,22 @@ def test_linear_partials_of_many_rows(ops, device, dtype, m, n, k):
     want = (x.double() @ w.double().T).cpu()
     scale = math.sqrt(k) * 0.05
     seen = 0
-    for weight in (w, ops.shuffle_weight(w)):
-        splits = ops.linear_partial_splits_rows(weight, m)
+    wide = torch.zeros(m, k + 48, dtype=dtype, device=device)      # the same rows, 48 elements further apart
+    wide[:, :k] = x
+    for weight, rows in ((w, x), (ops.shuffle_weight(w), x), (ops.shuffle_weight(w), wide[:, :k])):
+        splits = ops.linear_partial_splits_rows(weight, m, rows.stride(0))
         if splits == 0:
             with pytest.raises(ValueError, match="linear_partials"):
-                ops.linear_partials(x, weight, torch.empty(1, m, n, device=device))
+                ops.linear_partials(rows, weight, torch.empty(1, m, n, device=device))
             continue
         assert splits >= 2
         seen += 1
         part = torch.full((splits, m, n), float("nan"), device=device)
-        ops.linear_partials(x, weight, part)
+        ops.linear_partials(rows, weight, part)
         torch.testing.assert_close(part.double().sum(0).cpu(), want, atol=3e-5 * scale, rtol=1e-5)
         assert part.abs().amax(dim=(1, 2)).min() > 0             # every range did its share
         with pytest.raises(ValueError, match="partial must be"):
-            ops.linear_partials(x, weight, torch.empty(splits + 1, m, n, device=device))
+            ops.linear_partials(rows, weight, torch.empty(splits + 1, m, n, device=device))
     assert seen or (m, n, k) == (2048, 4096, 512)                # (many tiles, short K: nothing to split)
 
 
@@ -520,7 +524,8 @@ def test_attn_reference_vector_tables(ops, device, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,head_dim,page", [(4, 2, 16, 16), (6, 1, 32, 8), (28, 4, 128, 16), (5, 5, 48, 4)])
+@pytest.mark.parametrize("heads,kv_heads,head_dim,page", [(4, 2, 16, 16), (6, 1, 32, 8), (28, 4, 128, 16), (5, 5, 48, 4),
+                                                          (4, 2, 32, 12), (6, 3, 64, 24), (2, 1, 128, 48)])
 @pytest.mark.parametrize("window", [0, 9])
 def test_attn_prefill_portions(ops, device, dtype, heads, kv_heads, head_dim, page, window):
     """Portions of prompts at any offset: the query rows are the LAST q_len positions of kv_len keys."""
@@ -587,7 +592,7 @@ def test_attn_far_key_among_hundreds(ops, device):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("page,window", [(16, 0), (8, 0), (64, 0), (16, 70), (4, 33)])
+@pytest.mark.parametrize("page,window", [(16, 0), (8, 0), (64, 0), (16, 70), (4, 33), (12, 0), (24, 70), (48, 0), (20, 33)])
 def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
     """Each head's query points at ONE key that sits on an edge (of a page, of a 32-key block, of a split,
     of the window, of the sequence): a kernel that drops, doubles or misplaces that key is wrong by O(1),

@@ -24,20 +24,21 @@ from tiny_configs import TINY, make_folder
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
 
-LENGTHS = {"A": [37, 49, 70, 33, 64, 40], "B": [33, 41, 64, 100, 124, 35, 50], "C": [36, 65, 97, 130, 34, 48]}
+LENGTHS = {"A": [37, 49, 70, 33, 64, 40], "B": [33, 41, 64, 100, 124, 35, 50], "C": [36, 65, 97, 130, 34, 48],
+           "B320": [33, 41, 64, 100, 124, 35, 50]}
 
 
 def round64(n):
     return (n + 63) // 64 * 64
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "B320"])
 def tiny(request, tmp_path_factory, device):
     name = request.param
     folder = tmp_path_factory.mktemp(f"tiny{name}")
     cfg, page = make_folder(folder, name)
     config, weights = plain.read_folder(folder)
-    g = torch.Generator().manual_seed(100 + len(name) + ord(name))
+    g = torch.Generator().manual_seed(100 + len(name) + ord(name[0]))
     requests = {f"r{i}": torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist()
                 for i, n in enumerate(LENGTHS[name])}
     want = {rid: plain.forward(config, weights, toks).numpy() for rid, toks in requests.items()}
@@ -210,6 +211,21 @@ def test_mixed_with_few_pages(tiny, dtype, seed, tmp_path):
     assert peak < total                                       # the pool is smaller than all requests: pages are reused
     got = run_trace(tiny, dtype, steps, peak, tmp_path)
     compare(tiny, dtype, steps, got, starts)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page", [12, 24, 48, 20])
+def test_pages_whose_size_is_no_power_of_two(tiny, dtype, page, tmp_path):
+    """Every multiple of 4 is a page size the engine takes; the fast bfloat16 attention kernels want powers of
+    two, so these run the kernels that divide by the page size: mixed with few pages, and the last 32 one by one."""
+    other = dict(tiny, page=page)
+    steps, starts, peak = mixed_trace(other, 3)
+    got = run_trace(other, dtype, steps, peak, tmp_path / "mixed")
+    compare(other, dtype, steps, got, starts)
+    steps, starts = sequential(other, lambda t: ([t - 32] if t > 32 else []) + [1] * min(t, 32))
+    biggest = max(round64(len(t)) for t in other["requests"].values())
+    got = run_trace(other, dtype, steps, biggest, tmp_path / "single")
+    compare(other, dtype, steps, got, starts)
 
 
 def test_ways_of_cutting_agree_beyond_rounding(tiny, tmp_path):

@@ -23,8 +23,12 @@ TINY_C = dict(
     tie_word_embeddings=False, use_sliding_window=False, max_position_embeddings=1024, hidden_act="silu")
 TINY_C_PAGE, TINY_C_SEED = 32, 2
 
+# B with the intermediate size 320 (a multiple of 16: gate and up rows interleave and the SiLU-multiply runs in
+# the matrix kernel's epilogue, where B's 328 takes the separate kernel)
+TINY_B320 = dict(TINY_B, intermediate_size=320)
+
 TINY = {"A": (TINY_A, TINY_A_PAGE, TINY_A_SEED), "B": (TINY_B, TINY_B_PAGE, TINY_B_SEED),
-        "C": (TINY_C, TINY_C_PAGE, TINY_C_SEED)}
+        "C": (TINY_C, TINY_C_PAGE, TINY_C_SEED), "B320": (TINY_B320, TINY_B_PAGE, TINY_B_SEED)}
 
 
 def make_folder(path, name):
