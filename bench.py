@@ -11,9 +11,10 @@ sampling on the device, commit), so the last timed step reads 4,096 keys per
 request. One JSON line is printed: decoded tokens a second, a 2,048-token
 prefill, the decode step's HBM roofline (against the nominal 8 TB/s and against
 what a plain streaming reader reaches on this device, measured in the same run),
-and further points: decode at batch 1 and 64 at the same context; the same batch
+the library's rate on the prefill's matrix products (`prefill.library_gemm_tflops`; `frac_of_library` is the
+whole step's rate against it), and further points: decode at batch 1, 16, 32 and 64 at the same context; the same batch
 of 8 with the engine opened for 32,768 tokens a request (`decode_b8_open32k`)
-and with requests of that length (`decode_b8_ctx32k`: the cache is then as large
+and with requests of 16,384 tokens and of that length (`decode_b8_ctx16k`, `decode_b8_ctx32k`: the cache is then as large
 as the weights; `prefill_32k_prompts`: tokens a second over those prompts, which
 go through in portions of 2,048); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
 (`gen512_b*`, decoded tokens a second over the generated part).
@@ -59,7 +60,7 @@ def parse():
     p.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all of them)")
     p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     p.add_argument("--prefill-tokens", type=int, default=2048)
-    p.add_argument("--points", default="1,64", help="further decode batch sizes to measure")
+    p.add_argument("--points", default="1,16,32,64", help="further decode batch sizes to measure")
     p.add_argument("--max-context", type=int, default=0,
                    help="tokens a request may hold, which the engine is opened for (0: the context + 1)")
     p.add_argument("--no-extra-points", action="store_true",
@@ -196,6 +197,34 @@ def read_ceiling(torch, device, gigabytes=4):
     return n / (best / 1000) / 1e9
 
 
+def library_matrix_rate(torch, c, rows, layers, device, repeats=5):
+    """TFLOP/s of the library's bfloat16 matrix product (hipBLASLt through torch.matmul) over the four projections
+    of a layer at ROWS rows, LAYERS distinct weight sets in turn (so that, as in the model, weights come from HBM and
+    not from a cache): the yardstick the prefill's own matrix kernels are measured against. Not on the product path."""
+    qkv = (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim
+    shapes = [(qkv, c.hidden_size), (c.hidden_size, c.num_attention_heads * c.head_dim),
+              (2 * c.intermediate_size, c.hidden_size), (c.hidden_size, c.intermediate_size)]
+    layers = max(1, min(layers, 4))
+    weights = [[torch.randn(n, k, device=device, dtype=torch.bfloat16) * 0.02 for n, k in shapes] for _ in range(layers)]
+    inputs = [torch.randn(rows, k, device=device, dtype=torch.bfloat16) for _, k in shapes]
+    flops = layers * sum(2.0 * rows * n * k for n, k in shapes)
+    best = None
+    for i in range(repeats + 1):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for layer in weights:
+            for x, w in zip(inputs, layer):
+                torch.matmul(x, w.t())
+        end.record()
+        torch.cuda.synchronize()
+        if i:
+            ms = start.elapsed_time(end)
+            best = ms if best is None else min(best, ms)
+    del weights, inputs
+    torch.cuda.empty_cache()
+    return flops / (best / 1000) / 1e12
+
+
 def prefill_run(model, torch, tokens, dtype, seed, repeats=3):
     from tessweave_engine_amd.cache import CacheManager
     from tessweave_engine_amd.engine import StepEntry, Stepper
@@ -257,7 +286,8 @@ def main():
     element = 2 if args.dtype == "bfloat16" else 4
     layer_weights = c.hidden_size * (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim \
         + c.num_attention_heads * c.head_dim * c.hidden_size + 3 * c.hidden_size * c.intermediate_size
-    weight_bytes = (c.num_hidden_layers * layer_weights + c.vocab_size * c.hidden_size) * element
+    weight_bytes = model.weight_bytes()          # what the model's parts say a step reads once in full
+    assert abs(weight_bytes / ((c.num_hidden_layers * layer_weights + c.vocab_size * c.hidden_size) * element) - 1) < 2e-3
     mean_ctx = args.context - args.steps / 2
     kv_bytes = args.batch * mean_ctx * c.kv_bytes_per_token(element)
     achieved = (weight_bytes + kv_bytes) / (ms_per_step / 1000) / 1e9
@@ -271,6 +301,10 @@ def main():
     linear_flops = 2.0 * t * c.num_hidden_layers * layer_weights + 2.0 * c.vocab_size * c.hidden_size
     attn_flops = c.num_hidden_layers * 4.0 * c.num_attention_heads * c.head_dim * (t * (t + 1) / 2)
     prefill_tflops = (linear_flops + attn_flops) / (prefill_ms / 1000) / 1e12
+
+    # the library's rate on the same matrix products, and the engine's own rate on them if every other kernel of the
+    # step took no time at all (a lower bound of what its matrix kernels reach)
+    library = library_matrix_rate(torch, c, t, c.num_hidden_layers, model.device) if args.dtype == "bfloat16" else None
 
     points = {}
     for b in [int(v) for v in args.points.split(",") if v]:
@@ -289,6 +323,10 @@ def main():
         for b in (1, 8, 64):
             tps, _, _, _ = decode_run(model, torch, b, 1024 + 512, 504, 8, args.dtype, use_graphs, args.seed, opened)
             points[f"gen512_b{b}"] = round(tps, 1)
+        # a batch of 8 at half that length
+        if opened >= 32768:
+            tps, _, _, _ = decode_run(model, torch, args.batch, 16384, 32, 8, args.dtype, use_graphs, args.seed, opened)
+            points[f"decode_b{args.batch}_ctx16k"] = round(tps, 1)
         # and with requests that really are that long: the cache is then as large as the weights
         tps, _, _, prompts_tps = decode_run(model, torch, args.batch, opened - 16, 32, 8, args.dtype, use_graphs, args.seed, opened)
         points[f"decode_b{args.batch}_ctx{opened // 1024}k"] = round(tps, 1)
@@ -311,7 +349,9 @@ def main():
                    "parallelism": "single GPU", "hip_graphs": bool(use_graphs and replays > 0),
                    "sampling": "greedy on device"},
         "prefill": {"value": round(t / (prefill_ms / 1000), 1), "tokens": t, "ms": round(prefill_ms, 3),
-                    "frac": round(prefill_tflops / PEAK_TFLOPS[args.dtype], 4)},
+                    "frac": round(prefill_tflops / PEAK_TFLOPS[args.dtype], 4),
+                    **({"library_gemm_tflops": round(library, 1), "frac_of_library": round(prefill_tflops / library, 4)}
+                       if library else {})},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "measured_read_ceiling": round(ceiling, 1),
                      "frac_of_measured": round(achieved / ceiling, 4)},

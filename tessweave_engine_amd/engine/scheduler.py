@@ -26,8 +26,14 @@ named by its row in the sampler's output and resolved on the device, and the hos
 reads and commits tokens one turn late, while the device already runs the next
 turn; the host's work between turns no longer leaves the device idle. A request
 that turns out to have ended (EOS) has then run one token too far: that token is
-dropped, and what it wrote lies beyond anything the prefix index publishes. The
-tokens a request gets are the same with and without lookahead.
+dropped, and what it wrote lies beyond anything the prefix index publishes.
+With and without lookahead a request's logits are the same up to rounding: in
+32-bit its tokens are the same; in bfloat16 a choice between two words whose
+logits lie within bfloat16's rounding of each other (or a draw that falls on
+the edge between two words) may go either way, because lookahead retires a
+request one turn later, so the same token can meet another batch (beside a
+prompt portion it runs through the tiled kernels, alone through the streaming
+ones, which sum in another order). The same holds for any two schedules.
 """
 from __future__ import annotations
 

@@ -35,6 +35,9 @@ class StepEntry:
     seq: object                      # cache.Sequence
     tokens: list                     # the request's next tokens (at least one)
     want: list = field(default_factory=list)   # indices into tokens whose logits are wanted
+    positions: object = None         # None: every position axis counts the request's tokens (computed, computed + 1, ...);
+                                     # else one list of len(tokens) position ids per axis of the model's encodings.
+                                     # The cache and the causal order go by token order, whatever the ids say.
 
 
 def _round_up(v, m):
@@ -70,6 +73,7 @@ class Stepper:
         self.stream = torch.cuda.Stream(device=self.device)
         self.use_graphs = bool(use_graphs) and model.graph_safe_model
         self._defer_sums = bool(getattr(model, "defers_sums", False))
+        self.position_axes = max(1, int(getattr(model, "position_axes", 1)))
         self.max_tokens = 0
         self.max_seqs = 0
         self._graphs = OrderedDict()     # (batch size, length class) -> _Graph, least recently replayed first
@@ -99,7 +103,7 @@ class Stepper:
             offset += _round_up(count, 64)
 
         add("token_ids", max_tokens)
-        add("positions", max_tokens)
+        add("positions", self.position_axes * max_tokens)
         add("q_start", max_seqs + 1)
         add("kv_len", max_seqs)
         add("state_slots", max_seqs)
@@ -211,6 +215,9 @@ class Stepper:
                 raise ValueError(f"request {e.seq.id!r}: token ids must be integers in [0, {vocab})")
             if any(type(w) is not int or w < 0 or w >= len(e.tokens) for w in e.want):
                 raise ValueError(f"request {e.seq.id!r}: wanted places must index this step's tokens")
+            if e.positions is not None and (len(e.positions) != self.position_axes
+                                            or any(len(axis) != len(e.tokens) for axis in e.positions)):
+                raise ValueError(f"request {e.seq.id!r}: positions must be {self.position_axes} lists of one id per token")
         n_tokens = sum(len(e.tokens) for e in entries)
         if n_tokens > self.max_tokens or len(entries) > self.max_seqs:
             self._reserve(max(self.max_tokens, _round_up(n_tokens, 256)), max(self.max_seqs, len(entries)))
@@ -250,7 +257,12 @@ class Stepper:
             host[off:off + len(values)] = values
 
         put("token_ids", token_ids)
-        put("positions", positions)
+        axes = self.position_axes
+        ids = np.tile(positions, (axes, 1))                      # [axes, n_tokens]; `positions` stays the token order
+        for s_index, e in enumerate(ordered):
+            if e.positions is not None:
+                ids[:, q_start[s_index]:q_start[s_index + 1]] = np.asarray(e.positions, dtype=np.int64)
+        put("positions", ids.reshape(-1))
         put("q_start", q_start)
         put("kv_len", kv_len)
         put("state_slots", slots_of)
@@ -272,7 +284,7 @@ class Stepper:
         ctx.device, ctx.dtype = self.device, self.dtype
         ctx.n_tokens, ctx.n_seqs, ctx.n_decode, ctx.n_logits = n_tokens, n_seqs, n_decode, n_logits
         ctx.token_ids = self._dev("token_ids", n_tokens)
-        ctx.positions = self._dev("positions", n_tokens)
+        ctx.positions = self._dev("positions", axes * n_tokens).view(axes, n_tokens)
         ctx.q_start = self._dev("q_start", n_seqs + 1)
         ctx.kv_len = self._dev("kv_len", n_seqs)
         ctx.state_slots = self._dev("state_slots", n_seqs)

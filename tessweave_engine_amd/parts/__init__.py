@@ -1,4 +1,4 @@
-from .base import (Block, FeedForward, GroupStep, LayerRun, Mixer, Norm, Part, PositionEncoding,
+from .base import (Block, FeedForward, GroupStep, HeadHook, LayerRun, Mixer, Norm, Part, PositionEncoding,
                    StepContext, Workspace, fold_pending)
 from .linear import Linear
 from .norms import RMSNorm
@@ -9,7 +9,7 @@ from .blocks import PreNormBlock
 from .embedding import OutputHead, TokenEmbedding
 from .model import DecoderModel, walk
 
-__all__ = ["Block", "FeedForward", "GroupStep", "LayerRun", "Mixer", "Norm", "Part", "PositionEncoding",
+__all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer", "Norm", "Part", "PositionEncoding",
            "StepContext", "Workspace", "fold_pending", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEmbedding",
            "GroupedQueryAttention", "SwiGLU", "PreNormBlock", "OutputHead", "TokenEmbedding",
            "DecoderModel", "walk"]

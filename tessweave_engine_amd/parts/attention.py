@@ -19,7 +19,11 @@ import torch
 
 class GroupedQueryAttention(Mixer):
     def __init__(self, prefix, hidden, q_heads, kv_heads, head_dim, position, qkv_bias=True,
-                 o_bias=False, window=None, scale=None, packed=True):
+                 o_bias=False, window=None, scale=None, packed=True, head_hook=None):
+        """head_hook: an optional `HeadHook` that changes the projected q, k, v (bias added) in place before q
+        and k are rotated: a per-head norm, a scaling. With a hook the projection is finished by its own
+        kernel first (without one, few-row steps leave its split-K sums to the kernel that adds the bias,
+        rotates and writes the cache)."""
         if q_heads % kv_heads:
             raise ValueError("q_heads must be a multiple of kv_heads")
         if head_dim % 2 or not 2 <= head_dim <= 256:
@@ -41,17 +45,21 @@ class GroupedQueryAttention(Mixer):
                           [q_heads * head_dim, kv_heads * head_dim, kv_heads * head_dim], bias=qkv_bias, packed=packed,
                           pad_out=pad)
         self.o = Linear([prefix + "o_proj"], q_heads * head_dim, [hidden], bias=o_bias, pad_in=pad)
+        self.head_hook = head_hook
 
     def parts(self):
-        return [self.qkv, self.o, self.position]
+        return [self.qkv, self.o, self.position] + ([self.head_hook] if self.head_hook is not None else [])
 
     def tensor_specs(self):
-        return self.qkv.tensor_specs() + self.o.tensor_specs()
+        hook = self.head_hook.tensor_specs() if self.head_hook is not None else []
+        return self.qkv.tensor_specs() + self.o.tensor_specs() + hook
 
     def bind(self, tensors, dtype, device):
         self.qkv.bind(tensors, dtype, device)
         self.o.bind(tensors, dtype, device)
         self.position.bind(tensors, dtype, device)     # shared by layers; binding again is harmless
+        if self.head_hook is not None:
+            self.head_hook.bind(tensors, dtype, device)
 
     def cache_need(self):
         return CacheNeed(paged=PagedKV(self.kv_heads, self.head_dim, self.window))
@@ -64,7 +72,7 @@ class GroupedQueryAttention(Mixer):
         adjacent = self.position.pairing == "adjacent"
         keys, values, g = ctx.cache.keys_values(run.cache_slot)
         group = ctx.groups[g]
-        if n <= 64 and self.qkv.deferrable(n):
+        if n <= 64 and self.head_hook is None and self.qkv.deferrable(n):
             # few rows: the projection leaves split-K sums; bias, rotation and cache write finish them
             partial = self.qkv.forward_partials(ctx, h, "qkv")
             ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
@@ -73,6 +81,8 @@ class GroupedQueryAttention(Mixer):
                               adjacent=adjacent)
         else:
             self.qkv.forward(ctx, h, qkv)
+            if self.head_hook is not None:
+                self.head_hook.forward(ctx, qkv)
             ops.rope_kv_write(qkv, cos, sin, group.slot_mapping, keys, values, self.q_heads, self.kv_heads,
                               self.head_dim, ctx.cache.page_size, write_cache=run.writes_cache, adjacent=adjacent)
         out = ctx.scratch("attn.out", (n, self.q_heads * self.head_dim))

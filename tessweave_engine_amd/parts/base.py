@@ -47,6 +47,13 @@ class Part:
         """Sub-parts, for walking a model."""
         return []
 
+    def weight_tensors(self):
+        """The tensors (torch tensors or kernel-layout weights with `numel()` and `element_size()`) of THIS part,
+        not of its sub-parts, that a step reads once in full: matrices, biases, norm weights. What a step only
+        gathers rows from (an embedding table) or derives constants from is not among them. The bytes a decode
+        step must move, and so its roofline, are counted from this."""
+        return []
+
 
 class Norm(Part):
     #: True if `forward` takes `add`: pending partial sums (float32 [splits, n, hidden]) that the part
@@ -70,8 +77,25 @@ class PositionEncoding(Part):
     #: which two elements of a head turn together: "half" pairs element j with j + rotary_dim/2,
     #: "adjacent" pairs element 2j with 2j + 1
     pairing = "half"
+    #: position ids a token carries for this encoding: `ctx.positions` is [axes, n_tokens] with as many axes as
+    #: the model's encodings ask for at most. Axis 0 counts a request's tokens unless a step entry brings
+    #: its own ids; an encoding with one axis reads `ctx.positions[0]`.
+    position_axes = 1
 
     def tables(self, ctx):
+        """(cos, sin), float32 [n_tokens, rotary_dim / 2] each, from `ctx.positions`."""
+        raise NotImplementedError
+
+
+class HeadHook(Part):
+    """An operation on a mixer's projected heads between bias and rotation (a per-head norm, a scaling).
+
+    `forward(ctx, qkv)` changes qkv [n_tokens, (q_heads + 2 kv_heads) * head_dim] in place, in the compute
+    type, on the current stream. The part gets the head counts and sizes it needs as constructor parameters,
+    as every part does (head_dim is the size on the device: a multiple of 16, tails of zeros stay zeros).
+    """
+
+    def forward(self, ctx, qkv):
         raise NotImplementedError
 
 
@@ -173,7 +197,8 @@ class StepContext:
         self.n_seqs = 0
         self.n_decode = 0
         self.token_ids = None        # int32 [n_tokens]
-        self.positions = None        # int32 [n_tokens]
+        self.positions = None        # int32 [position axes, n_tokens]; axis 0: the token's index in its request
+                                     # unless the step entry brought its own ids
         self.q_start = None          # int32 [n_seqs + 1]
         self.kv_len = None           # int32 [n_seqs], this step's tokens included
         self.state_slots = None      # int32 [n_seqs]

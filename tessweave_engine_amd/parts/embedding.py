@@ -54,6 +54,9 @@ class OutputHead(Part):
     def matrix(self):
         return self.weight
 
+    def weight_tensors(self):
+        return [self.weight]          # (the embedding's table is not listed by its part: a step gathers a few rows of it)
+
     def forward(self, ctx, h):
         # The logits live in a shared scratch buffer: they are valid until the next step.
         logits = ctx.workspace.get("logits", (h.shape[0], self.vocab), torch.float32)

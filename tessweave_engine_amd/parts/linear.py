@@ -90,6 +90,9 @@ class Linear(Part):
         self.biases = [b.contiguous() for b in biases]
         del weights, biases
 
+    def weight_tensors(self):
+        return list(self.weights) + list(self.biases)
+
     def weight_bytes(self):
         return sum(w.numel() * w.element_size() for w in self.weights)
 

@@ -4,7 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..cache.spec import CacheLayout
-from .base import LayerRun, Norm, Part
+from .base import LayerRun, Norm, Part, PositionEncoding
 from .blocks import normalise
 
 
@@ -67,19 +67,21 @@ class DecoderModel(Part):
             raise ValueError(f"tensors no part took: {sorted(leftover)[:12]}")
         return self
 
+    @property
+    def position_axes(self):
+        """Position ids per token that the step's metadata must carry: the most any of the model's encodings asks for."""
+        return max([p.position_axes for p in walk(self) if isinstance(p, PositionEncoding)] + [1])
+
     def weight_bytes(self):
-        """Bytes of every weight a step reads once (matrices and vectors)."""
+        """Bytes of every weight a step reads once in full: what the parts name in `weight_tensors()`, each
+        allocation counted once (layers may share a part, a tied head has a matrix of its own)."""
         total, seen = 0, set()
         for part in walk(self):
-            for value in vars(part).values():
-                items = value if isinstance(value, (list, tuple)) else [value]
-                for t in items:
-                    t = getattr(t, "data", t) if type(t).__name__ == "ShuffledWeight" else t
-                    if isinstance(t, torch.Tensor) and t.is_floating_point() and id(t) not in seen and t.dim() >= 1:
-                        if getattr(part, "inv_freq", None) is t:
-                            continue
-                        seen.add(id(t))
-                        total += t.numel() * t.element_size()
+            for t in part.weight_tensors():
+                ident = id(getattr(t, "data", t))
+                if ident not in seen:
+                    seen.add(ident)
+                    total += t.numel() * t.element_size()
         return total
 
     def cache_layout(self):

@@ -26,6 +26,9 @@ class RMSNorm(Norm):
     def bind(self, tensors, dtype, device):
         self.weight = tensors.pop(self.name + ".weight").contiguous()
 
+    def weight_tensors(self):
+        return [self.weight]
+
     def forward(self, ctx, x, rows=None, add=None):
         tag = "norm.out" if rows is None else "norm.rows"        # a model's last norm (chosen rows) keeps its own buffer
         n_out = rows.numel() if rows is not None else x.shape[0]

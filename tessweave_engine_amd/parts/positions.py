@@ -28,7 +28,7 @@ class RotaryEmbedding(PositionEncoding):
     def bind(self, tensors, dtype, device):
         rot = self.rotary_dim
         inv = self.theta ** (-torch.arange(0, rot, 2, dtype=torch.float32) / rot)
-        self.inv_freq = inv.to(device)
+        self.inv_freq = inv.to(device)          # a constant the tables are derived from, not a weight
 
     def tables(self, ctx):
         """(cos, sin), float32 [n_tokens, rotary_dim / 2], computed once per step."""
@@ -38,7 +38,7 @@ class RotaryEmbedding(PositionEncoding):
             half = self.rotary_dim // 2
             cos = ctx.scratch(f"rotary.cos.{id(self)}", (ctx.n_tokens, half), torch.float32)
             sin = ctx.scratch(f"rotary.sin.{id(self)}", (ctx.n_tokens, half), torch.float32)
-            ops.rope_table(ctx.positions, self.inv_freq, cos, sin)
+            ops.rope_table(ctx.positions[0], self.inv_freq, cos, sin)
             hit = ctx.shared[key] = (cos, sin)
         return hit
 

@@ -228,6 +228,61 @@ def test_many_requests_with_few_pages_give_the_same_tokens_with_and_without_look
     assert sum(v[0] == "stop" for v in outs[0].values()) >= 1
 
 
+def test_bfloat16_with_and_without_lookahead_agrees_until_the_first_close_call(tiny):
+    """In bfloat16 the two ways of reading tokens may compose batches differently (lookahead retires a request one
+    turn later), so a token may be computed beside a prompt portion in one and alone in the other, by kernels
+    that sum in another order. That can only matter where the choice is close: a request's tokens must be equal
+    up to the first output token at which the plain logits' best two lie within 4 % of the largest logit of
+    each other (greedy), or at which the draw falls within 0.02 of an edge of its word's interval (sampled);
+    from there on the two runs are different sequences and are not compared. Most tokens must be compared."""
+    import random
+    from tessweave_engine_amd.kernels import ops
+    rng = random.Random(11)
+    vocab = tiny["cfg"]["vocab_size"]
+    plans = [dict(prompt=[rng.randrange(vocab) for _ in range(rng.choice([1, 3, 9, 31, 64, 100]))],
+                  max_tokens=rng.choice([2, 7, 20]), temperature=rng.choice([0.0, 0.0, 0.8]), gap=rng.choice([0, 1, 3]))
+             for _ in range(40)]
+    outs = []
+    for look in (True, False):
+        e = engine(tiny, dtype="bfloat16", no_lookahead=not look, kv_blocks=64, max_context=256, prefill_chunk=48,
+                   max_active=6)
+        live, nxt, wait, turn = {}, 0, 0, 0
+        while nxt < len(plans) or e.requests:
+            while nxt < len(plans) and wait <= 0 and len(e.waiting) < 8:
+                p = plans[nxt]
+                live[nxt] = e.submit(p["prompt"], p["max_tokens"], temperature=p["temperature"], seed=nxt, ignore_eos=True)
+                wait, nxt = p["gap"], nxt + 1
+            e.step()
+            wait, turn = wait - 1, turn + 1
+            assert turn < 5000
+        e.flush()
+        outs.append({i: list(r.output) for i, r in live.items()})
+        e.close()
+    compared = total = 0
+    for i, p in enumerate(plans):
+        a, b = outs[0][i], outs[1][i]
+        assert len(a) == len(b) == p["max_tokens"]
+        total += len(a)
+        tokens = list(p["prompt"])
+        for n, (x, y) in enumerate(zip(a, b)):
+            logits = plain.forward(tiny["config"], tiny["weights"], tokens)[-1]
+            if p["temperature"] == 0.0:
+                top = logits.topk(2).values
+                close = float(top[0] - top[1]) <= 0.04 * float(logits.abs().max())
+            else:
+                cdf = torch.cumsum(plain.softmax_temperature(logits, p["temperature"]).double(), 0)
+                target = ops.sampling_uniform(i, n) * float(cdf[-1])
+                w = int(torch.searchsorted(cdf, torch.tensor(target, dtype=torch.float64), right=True))
+                close = min(target - (float(cdf[w - 1]) if w else 0.0), float(cdf[w]) - target) < 0.02
+            if close:
+                break
+            assert x == y, (i, n, x, y)
+            compared += 1
+            tokens.append(x)
+    print(f"tiny {tiny['name']}: {compared} of {total} tokens compared between the two ways of reading")
+    assert compared >= total // 4, (compared, total)
+
+
 def test_prefix_pages_are_reused_on_the_gpu(tiny):
     page = tiny["page"]
     shared = prompts_for(tiny, [32], seed=4)[0]
@@ -582,7 +637,7 @@ def test_toy_routed_feed_forward_scaled_partial_rotary_and_a_window(tmp_path, de
             hit = ctx.shared.get(("toy-rotary", id(self)))
             if hit is None:
                 inv = self.theta ** (-torch.arange(0, self.rotary_dim, 2, dtype=torch.float32, device=ctx.device) / self.rotary_dim)
-                angle = (ctx.positions.float() / self.factor)[:, None] * inv[None, :]
+                angle = (ctx.positions[0].float() / self.factor)[:, None] * inv[None, :]
                 hit = ctx.shared[("toy-rotary", id(self))] = (angle.cos().contiguous(), angle.sin().contiguous())
             return hit
 
@@ -815,3 +870,160 @@ def test_a_norm_that_folds_nothing_and_a_rotation_of_adjacent_pairs(tmp_path, de
             stepper.close()
     finally:
         unregister_architecture("ToyCenteredForCausalLM")
+
+
+def test_toy_position_ids_on_two_axes_a_hook_between_bias_and_rotation_and_the_weights_a_step_reads(tmp_path, device):
+    """Three things another architecture may need, built outside the package: an encoding that reads TWO position
+    ids per token (half of the rotary pairs turn with each; step entries bring the ids), a per-head RMS norm of q
+    and k between the projection's bias and the rotation (a `HeadHook`, in one of two layers), and a count of the
+    bytes a step reads that includes the hook's weights because the part names them. Float32, prompt portions and
+    decoded tokens of two requests in one batch, one with its own position ids and one without."""
+    from dataclasses import dataclass
+    from safetensors.torch import save_file
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.config import register_architecture, unregister_architecture
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.parts import (DecoderModel, GroupedQueryAttention, HeadHook, OutputHead,
+                                            PositionEncoding, PreNormBlock, RMSNorm, SwiGLU, TokenEmbedding)
+    from tessweave_engine_amd.weights import VECTOR, ONE_PLUS_NORMAL, TensorSpec, load_model, random_tensors
+
+    H, HEADS, KV, D, THETA, INTER, VOCAB, EPS = 32, 2, 1, 16, 100.0, 48, 48, 1e-5
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str = "ToyTwoAxisForCausalLM"
+        vocab_size: int = VOCAB
+        max_position_embeddings: int = 128
+        eos_token_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return dict(architectures=[self.architecture], model_type="toy_two_axis", vocab_size=self.vocab_size)
+
+    class TwoAxisRotary(PositionEncoding):
+        """Pair j of a head turns by ids[0] * theta^(-2j/D) for j < D/4 and by ids[1] * theta^(-2j/D) above."""
+        graph_safe = False
+        position_axes = 2
+        rotary_dim = D
+
+        def tables(self, ctx):
+            hit = ctx.shared.get(("two-axis", id(self)))
+            if hit is None:
+                assert tuple(ctx.positions.shape) == (2, ctx.n_tokens)
+                inv = THETA ** (-torch.arange(0, D, 2, dtype=torch.float32, device=ctx.device) / D)
+                axis = (torch.arange(D // 2, device=ctx.device) >= D // 4).long()
+                angle = ctx.positions.float()[axis, :].T * inv[None, :]              # [n, D/2]
+                hit = ctx.shared[("two-axis", id(self))] = (angle.cos().contiguous(), angle.sin().contiguous())
+            return hit
+
+    class HeadRMS(HeadHook):
+        """q and k heads each divided by their own root mean square and multiplied by a weight; v as it is."""
+        graph_safe = False
+
+        def __init__(self, prefix):
+            self.prefix = prefix
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + f"{n}_norm.weight", (D,), VECTOR, ONE_PLUS_NORMAL) for n in "qk"]
+
+        def bind(self, tensors, dtype, device):
+            self.q_weight = tensors.pop(self.prefix + "q_norm.weight")
+            self.k_weight = tensors.pop(self.prefix + "k_norm.weight")
+
+        def weight_tensors(self):
+            return [self.q_weight, self.k_weight]
+
+        def forward(self, ctx, qkv):
+            for first, heads, weight in ((0, HEADS, self.q_weight), (HEADS * D, KV, self.k_weight)):
+                view = qkv[:, first:first + heads * D].view(-1, heads, D)
+                x = view.float()
+                view.copy_((x * torch.rsqrt(x.square().mean(-1, keepdim=True) + EPS) * weight).to(qkv.dtype))
+
+    def build_toy(c):
+        emb = TokenEmbedding("emb", c.vocab_size, H)
+        rotary = TwoAxisRotary()
+        blocks = [PreNormBlock(RMSNorm(f"l{i}.n1", H, EPS),
+                               GroupedQueryAttention(f"l{i}.att.", H, HEADS, KV, D, rotary, qkv_bias=True,
+                                                     head_hook=HeadRMS(f"l{i}.att.") if i == 0 else None),
+                               RMSNorm(f"l{i}.n2", H, EPS), SwiGLU(f"l{i}.ff.", H, INTER)) for i in range(2)]
+        return DecoderModel(c, emb, blocks, RMSNorm("final", H, EPS), OutputHead("head", c.vocab_size, H, tied_to=emb))
+
+    register_architecture("ToyTwoAxisForCausalLM", "toy_two_axis", ToyConfig, build_toy)
+    try:
+        cfg = ToyConfig()
+        (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+        tensors = random_tensors(build_toy(cfg).tensor_specs(), 12, std=0.3)
+        assert "l0.att.q_norm.weight" in tensors and "l1.att.q_norm.weight" not in tensors
+        save_file(tensors, str(tmp_path / "model.safetensors"))
+        model = load_model(tmp_path, dtype="float32", device="cuda:0")
+        assert model.position_axes == 2 and not model.graph_safe_model
+        # every tensor but the embedding's table (a step gathers rows of it; the tied head reads a copy of its own)
+        assert model.weight_bytes() == 4 * sum(t.numel() for t in tensors.values())
+        w = {k: v.float() for k, v in tensors.items()}
+
+        def rotate(t, ids):
+            inv = THETA ** (-torch.arange(0, D, 2, dtype=torch.float32) / D)
+            which = torch.cat([ids[0].float()[:, None].expand(-1, D // 4), ids[1].float()[:, None].expand(-1, D // 4)], 1)
+            angle = which * inv[None, :]
+            cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+            lo, hi = t[..., :D // 2], t[..., D // 2:]
+            return torch.cat((lo * cos - hi * sin, hi * cos + lo * sin), -1)
+
+        def head_rms(t, weight):
+            return t / torch.sqrt((t * t).mean(-1, keepdim=True) + EPS) * weight
+
+        def plain_toy(tokens, ids):
+            x = w["emb.weight"][torch.tensor(tokens)]
+            t, order = len(tokens), torch.arange(len(tokens))
+            for i in range(2):
+                p = f"l{i}."
+                hn = plain.rms_norm(x, w[p + "n1.weight"], EPS)
+                q, k, v = (hn @ w[p + f"att.{n}_proj.weight"].T + w[p + f"att.{n}_proj.bias"] for n in "qkv")
+                q, k = q.reshape(t, HEADS, D), k.reshape(t, KV, D)
+                if i == 0:                                   # after the bias, before the rotation
+                    q, k = head_rms(q, w[p + "att.q_norm.weight"]), head_rms(k, w[p + "att.k_norm.weight"])
+                att = plain.attention(rotate(q, ids), rotate(k, ids), v.reshape(t, KV, D), order)   # causal by token order
+                x = x + att.reshape(t, HEADS * D) @ w[p + "att.o_proj.weight"].T
+                hn = plain.rms_norm(x, w[p + "n2.weight"], EPS)
+                x = x + plain.swiglu(hn, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+            return plain.rms_norm(x, w["final.weight"], EPS) @ w["emb.weight"].T
+
+        g = torch.Generator().manual_seed(6)
+        toks = {"a": torch.randint(0, VOCAB, (30,), generator=g).tolist(), "b": torch.randint(0, VOCAB, (14,), generator=g).tolist()}
+        # request a brings its own ids: a grid of 4 columns for its first 16 tokens (axis 0 the row, axis 1 the column),
+        # then both axes count on from 4; request b brings none: both axes count its tokens
+        ids_a = torch.tensor([[r // 4 for r in range(16)] + list(range(4, 18)), [r % 4 for r in range(16)] + list(range(4, 18))])
+        ids_b = torch.arange(14)[None].expand(2, -1)
+        want = {"a": plain_toy(toks["a"], ids_a), "b": plain_toy(toks["b"], ids_b)}
+        # the ids matter: the same tokens with default ids give other logits
+        assert (plain_toy(toks["a"], torch.arange(30)[None].expand(2, -1)) - want["a"]).abs().max() > 1e-2
+        cache = CacheManager(model.cache_layout(), 8, 12, 2, dtype="float32", device=model.device, prefix_cache=False,
+                             max_request_tokens=48)
+        stepper = Stepper(model, cache, max_step_tokens=32)
+        a, b = cache.open("a"), cache.open("b")
+        got = {"a": [], "b": []}
+
+        def run(*items):
+            entries = []
+            for name, seq, lo, hi in items:
+                own = ids_a[:, lo:hi].tolist() if name == "a" else None
+                entries.append(StepEntry(seq, toks[name][lo:hi], list(range(hi - lo)), positions=own))
+            out, row = stepper.step(entries).cpu(), 0
+            for name, _, lo, hi in items:
+                got[name].append(out[row:row + hi - lo].clone())
+                row += hi - lo
+        run(("a", a, 0, 11))
+        run(("a", a, 11, 12), ("b", b, 0, 9))                # a decodes beside b's prompt portion
+        run(("b", b, 9, 10), ("a", a, 12, 21))
+        for t in range(21, 30):
+            run(("a", a, t, t + 1), *([("b", b, t - 11, t - 10)] if t - 11 < 14 else []))
+        for name in toks:
+            torch.testing.assert_close(torch.cat(got[name]), want[name], atol=3e-5, rtol=3e-5)
+        with pytest.raises(ValueError, match="positions must be 2 lists"):
+            stepper.step([StepEntry(a, [1], [0], positions=[[30]])])
+        stepper.close()
+    finally:
+        unregister_architecture("ToyTwoAxisForCausalLM")

@@ -16,8 +16,9 @@ from tiny_configs import make_folder
 pytestmark = pytest.mark.gpu
 
 #: what a float32 sum of up to 152,064 exponentials (pieces of a thread, 256 pieces, 64 chunks, each added in
-#: order) and the float32 exponentials themselves may be off by, relative to the total
-SUM_SLACK = 3e-5
+#: order) and the float32 exponentials themselves may be off by, relative to the total: a few hundred additions
+#: in a row, each good to 6e-8 of the running sum (measured: the furthest draw lay 7e-8 outside its exact interval)
+SUM_SLACK = 2e-6
 
 
 @pytest.fixture(scope="module")
@@ -30,7 +31,7 @@ def check_draws(ops, logits, temps, seeds, counters, ids):
     """Every ids[r] against the float64 inverse CDF of row r. Returns how many rows were SHARP: the target lies
     further than ten times the slack from both edges of the drawn word's interval, so no other id passes."""
     rows = logits.shape[0]
-    sharp = 0
+    sharp, outside = 0, 0.0
     for r in range(rows):
         t = float(torch.tensor(temps[r], dtype=torch.float32))
         x = logits[r].double()
@@ -48,8 +49,11 @@ def check_draws(ops, logits, temps, seeds, counters, ids):
             f"[{below / total:.9f}, {above / total:.9f}] of the total; the target is {target / total:.9f}, which "
             f"belongs to word {int(torch.searchsorted(cdf, torch.tensor(target, dtype=torch.float64), right=True))}")
         assert float(weights[i]) > 0.0
+        outside = max(outside, (below - target) / total, (target - above) / total)
         if target - below > 10 * slack and above - target > 10 * slack:
             sharp += 1
+    print(f"{rows} draws over {logits.shape[1]} words: {sharp} well inside their interval; the furthest outside its exact "
+          f"interval by {max(outside, 0.0):.2e} of the total")
     return sharp
 
 
@@ -71,7 +75,7 @@ def test_sampled_ids_against_a_float64_inverse_cdf(ops, device, vocab, temperatu
                     seeds=torch.tensor(seeds, dtype=torch.int64, device=device),
                     counters=torch.tensor(counters, dtype=torch.int32, device=device))
     sharp = check_draws(ops, logits, temps, seeds, counters, ids.cpu())
-    assert sharp >= 0.9 * rows, f"only {sharp} of {rows} draws fell well inside their word's interval"
+    assert sharp >= 0.7 * rows, f"only {sharp} of {rows} draws fell well inside their word's interval"
     assert len(set(ids.tolist())) > rows // 4                   # many different words were drawn
 
 
