@@ -78,7 +78,8 @@ class DecoderModel(Part):
         total, seen = 0, set()
         for part in walk(self):
             for t in part.weight_tensors():
-                ident = id(getattr(t, "data", t))
+                storage = t if isinstance(t, torch.Tensor) else t.data       # (a kernel-layout weight wraps its tensor)
+                ident = storage.data_ptr()
                 if ident not in seen:
                     seen.add(ident)
                     total += t.numel() * t.element_size()

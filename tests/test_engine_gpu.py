@@ -232,9 +232,11 @@ def test_bfloat16_with_and_without_lookahead_agrees_until_the_first_close_call(t
     """In bfloat16 the two ways of reading tokens may compose batches differently (lookahead retires a request one
     turn later), so a token may be computed beside a prompt portion in one and alone in the other, by kernels
     that sum in another order. That can only matter where the choice is close: a request's tokens must be equal
-    up to the first output token at which the plain logits' best two lie within 4 % of the largest logit of
-    each other (greedy), or at which the draw falls within 0.02 of an edge of its word's interval (sampled);
-    from there on the two runs are different sequences and are not compared. Most tokens must be compared."""
+    up to the first output token at which the plain logits' best two lie within 2 % of the largest logit of
+    each other (greedy; bfloat16 logits are themselves held to 2 % of the largest), or at which the draw falls
+    within 0.01 of an edge of its word's interval (sampled); from there on the two runs are different sequences
+    and are not compared. With random weights the logits are nearly flat, so a request's first close call comes
+    early: an eighth of all tokens must still be compared."""
     import random
     from tessweave_engine_amd.kernels import ops
     rng = random.Random(11)
@@ -268,19 +270,19 @@ def test_bfloat16_with_and_without_lookahead_agrees_until_the_first_close_call(t
             logits = plain.forward(tiny["config"], tiny["weights"], tokens)[-1]
             if p["temperature"] == 0.0:
                 top = logits.topk(2).values
-                close = float(top[0] - top[1]) <= 0.04 * float(logits.abs().max())
+                close = float(top[0] - top[1]) <= 0.02 * float(logits.abs().max())
             else:
                 cdf = torch.cumsum(plain.softmax_temperature(logits, p["temperature"]).double(), 0)
                 target = ops.sampling_uniform(i, n) * float(cdf[-1])
                 w = int(torch.searchsorted(cdf, torch.tensor(target, dtype=torch.float64), right=True))
-                close = min(target - (float(cdf[w - 1]) if w else 0.0), float(cdf[w]) - target) < 0.02
+                close = min(target - (float(cdf[w - 1]) if w else 0.0), float(cdf[w]) - target) < 0.01
             if close:
                 break
             assert x == y, (i, n, x, y)
             compared += 1
             tokens.append(x)
     print(f"tiny {tiny['name']}: {compared} of {total} tokens compared between the two ways of reading")
-    assert compared >= total // 4, (compared, total)
+    assert compared >= total // 8, (compared, total)
 
 
 def test_prefix_pages_are_reused_on_the_gpu(tiny):
