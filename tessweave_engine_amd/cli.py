@@ -189,10 +189,17 @@ def main(argv=None):
         c = read_model_config(args.model)
         layout = build_model(c).cache_layout()
         tokens = args.kv_blocks * args.block_size
+        # Two figures where they differ: the reference's formula over the checkpoint's head size, and what the
+        # device holds (the kernels lay a head out in multiples of 16 elements, the tail zeros).
+        formula = {f"kv_{name}_bytes_by_formula": c.kv_bytes_per_token(size) * tokens
+                   for name, size in (("bf16", 2), ("fp32", 4)) if hasattr(c, "kv_bytes_per_token")
+                   and c.kv_bytes_per_token(size) != layout.bytes_per_token(size)}
         print(json.dumps({"architecture": c.describe(),
-                          "kv_formula": "2 * layers * KV_heads * head_dim * bytes_per_element * blocks * block_size",
+                          "kv_formula": "2 * layers * KV_heads * head_dim * bytes_per_element * blocks * block_size"
+                                        + (" (on the device head_dim is rounded up to a multiple of 16)" if formula else ""),
                           "kv_bf16_bytes": layout.bytes_per_token(2) * tokens,
                           "kv_fp32_bytes": layout.bytes_per_token(4) * tokens,
+                          **formula,
                           "cache_groups": [{"layers": len(g.slots), "kv_heads": g.spec.kv_heads,
                                             "head_dim": g.spec.head_dim, "window": g.spec.window}
                                            for g in layout.groups],

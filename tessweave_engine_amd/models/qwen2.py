@@ -113,7 +113,9 @@ class Qwen2Config:
         }
 
     def kv_bytes_per_token(self, element_bytes):
-        """2 * layers * kv_heads * head_dim * bytes (flow_engine/config.py:64-65)."""
+        """2 * layers * kv_heads * head_dim * bytes (flow_engine/config.py:64-65), over the checkpoint's head
+        size. The device holds heads in multiples of 16 elements: what the cache really takes is
+        `model.cache_layout().bytes_per_token`, which `inspect` prints beside this where the two differ."""
         return 2 * self.num_hidden_layers * self.num_key_value_heads * self.head_dim * element_bytes
 
     def describe(self):

@@ -35,6 +35,15 @@ def test_doctor_inspect_random_weights_and_replay(tmp_path, capsys):
     per_token = 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"] * cfg["head_dim"]
     assert info["kv_bf16_bytes"] == per_token * 2 * 80 and info["kv_fp32_bytes"] == per_token * 4 * 80
     assert info["architecture"]["num_hidden_layers"] == 3 and info["cache_groups"][0]["window"] is None
+    assert "kv_bf16_bytes_by_formula" not in info               # head size 32: the device holds what the formula says
+    # a head of 18 elements lies in 32 on the device: both figures are printed
+    odd = tmp_path / "odd"
+    odd.mkdir()
+    (odd / "config.json").write_text(json.dumps(dict(cfg, head_dim=18, hidden_size=6 * 18)))
+    info = json.loads(run(capsys, "inspect", str(odd), "--kv-blocks", "10", "--block-size", "8"))
+    layers_heads = 2 * cfg["num_hidden_layers"] * cfg["num_key_value_heads"]
+    assert info["kv_bf16_bytes"] == layers_heads * 32 * 2 * 80 and info["kv_bf16_bytes_by_formula"] == layers_heads * 18 * 2 * 80
+    assert info["kv_fp32_bytes_by_formula"] * 32 == info["kv_fp32_bytes"] * 18
     with pytest.raises(SystemExit):
         cli.main(["inspect", str(tmp_path), "--kv-blocks", "0"])
     capsys.readouterr()
