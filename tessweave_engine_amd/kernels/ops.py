@@ -282,7 +282,7 @@ def linear_glu(x, weight, out, bias=None, force=0):
     return out
 
 
-GEMM_AUTO, GEMM_GENERIC, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY, GEMM_TILED_256, GEMM_TILED_256X192 = 0, 1, 3, 4, 5, 6, 7
+GEMM_AUTO, GEMM_GENERIC, GEMM_TILED, GEMM_TILED_WIDE, GEMM_SKINNY, GEMM_TILED_256, GEMM_TILED_256X192, GEMM_STREAM_CU = 0, 1, 3, 4, 5, 6, 7, 8
 
 
 def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_AUTO):

@@ -137,12 +137,13 @@ class Linear(Part):
     # ---- leave the split-K sums to the next kernel -------------------------------------------
     def _partial_splits(self, n_rows, lda=None):
         """K ranges of `forward_partials` for N_ROWS rows, LDA elements apart (default: contiguous); 0: none.
-        Up to 64 rows the streaming kernel's ranges depend on the matrix alone; above, the tiled kernels
-        choose them per row count and stride."""
+        Up to 64 rows the streaming kernels' ranges depend on the matrix and on how many tiles of 16 rows
+        there are; above, the tiled kernels choose them per row count and stride."""
         lda = self.weights[0].shape[1] if lda is None else int(lda)
-        key = ("splits", 64 if n_rows <= 64 else n_rows, lda)
+        tile = (n_rows + 15) // 16 * 16 if n_rows <= 64 else n_rows       # up to 64 rows: the same for a tile of 16 rows
+        key = ("splits", tile, lda)
         if key not in self._ws_floats:
-            self._ws_floats[key] = ops.linear_partial_splits_rows(self.weights[0], n_rows, lda)
+            self._ws_floats[key] = ops.linear_partial_splits_rows(self.weights[0], tile, lda)
         return self._ws_floats[key]
 
     def deferrable(self, n_rows):
@@ -159,7 +160,8 @@ class Linear(Part):
         n = x.shape[0]
         splits = self._partial_splits(n, x.stride(0) if n > 1 else None)
         if n <= 64:     # sized once for the largest such batch, so that it never regrows under a captured graph
-            buf = ctx.workspace.get("linear.partial." + tag, (splits, 64, w.shape[0]), torch.float32)
+            most = max(self._partial_splits(rows) for rows in (16, 32, 48, 64))
+            buf = ctx.workspace.get("linear.partial." + tag, (most, 64, w.shape[0]), torch.float32)
         else:
             buf = ctx.workspace.get("linear.partial.rows." + tag, (splits, n, w.shape[0]), torch.float32)
         partial = buf.view(-1)[:splits * n * w.shape[0]].view(splits, n, w.shape[0])

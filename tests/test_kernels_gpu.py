@@ -275,6 +275,7 @@ LINEAR_SHAPES = [  # m, n, k
     (130, 96, 4096), (257, 260, 2056),      # few tiles, long K: the tiled kernel splits K as well
     (300, 520, 800), (513, 300, 4128),      # K a multiple of 32: the larger tiles copy straight into LDS
     (8, 18950, 64), (16, 18944, 32),        # few rows, one K range, many columns: workgroups of two waves
+    (40, 9000, 256), (64, 45000, 96), (20, 2000, 1536), (48, 520, 9472),   # one workgroup per CU: rounds, K ranges, an idle wave
 ]
 
 
@@ -300,7 +301,7 @@ def test_linear_all_paths(ops, device, dtype, m, n, k):
         with pytest.raises(Exception, match="refused its arguments"):
             ops.linear(x, shuffled, torch.empty((m, n), dtype=dtype, device=device), force=ops.GEMM_TILED_256)
     for force in forces + [("shuffled", f) for f in (ops.GEMM_AUTO, ops.GEMM_GENERIC, ops.GEMM_TILED, ops.GEMM_TILED_WIDE)
-                           + big + ((ops.GEMM_SKINNY,) if m <= 64 else ())]:
+                           + big + ((ops.GEMM_SKINNY, ops.GEMM_STREAM_CU) if m <= 64 else ())]:
         wt = w
         if isinstance(force, tuple):
             wt, force = shuffled, force[1]
@@ -348,21 +349,31 @@ def test_linear_large_tiles_over_k_ranges(ops, device, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 389, 2048), (17, 130, 4096), (64, 96, 9472)])
+@pytest.mark.parametrize("m,n,k", [(1, 48, 64), (8, 389, 2048), (17, 130, 4096), (64, 96, 9472), (33, 4608, 3584),
+                                   (64, 3584, 2368), (48, 1000, 520)])
 def test_linear_partials(ops, device, dtype, m, n, k):
+    """Sums of K ranges left for the next kernel: row-major weights through the kernel with four column tiles a
+    workgroup, shuffled ones through the same (up to 16 rows: identical bits) or, above 16 rows, through the
+    kernel with one workgroup per CU, which names its own number of ranges."""
     x = rand((m, k), dtype, device, 1.0, seed=1)
     w = rand((n, k), dtype, device, 0.05, seed=2)
-    splits = ops.linear_partial_splits(dtype, n, k)
-    part = torch.full((splits, m, n), float("nan"), device=device)
-    ops.linear_partials(x, w, part)
     want = x.double().cpu() @ w.double().cpu().T
     scale = math.sqrt(k) * 0.05
-    torch.testing.assert_close(part.double().sum(0).cpu(), want, atol=3e-5 * scale, rtol=1e-5)
-    rows_sum = part.sum(0).clone()
-    w = ops.shuffle_weight(w)                    # the same from the shuffled layout: identical bits
-    part.fill_(float("nan"))
-    ops.linear_partials(x, w, part)
-    torch.testing.assert_close(part.sum(0), rows_sum, atol=0, rtol=0)
+    sums = []
+    for weight in (w, ops.shuffle_weight(w)):
+        splits = ops.linear_partial_splits_rows(weight, m)
+        assert splits >= 1
+        part = torch.full((splits, m, n), float("nan"), device=device)
+        ops.linear_partials(x, weight, part)
+        torch.testing.assert_close(part.double().sum(0).cpu(), want, atol=3e-5 * scale, rtol=1e-5)
+        if k >= 2048:
+            assert part.abs().amax(dim=(1, 2)).min() > 0         # every range did its share
+        with pytest.raises(ValueError, match="partial must be"):
+            ops.linear_partials(x, weight, torch.empty(splits + 1, m, n, device=device))
+        sums.append(part.sum(0).clone())
+    if m <= 16:
+        assert ops.linear_partial_splits_rows(w, m) == ops.linear_partial_splits(dtype, n, k)
+        torch.testing.assert_close(sums[0], sums[1], atol=0, rtol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -398,7 +409,8 @@ def test_linear_partials_of_many_rows(ops, device, dtype, m, n, k):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 64), (8, 208, 320), (17, 48, 1032), (64, 1040, 256), (65, 80, 64),
                                        (200, 400, 320), (130, 16, 101), (520, 272, 200), (520, 272, 320),
-                                       (8, 9472, 64), (3, 9488, 96)])     # so many columns that few rows run in workgroups of two waves
+                                       (8, 9472, 64), (3, 9488, 96),      # so many columns that few rows run in workgroups of two waves
+                                       (33, 2400, 128), (64, 18944, 96), (50, 176, 512)])   # one workgroup per CU: pairs in rounds
 def test_linear_glu(ops, device, dtype, m, inter, k):
     """silu(x gate^T + b) * (x up^T + b) from interleaved rows, every kernel and both layouts."""
     x = rand((m, k), dtype, device, 1.0, seed=1)
@@ -421,6 +433,8 @@ def test_linear_glu(ops, device, dtype, m, inter, k):
         want = torch.nn.functional.silu(g) * u
         for weight in layouts:
             big = [ops.GEMM_TILED_256, ops.GEMM_TILED_256X192] if (dtype == torch.bfloat16 and weight is not w) else []
+            if weight is not w and m <= 64:
+                big = big + [ops.GEMM_STREAM_CU]
             for force in forces + big:
                 out = torch.full((m, inter), float("nan"), dtype=dtype, device=device)
                 ops.linear_glu(x, weight, out, bias=b, force=force)
