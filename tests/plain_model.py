@@ -55,8 +55,12 @@ def rope(x, positions, theta):
     """
     d = x.shape[-1]
     half = d // 2
-    inv = theta ** (-torch.arange(0, d, 2, dtype=torch.float32) / d)       # fp32 as the reference
-    angle = positions.to(torch.float32)[:, None] * inv[None, :]             # [T, D/2] in fp32
+    # fp32 as the reference, and always on the host: a float32 power differs in its last bit between the host's
+    # and a GPU's routine, and an angle is that rate times a position of thousands (at position 4,000 the two
+    # rotations are 2e-4 rad apart, which shows in the logits as 7e-5: as much as four layers of float32
+    # rounding). The engine computes the rates on the host; so does this, wherever the rest of it runs.
+    inv = (theta ** (-torch.arange(0, d, 2, dtype=torch.float32, device="cpu") / d)).to(x.device)
+    angle = positions.to(device=x.device, dtype=torch.float32)[:, None] * inv[None, :]   # [T, D/2] in fp32
     cos, sin = angle.cos().to(x.dtype)[:, None, :], angle.sin().to(x.dtype)[:, None, :]
     lo, hi = x[..., :half], x[..., half:]
     return torch.cat((lo * cos - hi * sin, hi * cos + lo * sin), -1)

@@ -15,7 +15,7 @@ The weights are drawn on the GPU (two billion values) and the plain implementati
 (the yardstick), in float32 and in bfloat16. Both bars are calibrated rather than fixed, because rounding errors
 grow with depth, width and the number of columns the largest error is taken over (with one wide layer and 4,099
 columns bfloat16 is off by 1 % of the largest logit, with four layers and 152,064 columns by 2 %: the square
-root of the depth). float32: the engine may be off from float64 by at most four times what the plain
+root of the depth). float32: the engine may be off from float64 by at most twice what the plain
 implementation in float32 is off (+ 1e-6). bfloat16: the engine, which keeps the residual stream, the softmax
 and every sum in 32-bit, must be closer to float64 than the plain implementation with every tensor and every
 intermediate result in bfloat16 is.
@@ -148,6 +148,6 @@ def test_four_full_width_layers_and_the_full_vocabulary_through_replay(shape7b, 
           f"{len(steps)} steps; engine off by {worst_engine:.3e}, plain {dtype} off by {worst_plain:.3e}, "
           f"largest logit {largest:.3f}")
     if dtype == "float32":
-        assert worst_engine <= 4 * worst_plain + 1e-6, (worst_engine, worst_plain)
+        assert worst_engine <= 2 * worst_plain + 1e-6, (worst_engine, worst_plain)
     else:
         assert worst_engine <= worst_plain, (worst_engine, worst_plain)
