@@ -34,6 +34,48 @@ extern "C" int tw_graph_launch(void* exec, hipStream_t stream) {
 
 extern "C" int tw_graph_destroy(void* exec) { return (int)hipGraphExecDestroy((hipGraphExec_t)exec); }
 
+// ---- the step's metadata, fetched by a kernel ------------------------------------------------------------
+// A step's token ids, positions, block tables and so on are packed on the host into pinned memory and must
+// be on the device before the step's first kernel reads them. A memory copy for that goes through the copy
+// engine: the compute queue hands over to it and takes over again, which on this device leaves the queue idle
+// for 30 to 130 us around a copy of a few kilobytes. A kernel that reads the pinned memory itself stays in the
+// step's own queue: the same bytes arrive in a few microseconds with nothing to wait for on either side.
+#define TW_UPLOAD_MAX_SEGMENTS 16
+struct UploadSegments {
+  int n;
+  int offset[TW_UPLOAD_MAX_SEGMENTS];      // in 32-bit words, the same in source and destination
+  int count[TW_UPLOAD_MAX_SEGMENTS];
+};
+
+__global__ __launch_bounds__(256) void upload_words_kernel(const int* __restrict__ src, int* __restrict__ dst, UploadSegments seg) {
+  for (int s = blockIdx.y; s < seg.n; s += gridDim.y) {
+    const int* from = src + seg.offset[s];
+    int* to = dst + seg.offset[s];
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < seg.count[s]; i += gridDim.x * blockDim.x) to[i] = from[i];
+  }
+}
+
+// dst[offset[s] + i] = src[offset[s] + i] for i < count[s], s < n. `src` is pinned host memory (or any memory
+// the device can read), `dst` device memory; both hold 32-bit words.
+extern "C" int tw_upload_words(const int* src, int* dst, int n, const int* offsets, const int* counts, hipStream_t stream) {
+  TW_REQUIRE(src != nullptr && dst != nullptr && n >= 0 && n <= TW_UPLOAD_MAX_SEGMENTS);
+  if (n == 0) return 0;
+  UploadSegments seg;
+  seg.n = n;
+  int most = 0;
+  for (int s = 0; s < n; ++s) {
+    TW_REQUIRE(offsets[s] >= 0 && counts[s] >= 0);
+    seg.offset[s] = offsets[s];
+    seg.count[s] = counts[s];
+    if (counts[s] > most) most = counts[s];
+  }
+  int blocks = tw_div_up(most, 256);
+  if (blocks > 64) blocks = 64;
+  if (blocks < 1) blocks = 1;
+  upload_words_kernel<<<dim3(blocks, n), 256, 0, stream>>>(src, dst, seg);
+  return TW_LAUNCH_RESULT();
+}
+
 // ---- a yardstick, not part of any model: how fast can this device read memory at all? --------------------
 // Every wave streams 1 KB non-temporal loads, eight in flight, and adds them up; nothing is written unless
 // the sum takes one particular value (so the loads cannot be dropped). Benchmarks time it over gigabytes to

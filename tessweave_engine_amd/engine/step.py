@@ -26,6 +26,7 @@ from dataclasses import dataclass, field
 import numpy as np
 import torch
 
+from ..kernels import ops
 from ..kernels.lib import library, check
 from ..parts.base import GroupStep, StepContext, Workspace
 
@@ -189,9 +190,14 @@ class Stepper:
         self.steps += 1
 
     def upload(self, ctx):
-        """Copy the step's packed metadata to the device (on the current stream)."""
+        """Bring the step's packed metadata to the device (on the current stream): a kernel fetches the parts
+        this step filled from the pinned staging buffer, which keeps the step in one queue (a memory copy
+        would hand over to the copy engine and back, tens of microseconds of idle queue per step)."""
         k = ctx.staging_index
-        self._meta_dev.copy_(self._staging[k], non_blocking=True)
+        if ctx.staging_segments is not None and len(ctx.staging_segments) <= 16:
+            ops.upload_words(self._staging[k], self._meta_dev, ctx.staging_segments)
+        else:
+            self._meta_dev.copy_(self._staging[k], non_blocking=True)
         event = torch.cuda.Event()
         event.record(torch.cuda.current_stream(self.device))
         self._staging_events[k] = event
@@ -252,9 +258,12 @@ class Stepper:
             self._staging_events[k].synchronize()
         host = self._staging_np[k]
 
+        segments = []                        # (offset, words) of what this step fills: all that has to travel
+
         def put(name, values):
             off, _ = self._sections[name]
             host[off:off + len(values)] = values
+            segments.append((off, len(values)))
 
         put("token_ids", token_ids)
         axes = self.position_axes
@@ -279,6 +288,7 @@ class Stepper:
             put(f"slots{g}", np.where(pages >= 0, pages * page + positions % page, -1))
             off, _ = self._sections[f"table{g}"]
             host[off:off + n_seqs * width] = tables.reshape(-1)
+            segments.append((off, n_seqs * width))
 
         ctx = StepContext()
         ctx.device, ctx.dtype = self.device, self.dtype
@@ -307,6 +317,7 @@ class Stepper:
                      and rows == list(range(n_seqs)))
         ctx.capturing = graphable       # fixed launch shapes in warm-up, capture and replay alike
         ctx.staging_index = k
+        ctx.staging_segments = segments
         return ctx, ordered, graphable
 
     def _first_positions(self, group, computed):

@@ -18,6 +18,7 @@ _SIGNATURES = {
     "tw_graph_launch": (I, [P, P]),
     "tw_graph_destroy": (I, [P]),
     "tw_probe_read": (I, [P, L, P, I, ctypes.POINTER(c_long), P]),
+    "tw_upload_words": (I, [P, P, I, ctypes.POINTER(c_int), ctypes.POINTER(c_int), P]),
     "tw_embed_gather": (I, [I, P, P, P, I, I, I, P, I, P]),
     "tw_rmsnorm": (I, [I, P, P, P, P, I, I, F, P, I, L, P, P]),
     "tw_rope_table": (I, [P, P, P, P, I, I, P]),

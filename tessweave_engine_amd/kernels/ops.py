@@ -55,6 +55,23 @@ def probe_read(buffer, out, blocks=2048):
     return int(n.value)
 
 
+def upload_words(src, dst, segments):
+    """dst[o:o + n] = src[o:o + n] for every (o, n) of SEGMENTS (at most 16), by a kernel on the current stream.
+
+    src: a pinned int32 host tensor; dst: an int32 device tensor of the same length. A step's metadata goes to
+    the device this way: a copy through the copy engine leaves the compute queue idle around it for tens of
+    microseconds, a kernel that reads the pinned memory does not leave the queue."""
+    import ctypes
+    _need(src.dtype == torch.int32 and dst.dtype == torch.int32 and src.is_contiguous() and dst.is_contiguous(),
+          "upload_words moves contiguous int32 buffers")
+    _need(src.is_pinned() and dst.is_cuda and src.numel() == dst.numel(), "upload_words: pinned host words to as many device words")
+    segments = [(int(o), int(n)) for o, n in segments if n > 0]
+    _need(len(segments) <= 16 and all(o >= 0 and o + n <= dst.numel() for o, n in segments), "upload_words: bad segments")
+    offsets = (ctypes.c_int * 16)(*[o for o, _ in segments])
+    counts = (ctypes.c_int * 16)(*[n for _, n in segments])
+    check(library().tw_upload_words(src.data_ptr(), dst.data_ptr(), len(segments), offsets, counts, _stream()), "upload_words")
+
+
 def embed_gather(ids, table, out, feed=None):
     """out[n, :] = float32(table[ids[n], :]); an id -1 - k stands for feed[k] (int32, on the device)."""
     n = ids.numel()

@@ -223,6 +223,7 @@ class StepContext:
         self.workspace = None        # Workspace
         self.shared = {}             # per-step values shared by layers (rotary tables, ...)
         self.staging_index = 0       # which host staging buffer holds this step's metadata
+        self.staging_segments = None # (offset, words) of the parts of that buffer this step filled
 
     def scratch(self, tag, shape, dtype=None):
         """Per-token scratch [n, ...]: the buffer is sized once for the largest step."""
