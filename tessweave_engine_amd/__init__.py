@@ -1,2 +1,2 @@
-"""An inference engine for the Qwen2.5 dense decoder on AMD MI355X (gfx950)."""
+"""An inference engine on AMD MI355X (gfx950) for the architectures its registry names (`models/`)."""
 __version__ = "0.1.0"

@@ -45,8 +45,10 @@ def _engine_options(p):
 
 
 def build_parser():
+    from .config.registry import registered_architectures
+    names = ", ".join(registered_architectures()) or "none"
     parser = argparse.ArgumentParser(prog="flow-inference",
-                                     description="Qwen2.5 dense inference engine for AMD MI355X")
+                                     description=f"Inference engine for AMD MI355X; registered architectures: {names}")
     sub = parser.add_subparsers(dest="command", required=True)
     sub.add_parser("doctor", help="read-only report of the runtime and the accelerator")
     inspect = sub.add_parser("inspect", help="validate config.json and explain the cache allocation; no weights are read")

@@ -351,6 +351,17 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 typedef __attribute__((address_space(3))) void* tw_lds_ptr;
 #define TW_DMA_STAGES 4
 
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a constant
+// expression in the body (the scheduler's group barriers take constants only)
+template <int... Is, typename F>
+__device__ __forceinline__ void tw_unroll_impl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void tw_unroll(F&& f) {
+  tw_unroll_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
 template <typename OutT, int WM, int WN, bool GLU>
 __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict__ A, long lda,
                                                        const bf16_t* __restrict__ W, long k_steps,
@@ -415,12 +426,17 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
       w_src[b] = W + ((size_t)blk * k_steps + kt0) * 512 + lane * 8;
     }
   }
-  auto copy_tile = [&](int t_v) {                          // k-tile kt0 + t_v into stage t_v % 4
+  // k-tile kt0 + t_v into stage t_v % 4, in two halves: the A blocks and the W blocks
+  auto copy_a = [&](int t_v) {
     const int t = min(t_v, k_tiles - 1);                   // past the end: a copy nobody reads
     char* stage = lds + (t_v % TW_DMA_STAGES) * STAGE;
 #pragma unroll
     for (int b = 0; b < WM; ++b)
       __builtin_amdgcn_global_load_lds(a_src[b] + (size_t)t * 32, (tw_lds_ptr)(stage + (WM * wave + b) * 1024), 16, 0, 0);
+  };
+  auto copy_w = [&](int t_v) {
+    const int t = min(t_v, k_tiles - 1);
+    char* stage = lds + (t_v % TW_DMA_STAGES) * STAGE;
 #pragma unroll
     for (int b = 0; b < WN; ++b)
       __builtin_amdgcn_global_load_lds(w_src[b] + (size_t)t * 512, (tw_lds_ptr)(stage + BM * 64 + (WN * wave + b) * 1024), 16, 0, 0);
@@ -443,45 +459,86 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
 #pragma unroll
       for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[i], wf[j]);
   };
-  // Wait until at most `tiles` k-tiles of this wave's copies are in flight (copies finish in order), then
-  // meet the other waves. The count is an immediate of the instruction, hence the cases.
+  // Wait until at most `count` of this wave's copies are in flight (copies finish in order), then meet the
+  // other waves. The count is an immediate of the instruction, hence the cases.
 #define TW_DMA_WAIT(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)" ::: "memory")
-#define TW_DMA_PUBLISH(tiles)                                                 \
+#define TW_DMA_PUBLISH(count)                                                 \
   do {                                                                        \
-    if constexpr (COPIES * (tiles) == 8) TW_DMA_WAIT(8);                      \
-    else if constexpr (COPIES * (tiles) == 12) TW_DMA_WAIT(12);               \
-    else if constexpr (COPIES * (tiles) == 14) TW_DMA_WAIT(14);               \
-    else if constexpr (COPIES * (tiles) == 21) TW_DMA_WAIT(21);               \
-    else if constexpr (COPIES * (tiles) == 16) TW_DMA_WAIT(16);               \
-    else if constexpr (COPIES * (tiles) == 18) TW_DMA_WAIT(18);               \
-    else if constexpr (COPIES * (tiles) == 24) TW_DMA_WAIT(24);               \
+    if constexpr ((count) == 8) TW_DMA_WAIT(8);                               \
+    else if constexpr ((count) == 10) TW_DMA_WAIT(10);                        \
+    else if constexpr ((count) == 12) TW_DMA_WAIT(12);                        \
+    else if constexpr ((count) == 14) TW_DMA_WAIT(14);                        \
+    else if constexpr ((count) == 16) TW_DMA_WAIT(16);                        \
+    else if constexpr ((count) == 18) TW_DMA_WAIT(18);                        \
+    else if constexpr ((count) == 20) TW_DMA_WAIT(20);                        \
+    else if constexpr ((count) == 21) TW_DMA_WAIT(21);                        \
+    else if constexpr ((count) == 24) TW_DMA_WAIT(24);                        \
     else TW_DMA_WAIT(0);                                                      \
     __builtin_amdgcn_s_barrier();                                             \
     asm volatile("" ::: "memory");                                            \
   } while (0)
 #define TW_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-  // the order asked of the scheduler: G groups of (copies, fragment reads, MFMAs) per k-chunk pair
-  constexpr int G = (WM + WN) % 2 ? 1 : (WM * WN >= 16 ? 4 : 2);
 
   bf16x8 af[2][WM], wf[2][WN];
+  // One wave a SIMD issues in order, and the matrix unit takes an MFMA every 32 clocks: whatever else
+  // the wave issues between two MFMAs has to fit into that time, or the unit idles. So the other
+  // operations of a k-chunk pair follow its MFMAs one by one: first the fragment reads of the next pair
+  // (into the other set of registers), then the copies: the W blocks of k-tile t + 3 in the first pair of
+  // iteration t, the A blocks of k-tile t + 4 in the second (the stage those land in was freed by the
+  // barrier between the two pairs). The last MFMAs of a pair have nothing behind them: a copy counts as an
+  // access through both memory counters, after which every wait the compiler puts before an MFMA whose
+  // operands came from LDS is `lgkmcnt(0)`, and the one before the next pair's first MFMA should find the
+  // reads long done. The source is written in the order that is wanted, because a copy writes LDS and the
+  // compiler keeps LDS reads on their side of it; the group barriers only pin it.
+  auto copy_one = [&](const bf16_t* src, int t_v, int elems_per_tile, int block) {
+    const int t = min(t_v, k_tiles - 1);                   // past the end: a copy nobody reads
+    char* stage = lds + (t_v % TW_DMA_STAGES) * STAGE;
+    __builtin_amdgcn_global_load_lds(src + (size_t)t * elems_per_tile, (tw_lds_ptr)(stage + block * 1024), 16, 0, 0);
+  };
+  auto half = [&](int t_copy, auto copy_is_a, int t_read, const int cc_read, bf16x8* af_in, bf16x8* wf_in,
+                  bf16x8* af_out, bf16x8* wf_out) {
+    constexpr bool IS_A = decltype(copy_is_a)::value;
+    constexpr int NCOPY = IS_A ? WM : WN;
+    const int st = (t_read % TW_DMA_STAGES) * STAGE;
+    // S slots of one MFMA each; the Q other operations (R fragment reads, then the copies) follow the
+    // MFMAs of the first slots one by one (two where there are more operations than slots)
+    constexpr int S = WM * WN, R = WM + WN, Q = R + NCOPY;
+    tw_unroll<S>([&](auto index) {
+      constexpr int slot = decltype(index)::value, i = slot / WN, j = slot % WN;
+      tw_mma32(acc[i][j], af_in[i], wf_in[j]);
+      constexpr int q0 = Q <= S ? (slot < Q ? slot : Q) : slot * Q / S;
+      constexpr int q1 = Q <= S ? (slot + 1 < Q ? slot + 1 : Q) : (slot + 1) * Q / S;
+#pragma unroll
+      for (int q = q0; q < q1; ++q) {
+        if (q < WM) af_out[q] = *reinterpret_cast<const bf16x8*>(a_frag_cc[cc_read] + st + q * 2048);
+        else if (q < R) wf_out[q - WM] = *reinterpret_cast<const bf16x8*>(w_frag + st + cc_read * 512 + (q - WM) * 2048);
+        else if (IS_A) copy_one(a_src[q - R], t_copy, 32, WM * wave + (q - R));
+        else copy_one(w_src[q - R], t_copy, 512, BM / 16 + WN * wave + (q - R));
+      }
+      constexpr int reads_here = (q1 < R ? q1 : R) - (q0 < R ? q0 : R), copies_here = (q1 - q0) - reads_here;
+      TW_SGB(0x008, 1);
+      if constexpr (reads_here > 0) TW_SGB(0x100, reads_here);
+      if constexpr (copies_here > 0) TW_SGB(0x020, copies_here);
+    });
+  };
   if (k_tiles > 0) {
 #pragma unroll
-    for (int t = 0; t < TW_DMA_STAGES; ++t) copy_tile(t);
-    TW_DMA_PUBLISH(3);                                     // k-tile 0 has landed, for every wave
+    for (int t = 0; t < TW_DMA_STAGES - 1; ++t) {
+      copy_a(t);
+      copy_w(t);
+    }
+    copy_a(TW_DMA_STAGES - 1);
+    TW_DMA_PUBLISH(2 * COPIES + WM);                       // k-tile 0 has landed, for every wave
     read_frags(0, 0, af[0], wf[0]);
     for (int t = 0; t < k_tiles; ++t) {
-      read_frags(t, 1, af[1], wf[1]);
-      multiply(af[0], wf[0]);
-#pragma unroll
-      for (int q = 0; q < G; ++q) { TW_SGB(0x100, (WM + WN) / G); TW_SGB(0x008, WM * WN / G); }
+      half(t + TW_DMA_STAGES - 1, std::false_type{}, t, 1, af[0], wf[0], af[1], wf[1]);
       // every fragment of k-tile t is in registers now; k-tile t + 1 (copies of t + 2 and t + 3 may
-      // still be in flight) becomes visible, and t's stage is free for t + 4
-      TW_DMA_PUBLISH(2);
-      copy_tile(t + TW_DMA_STAGES);
-      read_frags(t + 1, 0, af[0], wf[0]);                  // (after the last k-tile: read, never used)
-      multiply(af[1], wf[1]);
-#pragma unroll
-      for (int q = 0; q < G; ++q) { TW_SGB(0x020, COPIES / G); TW_SGB(0x100, (WM + WN) / G); TW_SGB(0x008, WM * WN / G); }
+      // still be in flight) becomes visible, and t's stage is free for the A blocks of t + 4
+      __builtin_amdgcn_sched_barrier(0);                   // (nothing of either half moves across the barrier)
+      TW_DMA_PUBLISH(2 * COPIES);
+      __builtin_amdgcn_sched_barrier(0);
+      half(t + TW_DMA_STAGES, std::true_type{}, t + 1, 0, af[1], wf[1], af[0], wf[0]);   // (after the last k-tile: read, never used)
+      __builtin_amdgcn_sched_barrier(0);                   // (nor into the next iteration)
     }
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // no copy may land in the epilogue's staging area
@@ -579,6 +636,8 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
   if (mode) mode->splits = splits;
   const long n_blocks = (long)tiles_m * tiles_n * splits;
   TW_REQUIRE(n_blocks < (1L << 30));
+  // offsets within a tile's operands are 32-bit
+  TW_REQUIRE((long)BM * lda * 2 < (1L << 31) && (long)(BN / 16) * ldw * 1024 < (1L << 31));
   const int grid = (int)((n_blocks + 7) / 8 * 8);
   const size_t pipeline_bytes = TW_DMA_STAGES * (size_t)(BM + BN) * 64;
   const size_t epilogue_bytes = 4 * 32 * (size_t)(32 * WN + 4) * 4;
