@@ -337,19 +337,24 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ A
 // Workgroup = 4 waves in a 2x2 grid, wave tile (32*WM) x (32*WN): 128x128 (two workgroups a CU),
 // 128x256, 256x256 (one a CU, the accumulators in AGPRs).
 //
-// A k-tile is 32 elements of K (64 bytes a row, one k-step of the shuffled layout). A stage of
-// LDS holds the tile's blocks of A, then those of W; a block is 16 rows x 4 chunks of 16 bytes,
-// 1 KB. A W block is [chunk][row], which is how W lies in memory (a fragment read takes 256
-// consecutive bytes per 16 lanes); an A block is [row][chunk] with the chunks of a row swizzled
-// (see a_src below). Four stages: the copy of k-tile t+4 starts when k-tile t is in registers.
+// A k-tile is 32 elements of K (one k-step of the shuffled layout). What limits this kernel is the
+// number of 128-byte lines a CU's vector cache can have on their way from L2; a copy that takes 64 bytes
+// of a row of A brings in the whole line, and by the time the next k-tile wants the other half the line
+// is gone again (measured: 1.5 lines fetched per line used). So A is copied in PAIRS of k-tiles, a
+// whole line per row: a copy is 8 rows x 128 bytes, and LDS holds TW_DMA_A_SLOTS slots of BM rows x 128
+// bytes. In a slot row `row` keeps its 16-byte chunk c (0..3: the even k-tile, 4..7: the odd one) at
+// position c ^ (row / 2 % 8), so that the 16 rows one fragment read takes lie in 16 different 16-byte
+// columns. W is copied per k-tile into 4 stages; a W block is 16 rows x 4 chunks, [chunk][row], 1 KB,
+// which is how W lies in memory (a fragment read takes 256 consecutive bytes per 16 lanes).
 //
 // Per k-tile and wave: 2 k-chunk pairs of WM*WN MFMAs. The fragments of a pair are read while the
 // pair before is multiplied, so the barrier that publishes the next k-tile lies between the two
 // pairs of this one and the matrix unit has work queued on both sides of it.
-// splits > 1: as in gemm_tiled_kernel.
+// splits > 1: as in gemm_tiled_kernel (a split's k-tiles begin at an even one).
 // =====================================================================================
 typedef __attribute__((address_space(3))) void* tw_lds_ptr;
-#define TW_DMA_STAGES 4
+#define TW_DMA_STAGES 4       /* of W, one k-tile each */
+#define TW_DMA_A_SLOTS 3      /* of A, a pair of k-tiles each */
 
 // f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a constant
 // expression in the body (the scheduler's group barriers take constants only)
@@ -369,8 +374,11 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
                                                        long ldr, OutT* C, long ldc, int M, int N, int K,
                                                        int tiles_m, int n_blocks, int splits,
                                                        float* __restrict__ partial) {
+  static_assert(WM % 2 == 0, "the tail fix below assumes an even number of A copies per group");
   constexpr int BM = 64 * WM, BN = 64 * WN;
-  constexpr int STAGE = (BM + BN) * 64;                 // bytes: A blocks, then W blocks
+  constexpr int A_SLOT = BM * 128;                      // bytes: a pair of k-tiles of A
+  constexpr int W_STAGE = BN * 64;                      // bytes: one k-tile of W
+  constexpr int W_RING = TW_DMA_A_SLOTS * A_SLOT;       // the W stages lie behind the A slots
   constexpr int COPIES = WM + WN;                       // 1 KB copies per wave and k-tile
   extern __shared__ __attribute__((aligned(16))) char lds[];
   const int per_xcd = gridDim.x / 8;
@@ -399,80 +407,75 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // this workgroup's k-tiles: kt0 .. kt0 + k_tiles - 1
+  // this workgroup's k-tiles: kt0 .. kt0 + k_tiles - 1, kt0 even (a pair of k-tiles is never divided)
   const int k_tiles_all = K / 32;
-  const int per_split = (k_tiles_all + splits - 1) / splits;
+  const int per_split = ((k_tiles_all + splits - 1) / splits + 1) & ~1;
   const int kt0 = split * per_split;
   const int k_tiles = max(0, min(k_tiles_all, kt0 + per_split) - kt0);
+  const int pairs = (k_tiles + 1) / 2;
+  const bool half_pair = (k_tiles & 1) != 0;               // the last pair has its even k-tile only
 
-  // What this lane copies per k-tile: its slot of A blocks WM wave .. WM wave + WM - 1 and of W blocks
+  // What this lane copies: per pair of k-tiles its slot of the A blocks (8 rows each) 2 WM wave ..
+  // 2 WM wave + 2 WM - 1, in two groups of WM, and per k-tile its slot of the W blocks (16 rows each)
   // WN wave .. WN wave + WN - 1. Rows past M and blocks past N are clamped to the last valid one (their
   // products are never stored).
   const int n_blocks_w = (N + 15) / 16;
-  const bf16_t* a_src[4];                                  // (WM of them are used)
-  const bf16_t* w_src[4];                                  // (WN)
-  {
-    // slot l of an A block holds row l / 4, chunk (l % 4) ^ (row / 4 % 4): four neighbouring lanes fetch
-    // 64 consecutive bytes, and 16 rows of one chunk lie in 16 different 16-byte columns of LDS
-    const int row16 = lane >> 2, chunk = (lane & 3) ^ ((row16 >> 2) & 3);
+  // (A: byte offsets from the tile's first row, for group 0 and from group 0 to group 1; which group a
+  // copy belongs to is not known where it is compiled, and a choice between two pointers would put them
+  // into memory)
+  const char* const a_base = reinterpret_cast<const char*>(A + (size_t)m0 * lda + (size_t)kt0 * 32);
+  int a_off[WM], a_step[WM];
+  const bf16_t* w_src[WN];
 #pragma unroll
-    for (int b = 0; b < WM; ++b) {
-      const int row = min(m0 + (WM * wave + b) * 16 + row16, M - 1);
-      a_src[b] = A + (size_t)row * lda + (size_t)kt0 * 32 + chunk * 8;
-    }
+  for (int b = 0; b < WM; ++b) {
+    int off[2];
 #pragma unroll
-    for (int b = 0; b < WN; ++b) {
-      const int blk = min(n0 / 16 + WN * wave + b, n_blocks_w - 1);
-      w_src[b] = W + ((size_t)blk * k_steps + kt0) * 512 + lane * 8;
+    for (int grp = 0; grp < 2; ++grp) {
+      const int row_in_tile = ((2 * WM) * wave + grp * WM + b) * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ ((row_in_tile >> 1) & 7);   // slot l % 8 of the row holds this chunk
+      off[grp] = min(row_in_tile, M - 1 - m0) * (int)lda * 2 + chunk * 16;
     }
+    a_off[b] = off[0];
+    a_step[b] = off[1] - off[0];
   }
-  // k-tile kt0 + t_v into stage t_v % 4, in two halves: the A blocks and the W blocks
-  auto copy_a = [&](int t_v) {
-    const int t = min(t_v, k_tiles - 1);                   // past the end: a copy nobody reads
-    char* stage = lds + (t_v % TW_DMA_STAGES) * STAGE;
 #pragma unroll
-    for (int b = 0; b < WM; ++b)
-      __builtin_amdgcn_global_load_lds(a_src[b] + (size_t)t * 32, (tw_lds_ptr)(stage + (WM * wave + b) * 1024), 16, 0, 0);
+  for (int b = 0; b < WN; ++b) {
+    const int blk = min(n0 / 16 + WN * wave + b, n_blocks_w - 1);
+    w_src[b] = W + ((size_t)blk * k_steps + kt0) * 512 + lane * 8;
+  }
+  // In a last pair that has its even k-tile only, the lanes that would fetch chunks 4..7 (past the end of
+  // the row, and for the last row perhaps of the matrix) fetch chunks 0..3 again. Whether a lane's chunk
+  // is 4..7: bit 2 of l % 8, flipped in every other block of 8 rows.
+  const int tail_back[2] = {(lane & 4) ? -64 : 0, (lane & 4) ? 0 : -64};   // bytes
+  auto copy_a_one = [&](int pair_v, int grp, int b) {       // (grp, 0 or 1, is the same for the whole wave)
+    const int pair = min(pair_v, pairs - 1);               // past the end: a copy nobody reads
+    const int tail = (half_pair && pair == pairs - 1) ? -1 : 0;
+    char* slot = lds + (pair_v % TW_DMA_A_SLOTS) * A_SLOT;
+    const int off = a_off[b] + (a_step[b] & -grp) + (tail_back[b & 1] & tail);
+    __builtin_amdgcn_global_load_lds((const void*)(a_base + (size_t)pair * 128 + (long)off),
+                                     (tw_lds_ptr)(slot + ((2 * WM) * wave + grp * WM + b) * 1024), 16, 0, 0);
   };
-  auto copy_w = [&](int t_v) {
+  auto copy_w_one = [&](int t_v, int b) {
     const int t = min(t_v, k_tiles - 1);
-    char* stage = lds + (t_v % TW_DMA_STAGES) * STAGE;
-#pragma unroll
-    for (int b = 0; b < WN; ++b)
-      __builtin_amdgcn_global_load_lds(w_src[b] + (size_t)t * 512, (tw_lds_ptr)(stage + BM * 64 + (WN * wave + b) * 1024), 16, 0, 0);
+    char* stage = lds + W_RING + (t_v % TW_DMA_STAGES) * W_STAGE;
+    __builtin_amdgcn_global_load_lds((const void*)(w_src[b] + (size_t)t * 512), (tw_lds_ptr)(stage + (WN * wave + b) * 1024), 16, 0, 0);
   };
-  // this lane's fragment addresses in stage 0
-  const int a_row16 = r & 15, a_swz = (a_row16 >> 2) & 3;
-  const char* a_block = lds + (wm0 / 16 + (r >> 4)) * 1024 + a_row16 * 64;
-  const char* a_frag_cc[2] = {a_block + ((g ^ a_swz) * 16), a_block + (((2 + g) ^ a_swz) * 16)};
-  const char* w_frag = lds + BM * 64 + (wn0 / 16 + (r >> 4)) * 1024 + g * 256 + (r & 15) * 16;
-  auto read_frags = [&](int t, int cc, bf16x8* af, bf16x8* wf) {
-    const int st = (t % TW_DMA_STAGES) * STAGE;
-#pragma unroll
-    for (int i = 0; i < WM; ++i) af[i] = *reinterpret_cast<const bf16x8*>(a_frag_cc[cc] + st + i * 2048);
-#pragma unroll
-    for (int j = 0; j < WN; ++j) wf[j] = *reinterpret_cast<const bf16x8*>(w_frag + st + cc * 512 + j * 2048);
-  };
-  auto multiply = [&](const bf16x8* af, const bf16x8* wf) {
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j) tw_mma32(acc[i][j], af[i], wf[j]);
-  };
+  // this lane's fragment offsets: A in slot 0 for the k-chunk pairs of an even k-tile (an odd one's
+  // chunks are 4 further on: bit 6 of the offset flipped), W in stage 0
+  const int a_swz = (r >> 1) & 7;
+  const int a_frag[2] = {(wm0 + r) * 128 + ((g ^ a_swz) * 16), (wm0 + r) * 128 + (((2 + g) ^ a_swz) * 16)};
+  const char* w_frag = lds + W_RING + (wn0 / 16 + (r >> 4)) * 1024 + g * 256 + (r & 15) * 16;
   // Wait until at most `count` of this wave's copies are in flight (copies finish in order), then meet the
   // other waves. The count is an immediate of the instruction, hence the cases.
 #define TW_DMA_WAIT(n) asm volatile("s_waitcnt vmcnt(" #n ") lgkmcnt(0)" ::: "memory")
 #define TW_DMA_PUBLISH(count)                                                 \
   do {                                                                        \
-    if constexpr ((count) == 8) TW_DMA_WAIT(8);                               \
+    if constexpr ((count) == 6) TW_DMA_WAIT(6);                               \
+    else if constexpr ((count) == 8) TW_DMA_WAIT(8);                          \
     else if constexpr ((count) == 10) TW_DMA_WAIT(10);                        \
     else if constexpr ((count) == 12) TW_DMA_WAIT(12);                        \
     else if constexpr ((count) == 14) TW_DMA_WAIT(14);                        \
     else if constexpr ((count) == 16) TW_DMA_WAIT(16);                        \
-    else if constexpr ((count) == 18) TW_DMA_WAIT(18);                        \
-    else if constexpr ((count) == 20) TW_DMA_WAIT(20);                        \
-    else if constexpr ((count) == 21) TW_DMA_WAIT(21);                        \
-    else if constexpr ((count) == 24) TW_DMA_WAIT(24);                        \
     else TW_DMA_WAIT(0);                                                      \
     __builtin_amdgcn_s_barrier();                                             \
     asm volatile("" ::: "memory");                                            \
@@ -484,22 +487,17 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
   // the wave issues between two MFMAs has to fit into that time, or the unit idles. So the other
   // operations of a k-chunk pair follow its MFMAs one by one: first the fragment reads of the next pair
   // (into the other set of registers), then the copies: the W blocks of k-tile t + 3 in the first pair of
-  // iteration t, the A blocks of k-tile t + 4 in the second (the stage those land in was freed by the
-  // barrier between the two pairs). The last MFMAs of a pair have nothing behind them: a copy counts as an
-  // access through both memory counters, after which every wait the compiler puts before an MFMA whose
-  // operands came from LDS is `lgkmcnt(0)`, and the one before the next pair's first MFMA should find the
-  // reads long done. The source is written in the order that is wanted, because a copy writes LDS and the
-  // compiler keeps LDS reads on their side of it; the group barriers only pin it.
-  auto copy_one = [&](const bf16_t* src, int t_v, int elems_per_tile, int block) {
-    const int t = min(t_v, k_tiles - 1);                   // past the end: a copy nobody reads
-    char* stage = lds + (t_v % TW_DMA_STAGES) * STAGE;
-    __builtin_amdgcn_global_load_lds(src + (size_t)t * elems_per_tile, (tw_lds_ptr)(stage + block * 1024), 16, 0, 0);
-  };
-  auto half = [&](int t_copy, auto copy_is_a, int t_read, const int cc_read, bf16x8* af_in, bf16x8* wf_in,
-                  bf16x8* af_out, bf16x8* wf_out) {
+  // k-tile t, one group of the A blocks of k-tile pair t / 2 + 2 in the second (the slot those land in
+  // held pair t / 2 - 1, last read before the barrier of k-tile 2 (t / 2) - 1). The last MFMAs of a pair
+  // have nothing behind them: a copy counts as an access through both memory counters, after which every
+  // wait the compiler puts before an MFMA whose operands came from LDS is `lgkmcnt(0)`, and the one before
+  // the next pair's first MFMA should find the reads long done. The source is written in the order that
+  // is wanted, because a copy writes LDS and the compiler keeps LDS reads on their side of it; the group
+  // barriers only pin it.
+  auto half = [&](auto copy_is_a, int copy_index, int copy_group, const char* a_read, const char* w_read,
+                  bf16x8* af_in, bf16x8* wf_in, bf16x8* af_out, bf16x8* wf_out) {
     constexpr bool IS_A = decltype(copy_is_a)::value;
     constexpr int NCOPY = IS_A ? WM : WN;
-    const int st = (t_read % TW_DMA_STAGES) * STAGE;
     // S slots of one MFMA each; the Q other operations (R fragment reads, then the copies) follow the
     // MFMAs of the first slots one by one (two where there are more operations than slots)
     constexpr int S = WM * WN, R = WM + WN, Q = R + NCOPY;
@@ -510,10 +508,10 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
       constexpr int q1 = Q <= S ? (slot + 1 < Q ? slot + 1 : Q) : (slot + 1) * Q / S;
 #pragma unroll
       for (int q = q0; q < q1; ++q) {
-        if (q < WM) af_out[q] = *reinterpret_cast<const bf16x8*>(a_frag_cc[cc_read] + st + q * 2048);
-        else if (q < R) wf_out[q - WM] = *reinterpret_cast<const bf16x8*>(w_frag + st + cc_read * 512 + (q - WM) * 2048);
-        else if (IS_A) copy_one(a_src[q - R], t_copy, 32, WM * wave + (q - R));
-        else copy_one(w_src[q - R], t_copy, 512, BM / 16 + WN * wave + (q - R));
+        if (q < WM) af_out[q] = *reinterpret_cast<const bf16x8*>(a_read + q * 4096);
+        else if (q < R) wf_out[q - WM] = *reinterpret_cast<const bf16x8*>(w_read + (q - WM) * 2048);
+        else if (IS_A) copy_a_one(copy_index, copy_group, q - R);
+        else copy_w_one(copy_index, q - R);
       }
       constexpr int reads_here = (q1 < R ? q1 : R) - (q0 < R ? q0 : R), copies_here = (q1 - q0) - reads_here;
       TW_SGB(0x008, 1);
@@ -521,25 +519,42 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16_t* __restrict_
       if constexpr (copies_here > 0) TW_SGB(0x020, copies_here);
     });
   };
+  // k-tile t. Its barrier publishes k-tile t + 1. What has to have landed by then and what this wave
+  // has issued since: t + 1 odd: W of t + 1 (issued in the first pair of t - 2), since then A, W A, W;
+  // t + 1 even: its pair of A, whose second group went out in the second pair of t - 2, since then W A, W.
+  // One count for both (the parity of t is not known where the wait is compiled): the smaller.
+  auto k_tile = [&](int t) {
+    const int odd = t & 1;
+    const int a_now = ((t >> 1) % TW_DMA_A_SLOTS) * A_SLOT, a_next = (((t + 1) >> 1) % TW_DMA_A_SLOTS) * A_SLOT;
+    const int w_now = (t % TW_DMA_STAGES) * W_STAGE, w_next = ((t + 1) % TW_DMA_STAGES) * W_STAGE;
+    half(std::false_type{}, t + TW_DMA_STAGES - 1, 0, lds + ((a_frag[1] ^ (odd << 6)) + a_now), w_frag + w_now + 512,
+         af[0], wf[0], af[1], wf[1]);
+    __builtin_amdgcn_sched_barrier(0);                     // (nothing of either pair moves across the barrier)
+    TW_DMA_PUBLISH(2 * WN + WM);
+    __builtin_amdgcn_sched_barrier(0);
+    half(std::true_type{}, (t >> 1) + 2, odd, lds + ((a_frag[0] ^ ((odd ^ 1) << 6)) + a_next), w_frag + w_next,
+         af[1], wf[1], af[0], wf[0]);                      // (after the last k-tile: read, never used)
+    __builtin_amdgcn_sched_barrier(0);                     // (nor into the next k-tile)
+  };
   if (k_tiles > 0) {
+    // A of pair 0 and W of k-tile 0, then what may still be on its way when k-tile 0 is published:
+    // W of k-tile 1, A of pair 1, W of k-tile 2
 #pragma unroll
-    for (int t = 0; t < TW_DMA_STAGES - 1; ++t) {
-      copy_a(t);
-      copy_w(t);
-    }
-    copy_a(TW_DMA_STAGES - 1);
-    TW_DMA_PUBLISH(2 * COPIES + WM);                       // k-tile 0 has landed, for every wave
-    read_frags(0, 0, af[0], wf[0]);
-    for (int t = 0; t < k_tiles; ++t) {
-      half(t + TW_DMA_STAGES - 1, std::false_type{}, t, 1, af[0], wf[0], af[1], wf[1]);
-      // every fragment of k-tile t is in registers now; k-tile t + 1 (copies of t + 2 and t + 3 may
-      // still be in flight) becomes visible, and t's stage is free for the A blocks of t + 4
-      __builtin_amdgcn_sched_barrier(0);                   // (nothing of either half moves across the barrier)
-      TW_DMA_PUBLISH(2 * COPIES);
-      __builtin_amdgcn_sched_barrier(0);
-      half(t + TW_DMA_STAGES, std::true_type{}, t + 1, 0, af[1], wf[1], af[0], wf[0]);   // (after the last k-tile: read, never used)
-      __builtin_amdgcn_sched_barrier(0);                   // (nor into the next iteration)
-    }
+    for (int c = 0; c < 2 * WM; ++c) copy_a_one(0, c / WM, c % WM);
+#pragma unroll
+    for (int b = 0; b < WN; ++b) copy_w_one(0, b);
+#pragma unroll
+    for (int b = 0; b < WN; ++b) copy_w_one(1, b);
+#pragma unroll
+    for (int c = 0; c < 2 * WM; ++c) copy_a_one(1, c / WM, c % WM);
+#pragma unroll
+    for (int b = 0; b < WN; ++b) copy_w_one(2, b);
+    TW_DMA_PUBLISH(2 * COPIES);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) af[0][i] = *reinterpret_cast<const bf16x8*>(lds + a_frag[0] + i * 4096);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) wf[0][j] = *reinterpret_cast<const bf16x8*>(w_frag + j * 2048);
+    for (int t = 0; t < k_tiles; ++t) k_tile(t);
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");   // no copy may land in the epilogue's staging area
 #undef TW_SGB
@@ -639,7 +654,8 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
   // offsets within a tile's operands are 32-bit
   TW_REQUIRE((long)BM * lda * 2 < (1L << 31) && (long)(BN / 16) * ldw * 1024 < (1L << 31));
   const int grid = (int)((n_blocks + 7) / 8 * 8);
-  const size_t pipeline_bytes = TW_DMA_STAGES * (size_t)(BM + BN) * 64;
+  const size_t pipeline_bytes = TW_DMA_A_SLOTS * (size_t)BM * 128 + TW_DMA_STAGES * (size_t)BN * 64;
+  static_assert(TW_DMA_A_SLOTS * BM * 128 + TW_DMA_STAGES * BN * 64 <= 160 * 1024, "a workgroup has 160 KB of LDS");
   const size_t epilogue_bytes = 4 * 32 * (size_t)(32 * WN + 4) * 4;
   const size_t lds_bytes = pipeline_bytes > epilogue_bytes ? pipeline_bytes : epilogue_bytes;
   auto kernel = gemm_dma_kernel<OutT, WM, WN, GLU>;
@@ -667,7 +683,7 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
 #define TW_DMA_SHAPES 0xC      /* bit s: shape s uses the direct-to-LDS kernel (at 128x128 it gains nothing) */
 #endif
 static const int kTileM[5] = {0, 128, 128, 256, 256}, kTileN[5] = {0, 128, 256, 256, 192};
-static const double kTileRate[5] = {0, 0.80, 0.93, 1.15, 1.00};
+static const double kTileRate[5] = {0, 0.76, 0.90, 1.05, 1.00};
 
 static int choose_shape(bool big_ok, int M, int N) {
   if (!big_ok) return 1;
