@@ -24,6 +24,7 @@
 //                        of each); partial results are merged in a fixed order.
 //   attn_prefill_kernel  rows = (token, head) pairs of a prompt portion; each
 //                        wave walks the keys its rows can see.
+#include <type_traits>
 #include "tw_common.h"
 
 template <typename T> __device__ __forceinline__ float tw_exp(float v);
@@ -622,7 +623,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a) {
 // K or V fragment a wave reads from LDS serves both of its 16-row tiles.
 // Key/row layout inside a block as in the decode kernel above.
 // =====================================================================================
-#define TW_PF_VROW 80                       /* LDS bytes per value row (32 keys = 64 B, padded) */
+#define TW_PF_VROW 64                       /* LDS bytes per value row (32 keys; the 16-byte pieces of row d lie at piece ^ (d / 4 % 4)) */
+#define TW_PF_SLACK 8.f                     /* how far, in powers of two, a score may exceed the reference of its row before that is moved */
+#define TW_PF_STAGES 3                      /* blocks in LDS: the one whose probabilities are formed, the one whose scores are, the one being written */
 
 
 // EXACT: head_dim == 16 * DTMAX, so every loop over the head has compile-time bounds (with run-time
@@ -641,7 +644,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   constexpr bool ALL_USED = EXACT && (32 * CH) % 256 == 0 && (DTMAX * 16 * 4) % 256 == 0;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   char* lds_k = lds;
-  char* lds_v = lds + 2 * KSTAGE;
+  char* lds_v = lds + TW_PF_STAGES * KSTAGE;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // the same for the wave's lanes: what follows from it stays scalar
@@ -752,7 +755,10 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     const int key_c = min(key, 31), chunk_c = min(chunk, chunks - 1);   // an unused piece loads a used one's bytes
     k_slot[i] = P >= 32 ? 0 : (key_c >> pshift);           // which of the block's pages
     k_goff[i] = (P >= 32 ? key_c : (key_c & pmask)) * D + chunk_c * 8;
-    k_loff[i] = key * KROW + chunk * 16;
+    // key k lies in LDS row (k / 8 % 4) * 4 + k % 4 + 16 * (k / 4 % 2): the 16 keys whose scores one MFMA
+    // forms (k % 8 < 4, or >= 4) are 16 consecutive rows, which with the odd row length (in 16-byte units)
+    // a fragment read finds in 16 different 16-byte columns of the banks
+    k_loff[i] = (((key >> 3) & 3) * 4 + (key & 3) + 16 * ((key >> 2) & 1)) * KROW + chunk * 16;
   }
 #pragma unroll
   for (int i = 0; i < VPIECES; ++i) {
@@ -761,7 +767,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     v_oct[i] = oct;
     v_slot[i] = P >= 32 ? 0 : ((8 * oct) >> pshift);
     v_goff[i] = min(d, D - 1) * P + (P >= 32 ? 8 * oct : ((8 * oct) & pmask));
-    v_loff[i] = d * TW_PF_VROW + oct * 16;
+    v_loff[i] = d * TW_PF_VROW + ((oct ^ ((d >> 2) & 3)) * 16);
   }
   // global -> registers. Loads carry no predicate: a page of the block that holds no key of
   // [lo, kv_len) may not be held at all and is replaced by one of the block that is, so every
@@ -838,20 +844,23 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const char* k_frag[2];
 #pragma unroll
   for (int tile = 0; tile < 2; ++tile)
-    k_frag[tile] = lds_k + (8 * (r >> 2) + 4 * tile + (r & 3)) * KROW + g * 16;
-  const char* v_frag = lds_v + r * TW_PF_VROW + g * 16;
+    k_frag[tile] = lds_k + (16 * tile + r) * KROW + g * 16;   // (lane r's key of the tile: 8 (r / 4) + 4 tile + r % 4)
+  const char* v_frag = lds_v + r * TW_PF_VROW + ((g ^ ((r >> 2) & 3)) * 16);
 
+  // A block is worked on in two steps, one iteration apart: its SCORES, S^T = K Q^T, and, an iteration
+  // later, the softmax of those and the PV products. In an iteration the scores of block b + 1 (matrix
+  // unit) and the softmax of block b (vector unit) do not depend on each other, so one wave keeps both
+  // units busy; with both in one step the two took turns.
   // edge: some key of the block is hidden from some row of the wave; only then are scores masked.
-  // The branch covers the masking alone, so the two cases share every register of the rest.
-  auto compute = [&](int blk, int buf, bool edge) {
+  // (with the largest heads and 128-row tiles the two steps stay in one iteration: there are not the
+  // registers for two blocks' scores beside the output)
+  constexpr bool PIPELINED = DTMAX * RT <= 16;
+  auto scores = [&](int blk, int buf, bool edge, f32x4 (&s)[RT][2]) {
     const int p0 = blk * 32;
-    f32x4 s[RT][2];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int tile = 0; tile < 2; ++tile) s[rt][tile] = f32x4{0.f, 0.f, 0.f, 0.f};
-    // every key fragment of the block is asked for before the first is multiplied, and the value
-    // fragments before the softmax, so that LDS latency passes behind other work
     bf16x8 kf[2][NSMAX];
 #pragma unroll
     for (int tile = 0; tile < 2; ++tile) {
@@ -870,11 +879,6 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         if (EXACT || st * 4 < chunks)
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt) tw_mma16(s[rt][tile], kf[tile][st], qf[rt][st]);
-    const char* vbase = v_frag + buf * VSTAGE;
-    bf16x8 vf[DTMAX];
-#pragma unroll
-    for (int dt = 0; dt < DTMAX; ++dt)
-      if (EXACT || dt < dts) vf[dt] = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
     if (edge) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
@@ -886,17 +890,36 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         }
       }
     }
-    // Row tile by row tile: softmax, rescaling if the maximum moved, PV products. The products of one row
-    // tile do not depend on the softmax of the next, so the matrix unit works on them meanwhile
-    // (8,192 tokens: 2 % faster than all softmaxes first and all products after).
+  };
+  // Row tile by row tile: softmax, rescaling if the maximum moved, PV products. The products of one row
+  // tile do not depend on the softmax of the next, so the matrix unit works on them meanwhile.
+  // mixed: the scores of the next block are formed in the same stretch of code; the scheduler is asked to
+  // issue the MFMAs that do not depend on this softmax (those scores, then the first row tile's products)
+  // one by one between its vector instructions: a wave issues in order, and MFMAs issued in a row keep it
+  // from issuing anything else until the last has been taken.
+  auto finish = [&](int buf, f32x4 (&s)[RT][2], auto mixed) {
+    constexpr bool MIXED = decltype(mixed)::value;
+    const char* vbase = v_frag + buf * VSTAGE;
+    bf16x8 vf[DTMAX];
+#pragma unroll
+    for (int dt = 0; dt < DTMAX; ++dt)
+      if (EXACT || dt < dts) vf[dt] = *reinterpret_cast<const bf16x8*>(vbase + dt * 16 * TW_PF_VROW);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float mx = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 8; ++e) mx = fmaxf(mx, s[rt][e >> 2][e & 3]);
       mx = tw_rows_max(mx);
-      // m is kept in the scaled log2 domain: m = max(score) * c2 (c2 > 0)
-      const float m_new = fmaxf(m[rt], mx * c2);
+      // m, in the scaled log2 domain (score * c2, c2 > 0), is the REFERENCE the exponentials are taken
+      // against: the row's largest score when it was last moved, and it is moved only when a score
+      // exceeds it by more than TW_PF_SLACK (then the running sum and output are rescaled). Until then
+      // probabilities may be as large as 2^TW_PF_SLACK instead of 1; sum and output are relative to the
+      // same reference, so their quotient is what it would be against the true maximum, float32 and
+      // bfloat16 keep their relative precision at that size, and the rescaling, which makes all four
+      // waves of the workgroup wait for the one that does it, happens in the first block of a row tile
+      // and hardly ever again instead of in every third block of a long prompt.
+      const float cand = mx * c2;
+      const float m_new = cand > m[rt] + TW_PF_SLACK ? cand : m[rt];
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);
       float sum = 0.f;
@@ -911,38 +934,116 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       // once, after the loop
       l[rt] = l[rt] * alpha + sum;
       m[rt] = m_new;
+      if constexpr (MIXED) {
+        // (the probabilities are wanted here, before the branch below: the compiler would form them
+        // behind it, where only the products wait for them, and nothing could be mixed with them)
+        asm volatile("" : "+v"(pb), "+v"(l[rt]));
+        if (rt == 0) {
+#pragma unroll
+          for (int i = 0; i < 2 * NSMAX * RT; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < DTMAX; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+          }
+        }
+      }
       if (__any(alpha != 1.f)) {                               // rescale the running output only if a row's maximum moved
+        // The output lives in accumulation registers, which only MFMAs and moves can name. Written as
+        // plain multiplications, the compiler moves all of it into vector registers at the top of EVERY
+        // iteration, for the sake of this branch that is hardly ever taken (80 moves a block, a quarter
+        // of the loop's vector instructions). As opaque code the moves stay in here.
 #pragma unroll
         for (int dt = 0; dt < DTMAX; ++dt)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) acc[rt][dt][j] *= alpha;
+          for (int j = 0; j < 4; ++j) {
+            float o = acc[rt][dt][j], t;
+            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
+                         : "+a"(o), "=&v"(t)
+                         : "v"(alpha));
+            acc[rt][dt][j] = o;
+          }
       }
 #pragma unroll
       for (int dt = 0; dt < DTMAX; ++dt)
         if (EXACT || dt < dts) tw_mma16(acc[rt][dt], vf[dt], pb);
     }
   };
-  auto compute_if_seen = [&](int blk, int buf) {
+  auto seen = [&](int blk) { return wave_live && blk < blk_end && blk * 32 <= wave_t_max; };
+  auto edge_of = [&](int blk) {
     const int p0 = blk * 32;
-    if (wave_live && p0 <= wave_t_max)
-      compute(blk, buf, !(wave_full && p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len));
+    return !(wave_full && p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len);
   };
+  // One iteration: block blk lies in stage buf and its scores in s_now; block blk + 1 lies in the next
+  // stage, its scores go to s_then; block blk + 2, in registers since the iteration before, is written to
+  // the stage after that (which held block blk - 1: every wave has left the iteration that read it), and
+  // block blk + 3 is fetched. Fetches are unconditional (no register copies): past the end the last block
+  // is fetched again.
+  // The iterations in which the wave needs both steps and no masking (nearly all of them) run in a loop
+  // of their own, whose body is one stretch of code without a branch between the two steps; what comes
+  // before and after runs in loops whose body decides step by step. (One loop with both bodies behind a
+  // branch made the compiler copy all 64 accumulators where the branches met.)
+  f32x4 s_now[RT][2], s_then[RT][2];
+  int blk = blk_begin, buf = 0;
+  auto run_to = [&](int end, auto body) {
+    for (; blk < end; ++blk) {
+      const int buf1 = buf == TW_PF_STAGES - 1 ? 0 : buf + 1, buf2 = buf1 == TW_PF_STAGES - 1 ? 0 : buf1 + 1;
+      body(blk, buf, buf1);
+      // block blk + 2, fetched an iteration ago, goes to LDS; the registers it leaves take block blk + 3.
+      // All of this stands behind the last MFMAs of the body, whose time it shares.
+      stash(buf2);
+      fetch(min(blk + 3, blk_end - 1));
+      lookup(blk + 4);                                       // (its page numbers replace those just used)
+      __syncthreads();
+      buf = buf1;
+      if constexpr (PIPELINED) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int tile = 0; tile < 2; ++tile) s_now[rt][tile] = s_then[rt][tile];
+      }
+    }
+  };
+  auto step_by_step = [&](int blk, int buf, int buf1) {
+    if constexpr (PIPELINED) {
+      if (seen(blk + 1)) scores(blk + 1, buf1, edge_of(blk + 1), s_then);
+      if (seen(blk)) finish(buf, s_now, std::false_type{});
+    } else if (seen(blk)) {
+      scores(blk, buf, edge_of(blk), s_now);
+      finish(buf, s_now, std::false_type{});
+    }
+  };
+  auto both_steps = [&](int blk, int buf, int buf1) {
+    scores(blk + 1, buf1, false, s_then);
+    finish(buf, s_now, std::true_type{});
+  };
+  // both_steps for the blocks b of [both_begin, both_end): b + 1 is a block of this workgroup every key
+  // of which every row of the wave sees (then so is b seen)
+  int both_begin = blk_begin, both_end = blk_begin;
+  if (PIPELINED && wave_live && wave_full) {
+    const int last_next = min(min(blk_end - 1, (wave_t_min + 1) / 32 - 1), kv_len / 32 - 1);   // the largest b + 1
+    both_begin = max(blk_begin, (wave_lo_max + 31) / 32 - 1);
+    both_end = max(both_begin, last_next);
+  }
 
   lookup(blk_begin);
   fetch(blk_begin);
   lookup(blk_begin + 1);
   stash(0);
+  fetch(min(blk_begin + 1, blk_end - 1));
+  lookup(blk_begin + 2);
+  stash(1);
+  fetch(min(blk_begin + 2, blk_end - 1));
+  lookup(blk_begin + 3);
   __syncthreads();
-  int blk = blk_begin;
-  for (; blk + 1 < blk_end; ++blk) {                        // every fetch unconditional: no register copies
-    const int buf = (blk - blk_begin) & 1;
-    fetch(blk + 1);
-    lookup(blk + 2);                                         // (its page numbers replace those just used)
-    compute_if_seen(blk, buf);
-    stash(buf ^ 1);
-    __syncthreads();
-  }
-  compute_if_seen(blk, (blk - blk_begin) & 1);                // the last block (blk_end > blk_begin always)
+  if (PIPELINED && seen(blk_begin)) scores(blk_begin, 0, edge_of(blk_begin), s_now);
+  run_to(both_begin, step_by_step);
+  run_to(both_end, both_steps);
+  run_to(blk_end, step_by_step);                             // (blk_end > blk_begin always)
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) l[rt] = tw_rows_sum(l[rt]);   // (the running maximum, and so every rescaling, was the row's: the same for the four)
 
@@ -1081,7 +1182,7 @@ static int prefill_bf16_launch(AttnArgs a, int n_seqs, int max_q_len, hipStream_
   TW_REQUIRE(total < (1L << 30));
   TW_REQUIRE((long)a.kv_heads * a.page_size * a.head_dim * 2 < (1L << 31));      // a page's bytes: 32-bit in the kernel
   dim3 grid((unsigned)total);
-  const size_t lds_bytes = 2 * 32 * (DTMAX * 32 + 16) + 2 * DTMAX * 16 * TW_PF_VROW;
+  const size_t lds_bytes = TW_PF_STAGES * (32 * (DTMAX * 32 + 16) + DTMAX * 16 * TW_PF_VROW);
   static bool attribute_set = false;
   if (!attribute_set) {
     hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_bf16_kernel<DTMAX, EXACT, 1>,
