@@ -652,6 +652,38 @@ def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
         torch.testing.assert_close(out.float().cpu().reshape(q_len, heads, d), want, **ATTN_TOL[dtype])
 
 
+@pytest.mark.parametrize("head_dim", [128, 64])
+def test_attn_prefill_scores_that_keep_rising(ops, device, head_dim):
+    """Scores grow from one 32-key block to the next, by a different amount per head: little (the softmax
+    reference of the fast kernel stays where the first block put it and probabilities exceed 1), about as
+    much as the kernel lets a score exceed its reference, and more (the reference moves and sum and output
+    are rescaled, block after block). A wrong rescaling, or a reference that is moved for one of sum and
+    output only, is wrong by O(1)."""
+    dtype, n, q_len, page = torch.bfloat16, 448, 96, 16
+    steps = [0.4, 2.0, 5.0, 5.6, 9.0, 0.0]                               # score gained per block, natural units
+    heads = len(steps)
+    gen = torch.Generator().manual_seed(5)
+    unit = torch.nn.functional.normalize(torch.randn(head_dim, generator=gen), dim=0)
+    block = (torch.arange(n) // 32).float()
+    k = (unit[None] * block[:, None] + 0.02 * torch.randn(n, head_dim, generator=gen))[:, None, :]
+    v = torch.randn(n, 1, head_dim, generator=gen)
+    k, v = k.to(dtype).float(), v.to(dtype).float()
+    q_one = torch.stack([unit * (s * head_dim ** 0.5) for s in steps]).to(dtype)       # q.k / sqrt(d) = s * block
+    q = q_one[None].expand(q_len, heads, head_dim).contiguous()
+    want = plain.attention(q.float(), k, v, torch.arange(n - q_len, n))
+    keys, values, table = build_paged([k], [v], [n], page, n // page + 4, device, dtype, seed=4)
+    kv_len = torch.tensor([n], dtype=torch.int32, device=device)
+    q_start = torch.tensor([0, q_len], dtype=torch.int32, device=device)
+    for generic, chunk, tile_rows in ((False, 0, 64), (False, 0, 128), (True, 0, 0), (False, 64, 128), (False, 160, 64)):
+        out = torch.full((q_len, heads * head_dim), float("nan"), dtype=dtype, device=device)
+        split = (math.ceil((n + 31) / chunk) + 1 if chunk else 1, chunk, tile_rows)
+        ws = torch.full((ops.attn_prefill_workspace_floats(q_len, heads, head_dim, split[0]),), float("nan"),
+                        device=device) if chunk else None
+        ops.attn_prefill(q.reshape(q_len, -1).to(device), keys, values, table, q_start, kv_len, 0, 1, q_len, out, heads, 1,
+                         head_dim, head_dim ** -0.5, generic=generic, split=split, workspace=ws)
+        torch.testing.assert_close(out.float().cpu().reshape(q_len, heads, head_dim), want, **ATTN_TOL[dtype])
+
+
 # ---------------------------------------------------------------------------------------
 def test_sampling_greedy_ties_and_distribution(ops, device):
     vocab = 389
