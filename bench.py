@@ -68,6 +68,8 @@ def parse():
     p.add_argument("--no-graphs", action="store_true")
     p.add_argument("--prefill-only", action="store_true", help="measure only the prefill (profiling runs)")
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--yardstick", default="", help="rows, comma separated: time the four projections of a layer at these row "
+                   "counts with this engine's kernels and with the library's (a table, no model is built)")
     p.add_argument("--serve", action="store_true",
                    help="instead: continuous batching of --requests requests (prompts of 128..4096 tokens, 256 "
                         "generated each, Poisson arrivals at --rate a second, prompt portions of 512)")
@@ -225,6 +227,49 @@ def library_matrix_rate(torch, c, rows, layers, device, repeats=5):
     return flops / (best / 1000) / 1e12
 
 
+def yardstick_table(torch, c, rows_list, device, copies=4, repeats=5):
+    """Microseconds and TFLOP/s of the four projections of a layer at each row count: this engine's kernels (shuffled
+    weights, the choice `ops.linear` makes itself; gate_up with its SiLU-multiply epilogue) beside the library's
+    bfloat16 product (hipBLASLt through torch.matmul; not on the product path). COPIES weight sets in turn, so that
+    weights come from HBM as in the model."""
+    from tessweave_engine_amd.kernels import ops
+    qkv = (c.num_attention_heads + 2 * c.num_key_value_heads) * c.head_dim
+    shapes = [("qkv", qkv, c.hidden_size, False), ("o", c.hidden_size, c.num_attention_heads * c.head_dim, False),
+              ("gate_up", 2 * c.intermediate_size, c.hidden_size, True), ("down", c.hidden_size, c.intermediate_size, False)]
+    lines = []
+    for name, n, k, glu in shapes:
+        plain = [torch.randn(n, k, device=device, dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
+        shuffled = [ops.shuffle_weight(w) for w in plain]
+        for rows in rows_list:
+            x = torch.randn(rows, k, device=device, dtype=torch.bfloat16) * 0.1
+            out = torch.empty(rows, n // 2 if glu else n, device=device, dtype=torch.bfloat16)
+            work = torch.empty(max(ops.linear_workspace_bytes(torch.bfloat16, rows, n, k) // 4, 16), device=device)
+            timed = {}
+            engine = (lambda i: ops.linear_glu(x, shuffled[i], out)) if glu else \
+                (lambda i: ops.linear(x, shuffled[i], out, workspace=work))
+            for who, call in (("engine", engine),
+                              ("library", lambda i: torch.matmul(x, plain[i].t()))):
+                best = None
+                for r in range(repeats + 1):
+                    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    start.record()
+                    for i in range(2 * copies):
+                        call(i % copies)
+                    end.record()
+                    torch.cuda.synchronize()
+                    if r:
+                        us = start.elapsed_time(end) * 1000 / (2 * copies)
+                        best = us if best is None else min(best, us)
+                timed[who] = best
+            flops = 2.0 * rows * n * k
+            lines.append({"projection": name, "rows": rows, "n": n, "k": k,
+                          "engine_us": round(timed["engine"], 1), "engine_tflops": round(flops / timed["engine"] / 1e6, 1),
+                          "library_us": round(timed["library"], 1), "library_tflops": round(flops / timed["library"] / 1e6, 1)})
+        del plain, shuffled
+        torch.cuda.empty_cache()
+    return lines
+
+
 def prefill_run(model, torch, tokens, dtype, seed, repeats=3):
     from tessweave_engine_amd.cache import CacheManager
     from tessweave_engine_amd.engine import StepEntry, Stepper
@@ -266,6 +311,10 @@ def main():
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     config = config_from_dict(cfg)
+    if args.yardstick:
+        for line in yardstick_table(torch, config, [int(v) for v in args.yardstick.split(",")], "cuda:0"):
+            print(json.dumps(line))
+        return 0
     model = random_model(config, args.seed, dtype=args.dtype, device="cuda:0")
     c = config
     use_graphs = not args.no_graphs
