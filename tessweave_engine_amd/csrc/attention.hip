@@ -706,7 +706,9 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     row_ok[rt] = row < rows;
     tok[rt] = row / G;
     head[rt] = kvh * G + row % G;
-    t_row[rt] = row_ok[rt] ? first_pos + tok[rt] : -1;
+    // (a row past the end stands in for the last token with a query of zeros: it sees what the wave's
+    // other rows see, needs no mask of its own, and is never stored)
+    t_row[rt] = first_pos + (row_ok[rt] ? tok[rt] : (rows - 1) / G);
     const bf16_t* q_row = (const bf16_t*)a.q + (size_t)(token0 + tok[rt]) * a.ldq + (size_t)head[rt] * D;
 #pragma unroll
     for (int st = 0; st < NSMAX; ++st) {
@@ -738,7 +740,6 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   const int wave_t_max = first_pos + min(rows - 1, wg_row0 + wave * 16 * RT + 16 * RT - 1) / G;
   const int wave_t_min = first_pos + min(rows - 1, wg_row0 + wave * 16 * RT) / G;
   const bool wave_live = wg_row0 + wave * 16 * RT < rows;
-  const bool wave_full = wg_row0 + wave * 16 * RT + 16 * RT <= rows;
   const int wave_lo_max = a.window > 0 ? wave_t_max - a.window + 1 : 0;  // largest lower bound among the wave's rows
 
   // This thread's share of a block, fixed for the whole loop: K piece i is 16 bytes
@@ -976,7 +977,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   auto seen = [&](int blk) { return wave_live && blk < blk_end && blk * 32 <= wave_t_max; };
   auto edge_of = [&](int blk) {
     const int p0 = blk * 32;
-    return !(wave_full && p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len);
+    return !(p0 + 31 <= wave_t_min && p0 >= wave_lo_max && p0 + 32 <= kv_len);
   };
   // One iteration: block blk lies in stage buf and its scores in s_now; block blk + 1 lies in the next
   // stage, its scores go to s_then; block blk + 2, in registers since the iteration before, is written to
@@ -1024,7 +1025,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   // both_steps for the blocks b of [both_begin, both_end): b + 1 is a block of this workgroup every key
   // of which every row of the wave sees (then so is b seen)
   int both_begin = blk_begin, both_end = blk_begin;
-  if (PIPELINED && wave_live && wave_full) {
+  if (PIPELINED && wave_live) {
     const int last_next = min(min(blk_end - 1, (wave_t_min + 1) / 32 - 1), kv_len / 32 - 1);   // the largest b + 1
     both_begin = max(blk_begin, (wave_lo_max + 31) / 32 - 1);
     both_end = max(both_begin, last_next);
