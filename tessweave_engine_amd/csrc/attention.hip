@@ -56,6 +56,8 @@ struct AttnArgs {
   float* part_ml;         // [seq - seq0][q_heads][splits][2]  (max, sum)
   int q_heads, kv_heads, head_dim, page_size, window;
   float scale;
+  float softcap;          // > 0: scores (after the scale) pass through softcap * tanh(score / softcap); the kernels
+                          // that take every type and page size only
   int splits;
   int page_shift;         // log2(page_size) if it is a power of two, else -1
   int n_seqs, max_tiles;  // prefill (bfloat16 kernel): sequences of the launch, row tiles of the longest
@@ -120,7 +122,9 @@ struct RowTile {
     for (int j = 0; j < 4; ++j) {
       const int p = p0 + 4 * g + j;
       const bool ok = p < kv_len && p <= t_row && p >= lo_row;
-      s[j] = ok ? s[j] * a.scale : -INFINITY;
+      float sc = s[j] * a.scale;
+      if (a.softcap > 0.f) sc = a.softcap * tanhf(sc / a.softcap);
+      s[j] = ok ? sc : -INFINITY;
       mx = fmaxf(mx, s[j]);
     }
     mx = tw_rows_max(mx);
@@ -1281,13 +1285,16 @@ extern "C" int tw_attn_decode(int dtype, const void* q, long ldq, const void* ke
                               const int* block_table, int table_stride, const int* q_start,
                               const int* kv_len, int seq0, int n_seqs, void* out, long ldo,
                               float* workspace, long workspace_floats, int q_heads, int kv_heads,
-                              int head_dim, int page_size, int window, float scale, int splits,
+                              int head_dim, int page_size, int window, float scale, float softcap, int splits,
                               int generic, hipStream_t stream) {
   AttnArgs a;
   a.q = q; a.ldq = ldq; a.keys = keys; a.values = values; a.block_table = block_table;
   a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = splits;
+  TW_REQUIRE(softcap >= 0.f);
+  a.softcap = softcap;
+  if (softcap > 0.f) generic = 1;
   a.part_o = nullptr; a.part_ml = nullptr;
   a.page_shift = -1;
   for (int sh = 0; sh < 20; ++sh)
@@ -1334,7 +1341,7 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
                                const int* kv_len, int seq0, int n_seqs, int max_q_len, void* out,
                                long ldo, float* workspace, long workspace_floats, int n_tokens, int max_chunks,
                                int kv_chunk, int tile_rows, int q_heads, int kv_heads, int head_dim, int page_size,
-                               int window, float scale, int generic, hipStream_t stream) {
+                               int window, float scale, float softcap, int generic, hipStream_t stream) {
   AttnArgs a;
   TW_REQUIRE(tile_rows == 0 || tile_rows == 64 || tile_rows == 128);
   a.tile_rows = tile_rows;
@@ -1342,6 +1349,9 @@ extern "C" int tw_attn_prefill(int dtype, const void* q, long ldq, const void* k
   a.table_stride = table_stride; a.q_start = q_start; a.kv_len = kv_len; a.seq0 = seq0;
   a.out = out; a.ldo = ldo; a.q_heads = q_heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
   a.page_size = page_size; a.window = window; a.scale = scale; a.splits = 1;
+  TW_REQUIRE(softcap >= 0.f);
+  a.softcap = softcap;
+  if (softcap > 0.f) generic = 1;
   a.part_o = nullptr; a.part_ml = nullptr;
   a.max_chunks = 1; a.kv_chunk = 0;
   a.page_shift = -1;

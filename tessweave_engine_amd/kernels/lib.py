@@ -32,10 +32,10 @@ _SIGNATURES = {
     "tw_linear": (I, [I, I, P, L, P, L, I, P, P, L, P, L, P, L, I, I, I, I, P]),
     "tw_attn_decode_splits": (I, [I, I, I, I]),
     "tw_attn_decode_workspace_floats": (L, [I, I, I, I]),
-    "tw_attn_decode": (I, [I, P, L, P, P, P, I, P, P, I, I, P, L, P, L, I, I, I, I, I, F, I, I, P]),
+    "tw_attn_decode": (I, [I, P, L, P, P, P, I, P, P, I, I, P, L, P, L, I, I, I, I, I, F, F, I, I, P]),
     "tw_attn_prefill_split": (I, [I, I, I, I, I, I, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "tw_attn_prefill_workspace_floats": (L, [I, I, I, I]),
-    "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, I, P]),
+    "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),
     "tw_sample_rows": (I, [P, L, I, I, P, P, P, P, P, L, P]),

@@ -358,11 +358,12 @@ def _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads
 
 
 def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out, q_heads, kv_heads,
-                head_dim, scale, window=0, splits=1, workspace=None, generic=False):
+                head_dim, scale, window=0, splits=1, workspace=None, generic=False, softcap=0.0):
     """Attention of sequences seq0..seq0+n_seqs-1, each with ONE query token, over their pages.
 
     generic=True forces the kernel that takes every type and page size (bfloat16 with
-    pages of a multiple of 8 keys otherwise runs a faster kernel of its own).
+    pages of a multiple of 8 keys otherwise runs a faster kernel of its own). softcap > 0 passes the scaled
+    scores through softcap * tanh(score / softcap) (that kernel only).
     """
     ldq, ldo = _check_attention(q, keys, values, block_table, q_start, kv_len, out, q_heads, kv_heads, head_dim)
     _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0], "sequence range exceeds the metadata")
@@ -374,8 +375,8 @@ def attn_decode(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, out
                                    _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
                                    _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
                                    seq0, n_seqs, _dev(out), ldo, ws_ptr, ws_floats, q_heads, kv_heads, head_dim,
-                                   keys.shape[2], int(window or 0), float(scale), int(splits), 1 if generic else 0,
-                                   _stream()),
+                                   keys.shape[2], int(window or 0), float(scale), float(softcap or 0.0), int(splits),
+                                   1 if generic else 0, _stream()),
           "attn_decode")
     return out
 
@@ -396,7 +397,7 @@ def attn_prefill_workspace_floats(n_tokens, q_heads, head_dim, max_chunks):
 
 
 def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_q_len, out, q_heads,
-                 kv_heads, head_dim, scale, window=0, generic=False, split=None, workspace=None):
+                 kv_heads, head_dim, scale, window=0, generic=False, split=None, workspace=None, softcap=0.0):
     """Attention of sequences seq0..seq0+n_seqs-1 with up to max_q_len query tokens each.
 
     split = (max_chunks, kv_chunk[, tile_rows]) from attn_prefill_split with a float32 workspace of
@@ -416,8 +417,8 @@ def attn_prefill(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, ma
                                     _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
                                     seq0, n_seqs, int(max_q_len), _dev(out), ldo, ws_ptr, ws_floats, q.shape[0],
                                     max_chunks, kv_chunk, tile_rows, q_heads, kv_heads, head_dim,
-                                    keys.shape[2], int(window or 0), float(scale), 1 if generic else 0,
-                                    _stream()), "attn_prefill")
+                                    keys.shape[2], int(window or 0), float(scale), float(softcap or 0.0),
+                                    1 if generic else 0, _stream()), "attn_prefill")
     return out
 
 

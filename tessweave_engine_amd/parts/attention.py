@@ -19,8 +19,10 @@ import torch
 
 class GroupedQueryAttention(Mixer):
     def __init__(self, prefix, hidden, q_heads, kv_heads, head_dim, position, qkv_bias=True,
-                 o_bias=False, window=None, scale=None, packed=True, head_hook=None):
-        """head_hook: an optional `HeadHook` that changes the projected q, k, v (bias added) in place before q
+                 o_bias=False, window=None, scale=None, packed=True, head_hook=None, softcap=None):
+        """softcap: scaled scores pass through softcap * tanh(score / softcap) before the softmax (the attention
+        kernels that take every type and page size then run; the fast bfloat16 ones have no such step).
+        head_hook: an optional `HeadHook` that changes the projected q, k, v (bias added) in place before q
         and k are rotated: a per-head norm, a scaling. With a hook the projection is finished by its own
         kernel first (without one, few-row steps leave its split-K sums to the kernel that adds the bias,
         rotates and writes the cache)."""
@@ -41,6 +43,7 @@ class GroupedQueryAttention(Mixer):
         self.position = position
         self.window = window
         self.scale = float(scale) if scale is not None else self.checkpoint_head_dim ** -0.5
+        self.softcap = float(softcap) if softcap else 0.0
         self.qkv = Linear([prefix + "q_proj", prefix + "k_proj", prefix + "v_proj"], hidden,
                           [q_heads * head_dim, kv_heads * head_dim, kv_heads * head_dim], bias=qkv_bias, packed=packed,
                           pad_out=pad)
@@ -103,7 +106,7 @@ class GroupedQueryAttention(Mixer):
                 ws = ctx.workspace.get("attn.split", (floats,), torch.float32)
             ops.attn_decode(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode, out,
                             self.q_heads, self.kv_heads, self.head_dim, self.scale, window=window,
-                            splits=splits, workspace=ws)
+                            splits=splits, workspace=ws, softcap=self.softcap)
         if ctx.n_seqs > ctx.n_decode:
             # long key ranges are cut into chunks for separate workgroups when there are few tiles of rows
             longest = min(ctx.max_kv_len, window + ctx.max_q_len) if window else ctx.max_kv_len
@@ -114,7 +117,8 @@ class GroupedQueryAttention(Mixer):
                     n, self.q_heads, self.head_dim, split[0]),), torch.float32)
             ops.attn_prefill(qkv, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode,
                              ctx.n_seqs - ctx.n_decode, ctx.max_q_len, out, self.q_heads, self.kv_heads,
-                             self.head_dim, self.scale, window=window, split=split, workspace=ws)
+                             self.head_dim, self.scale, window=window, split=split, workspace=ws,
+                             softcap=self.softcap)
         if ctx.defer_sums and not self.o.biases and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # the next norm adds them into x
         self.o.forward(ctx, out, x, residual=x)

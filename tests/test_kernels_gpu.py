@@ -652,6 +652,43 @@ def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
         torch.testing.assert_close(out.float().cpu().reshape(q_len, heads, d), want, **ATTN_TOL[dtype])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_soft_capped_scores(ops, device, dtype):
+    """softcap * tanh(score / softcap) before the softmax, decode and prompt portions, against the formula in
+    torch. Queries are long enough that uncapped scores reach several times the cap: without the cap, or with
+    the cap before the scale, the result is wrong by O(1)."""
+    heads, kv_heads, d, page, n, q_len, cap = 4, 2, 32, 8, 75, 9, 5.0
+    gen = torch.Generator().manual_seed(8)
+    k = torch.randn(n, kv_heads, d, generator=gen).to(dtype).float()
+    v = torch.randn(n, kv_heads, d, generator=gen).to(dtype).float()
+    q = (torch.randn(q_len, heads, d, generator=gen) * 6.0).to(dtype)
+    pos = torch.arange(n - q_len, n)
+    kk = k.repeat_interleave(heads // kv_heads, 1)
+    vv = v.repeat_interleave(heads // kv_heads, 1)
+    scores = torch.einsum("qhd,khd->hqk", q.float(), kk) * d ** -0.5
+    assert scores.abs().max() > 3 * cap
+    capped = cap * torch.tanh(scores / cap)
+    capped = capped.masked_fill(torch.arange(n)[None, None, :] > pos[None, :, None], float("-inf"))
+    want = torch.einsum("hqk,khd->qhd", torch.softmax(capped, -1), vv)
+    uncapped = torch.einsum("hqk,khd->qhd", torch.softmax(scores.masked_fill(
+        torch.arange(n)[None, None, :] > pos[None, :, None], float("-inf")), -1), vv)
+    assert (want - uncapped).abs().max() > 0.1                             # the cap matters here
+    keys, values, table = build_paged([k], [v], [n], page, n // page + 3, device, dtype, seed=2)
+    kv_len = torch.tensor([n], dtype=torch.int32, device=device)
+    out = torch.full((q_len, heads * d), float("nan"), dtype=dtype, device=device)
+    ops.attn_prefill(q.reshape(q_len, -1).to(device), keys, values, table,
+                     torch.tensor([0, q_len], dtype=torch.int32, device=device), kv_len, 0, 1, q_len, out, heads,
+                     kv_heads, d, d ** -0.5, softcap=cap)
+    torch.testing.assert_close(out.float().cpu().reshape(q_len, heads, d), want, **ATTN_TOL[dtype])
+    for splits in (1, 3):
+        out1 = torch.full((1, heads * d), float("nan"), dtype=dtype, device=device)
+        ws = torch.empty(max(1, ops.attn_decode_workspace_floats(1, heads, d, splits)), device=device)
+        ops.attn_decode(q[-1:].reshape(1, -1).to(device), keys, values, table,
+                        torch.tensor([0, 1], dtype=torch.int32, device=device), kv_len, 0, 1, out1, heads, kv_heads, d,
+                        d ** -0.5, splits=splits, workspace=ws, softcap=cap)
+        torch.testing.assert_close(out1.float().cpu().reshape(heads, d), want[-1], **ATTN_TOL[dtype])
+
+
 @pytest.mark.parametrize("head_dim", [128, 64])
 def test_attn_prefill_scores_that_keep_rising(ops, device, head_dim):
     """Scores grow from one 32-key block to the next, by a different amount per head: little (the softmax

@@ -143,7 +143,19 @@ def test_whole_model_structure():
 def test_greedy_and_temperature_helpers():
     cfg, w = tiny(tied=True)
     out = plain.greedy(cfg, w, [1, 2, 3], 4)
-    assert len(out) == 4 and all(0 <= t < 50 for t in out)
+    # each token is the arg max of the last position's logits over everything before it; the logits of the
+    # whole sequence, computed once, hold those of every prefix (causality), so a helper that forgets to
+    # append, appends twice or reads another position fails
+    whole = plain.forward(cfg, w, [1, 2, 3] + out)
+    assert out == [int(whole[2 + i].argmax()) for i in range(4)]
+    # the margin of each choice is far above float32 noise, so the comparison above is not a coin toss
+    top2 = torch.topk(whole[2:6], 2, dim=-1).values
+    assert float((top2[:, 0] - top2[:, 1]).min()) > 1e-4
+    # a token changed in the prompt changes what follows (the helper reads its prompt)
+    assert plain.greedy(cfg, w, [1, 2, 4], 4) != out or plain.greedy(cfg, w, [7, 2, 3], 4) != out
     logits = torch.tensor([1.0, 2.0, 3.0])
     p = plain.softmax_temperature(logits, 0.5)
     torch.testing.assert_close(p, torch.softmax(logits / 0.5, -1))
+    # temperature sharpens: T -> 0 puts everything on the largest logit, T large flattens
+    assert plain.softmax_temperature(logits, 0.01)[2] > 0.999
+    torch.testing.assert_close(plain.softmax_temperature(logits, 1e6), torch.full((3,), 1 / 3), atol=1e-5, rtol=0)
