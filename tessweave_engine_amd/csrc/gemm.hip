@@ -275,15 +275,11 @@ __global__ __launch_bounds__(TW_CU_WAVES * 64) void gemm_stream_cu_kernel(
   const int r = lane & 15, g = lane >> 4;
 
 #define TW_CU_WAIT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
-#ifdef TW_CU_NOBARRIER
-#define TW_CU_BARRIER() asm volatile("" ::: "memory")
-#else
 #define TW_CU_BARRIER()                   \
   do {                                    \
     __builtin_amdgcn_s_barrier();         \
     asm volatile("" ::: "memory");        \
   } while (0)
-#endif
   // Wait until at most `n` of this wave's loads and copies are in flight (they finish in the order they
   // were issued). The count is an immediate of the instruction, hence the cases.
   auto wait_for = [&](auto n) {
@@ -370,7 +366,6 @@ __global__ __launch_bounds__(TW_CU_WAVES * 64) void gemm_stream_cu_kernel(
         wf[buf][u] = tw_load_frag_stream(w_row + (size_t)min(stage * U + u, last_step) * (64 * EPF));
     };
     auto multiply = [&](const int buf) {
-#ifndef TW_CU_NOMMA
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         Frag xf[MT];
@@ -383,10 +378,6 @@ __global__ __launch_bounds__(TW_CU_WAVES * 64) void gemm_stream_cu_kernel(
         // that reading a whole stage ahead would take are what the weights in flight need
         if (MT > 1) __builtin_amdgcn_sched_barrier(0);
       }
-#else
-#pragma unroll
-      for (int u = 0; u < U; ++u) acc[0] = acc[0] + __builtin_bit_cast(f32x4, wf[buf][u]);
-#endif
     };
     // Stage i: wait for this wave's copies of stage i, meet the others (stage i's activations are in LDS,
     // stage i - 1's are read), ask for the weights and copies of stage i + NBUF - 1, multiply. In the main
@@ -630,11 +621,7 @@ static int launch_skinny_lds(const T* A, long lda, const T* W, long ldw, const f
   // waves where twice as many of them lie more evenly on the CUs (N = 37,888: 592 workgroups are 2.3 a CU,
   // three on some; 1,184 are 4.6, five on some). With more rows every workgroup stages its own copy of
   // the activations, so the larger workgroups stay.
-#ifdef TW_W2_ALL
-  if constexpr (!PARTIAL) {
-#else
   if constexpr (MT == 1 && !PARTIAL) {
-#endif
     if (splits == 1 && cu_imbalance(tw_div_up(N, 32)) < cu_imbalance(tw_div_up(N, 64)) - 0.03) {
       const int groups = tw_div_up(N, 32);
       gemm_skinny_lds_kernel<T, OutT, MT, U, 2, PARTIAL, SHUF, GLU><<<groups, 128, 0, stream>>>(
