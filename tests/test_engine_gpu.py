@@ -874,6 +874,111 @@ def test_a_norm_that_folds_nothing_and_a_rotation_of_adjacent_pairs(tmp_path, de
         unregister_architecture("ToyCenteredForCausalLM")
 
 
+def test_toy_attention_with_soft_capped_scores(tmp_path, device):
+    """A toy model, built outside the package, whose attention passes its scaled scores through
+    cap * tanh(score / cap): one of two layers, with scores several times the cap. Both precisions
+    (bfloat16 takes the attention kernels for every type and page size, since the fast ones have no such step),
+    a prompt in portions, decoded tokens, two requests in one batch; against the formula written out here."""
+    from dataclasses import dataclass
+    from safetensors.torch import save_file
+    from tessweave_engine_amd.cache import CacheManager
+    from tessweave_engine_amd.config import register_architecture, unregister_architecture
+    from tessweave_engine_amd.engine import StepEntry, Stepper
+    from tessweave_engine_amd.parts import (DecoderModel, GroupedQueryAttention, OutputHead, PreNormBlock, RMSNorm,
+                                            RotaryEmbedding, SwiGLU, TokenEmbedding)
+    from tessweave_engine_amd.weights import load_model, random_tensors
+
+    H, HEADS, KV, D, THETA, INTER, VOCAB, CAP = 32, 4, 2, 16, 100.0, 48, 43, 2.0
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        architecture: str = "ToyCappedForCausalLM"
+        vocab_size: int = VOCAB
+        max_position_embeddings: int = 128
+        eos_token_ids: tuple = ()
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls()
+
+        def to_dict(self):
+            return dict(architectures=[self.architecture], model_type="toy_capped", vocab_size=self.vocab_size)
+
+    def build_toy(c):
+        emb = TokenEmbedding("emb", c.vocab_size, H)
+        rotary = RotaryEmbedding(D, THETA)
+        blocks = [PreNormBlock(RMSNorm(f"l{i}.n1", H, 1e-5),
+                               GroupedQueryAttention(f"l{i}.att.", H, HEADS, KV, D, rotary, qkv_bias=True,
+                                                     softcap=CAP if i == 0 else None),
+                               RMSNorm(f"l{i}.n2", H, 1e-5), SwiGLU(f"l{i}.ff.", H, INTER)) for i in range(2)]
+        return DecoderModel(c, emb, blocks, RMSNorm("final", H, 1e-5), OutputHead("head", c.vocab_size, H, tied_to=emb))
+
+    register_architecture("ToyCappedForCausalLM", "toy_capped", ToyConfig, build_toy)
+    try:
+        cfg = ToyConfig()
+        (tmp_path / "config.json").write_text(json.dumps(cfg.to_dict()))
+        tensors = random_tensors(build_toy(cfg).tensor_specs(), 12, std=0.3)
+        save_file(tensors, str(tmp_path / "model.safetensors"))
+        biggest = []
+
+        def plain_toy(tokens, w):
+            x = w["emb.weight"][torch.tensor(tokens)]
+            t, pos = len(tokens), torch.arange(len(tokens))
+            for i in range(2):
+                p = f"l{i}."
+                hn = plain.rms_norm(x, w[p + "n1.weight"], 1e-5)
+                q, k, v = (hn @ w[p + f"att.{n}_proj.weight"].T + w[p + f"att.{n}_proj.bias"] for n in "qkv")
+                q, k, v = plain.rope(q.reshape(t, HEADS, D), pos, THETA), plain.rope(k.reshape(t, KV, D), pos, THETA), v.reshape(t, KV, D)
+                if i == 0:
+                    kk, vv = k.repeat_interleave(HEADS // KV, 1), v.repeat_interleave(HEADS // KV, 1)
+                    scores = torch.einsum("qhd,khd->hqk", q, kk) * D ** -0.5
+                    biggest.append(float(scores.abs().max()))
+                    scores = CAP * torch.tanh(scores / CAP)
+                    scores = scores.masked_fill(pos[None, None, :] > pos[None, :, None], float("-inf"))
+                    att = torch.einsum("hqk,khd->qhd", torch.softmax(scores, -1), vv)
+                else:
+                    att = plain.attention(q, k, v, pos)
+                x = x + att.reshape(t, HEADS * D) @ w[p + "att.o_proj.weight"].T
+                hn = plain.rms_norm(x, w[p + "n2.weight"], 1e-5)
+                x = x + plain.swiglu(hn, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+            return plain.rms_norm(x, w["final.weight"], 1e-5) @ w["emb.weight"].T
+
+        g = torch.Generator().manual_seed(6)
+        seqs = {name: torch.randint(0, VOCAB, (n,), generator=g).tolist() for name, n in (("a", 37), ("b", 21))}
+        for dtype in ("float32", "bfloat16"):
+            w = {k: (v.to(torch.bfloat16).float() if dtype == "bfloat16" and v.dtype.is_floating_point else v.float())
+                 for k, v in tensors.items()}
+            wants = {name: plain_toy(toks, w) for name, toks in seqs.items()}
+            assert max(biggest) > 3 * CAP                                 # the cap matters
+            model = load_model(tmp_path, dtype=dtype, device="cuda:0")
+            cache = CacheManager(model.cache_layout(), 8, 12, 2, dtype=dtype, device=model.device, prefix_cache=False,
+                                 max_request_tokens=40)
+            stepper = Stepper(model, cache, max_step_tokens=32)
+            a, b = cache.open("a"), cache.open("b")
+            got = {"a": [], "b": []}
+
+            def run(*items):
+                entries = [StepEntry(seq, seqs[name][lo:hi], list(range(hi - lo))) for name, seq, lo, hi in items]
+                out, row = stepper.step(entries).float().cpu(), 0
+                for name, _, lo, hi in items:
+                    got[name].append(out[row:row + hi - lo].clone())
+                    row += hi - lo
+            run(("a", a, 0, 13))
+            run(("a", a, 13, 14), ("b", b, 0, 9))                         # a decodes beside b's prompt portion
+            run(("b", b, 9, 21), ("a", a, 14, 20))
+            for t in range(20, 37):
+                run(("a", a, t, t + 1))
+            for name in seqs:
+                # (bfloat16: the bar of the replay tests, 2 % of the largest logit, absolute)
+                tol = dict(atol=3e-5, rtol=3e-5) if dtype == "float32" else dict(atol=0.02 * float(wants[name].abs().max()), rtol=0)
+                torch.testing.assert_close(torch.cat(got[name]), wants[name], **tol)
+            cache.close(a), cache.close(b)
+            cache.check()
+            stepper.close()
+    finally:
+        unregister_architecture("ToyCappedForCausalLM")
+
+
 def test_toy_position_ids_on_two_axes_a_hook_between_bias_and_rotation_and_the_weights_a_step_reads(tmp_path, device):
     """Three things another architecture may need, built outside the package: an encoding that reads TWO position
     ids per token (half of the rotary pairs turn with each; step entries bring the ids), a per-head RMS norm of q
