@@ -1083,14 +1083,18 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
   // The sums of the probabilities are formed by the matrix unit too, as one more product a row tile
   // (ones x P, of the probabilities as rounded for the products): the vector unit is what bounds this
   // loop, and eight additions a row tile cost it twice the time the MFMA costs the matrix unit.
-  auto ordered_iteration = [&](int blk, int buf, int buf1, int buf2, f32x4 (&s)[RT][2], f32x4 (&s_next)[RT][2]) {
+  constexpr int KF_AHEAD = 2 * NSMAX < 4 ? 2 * NSMAX : 4;
+  auto ordered_iteration = [&](int blk, int buf, int buf1, int buf2, f32x4 (&s)[RT][2], f32x4 (&s_next)[RT][2],
+                               bf16x8 (&ahead)[KF_AHEAD]) {
     constexpr int NQK = 2 * NSMAX * RT, NPV = DTMAX * RT, NSLOT = NQK + NPV + RT;
-    constexpr int NKF = 2 * NSMAX, KF_AHEAD = NKF < 4 ? NKF : 4, NP = KPIECES + VPIECES;
-    constexpr int NMEM = NKF - KF_AHEAD + DTMAX + 3 * NP, MPS = (NMEM + NSLOT - 1) / NSLOT;
+    constexpr int NKF = 2 * NSMAX, NP = KPIECES + VPIECES;
+    constexpr int NMEM = NKF + DTMAX + 3 * NP, MPS = (NMEM + NSLOT - 1) / NSLOT;
     constexpr int VF_FIRST = NKF - KF_AHEAD + 2 * NP;       // V fragment dt is memory operation VF_FIRST + dt
+    constexpr int BARRIER_SLOT = (VF_FIRST + DTMAX + NP - 1) / MPS;   // the slot of the last operation before the barrier
     constexpr int NPROB = 8 * RT, P_AHEAD = 2, P_SPAN = NQK - 1;
     constexpr int NMX = 4 * RT;
     static_assert(VF_FIRST / MPS + 2 <= NQK, "the first V fragment is read two slots before its product");
+    static_assert(BARRIER_SLOT < NSLOT - 1);
     static_assert(P_AHEAD < NPROB && P_SPAN >= 1);
     bf16x8 kf[NKF], vf[DTMAX], pb[RT], ones;
     float mx[RT];
@@ -1102,19 +1106,22 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     const unsigned k_in = in_page * (unsigned)D * 2u, v_in = in_page * 2u;
     const int* entry = table + ((lookup_blk * 32) >> pshift);
     const char* kbase = k_frag[0] + buf1 * KSTAGE;           // (tile 1's fragments lie 16 rows further)
+    const char* kbase_next = k_frag[0] + buf2 * KSTAGE;
     const char* vbase = v_frag + buf * VSTAGE;
-    auto k_fragment = [&](int k) {                            // k = 2 * step + tile
-      kf[k] = *reinterpret_cast<const bf16x8*>(kbase + (k & 1) * 16 * KROW + (k >> 1) * 64);
+    auto k_fragment = [&](auto& to, const char* base, int k) {   // k = 2 * step + tile
+      to[k] = *reinterpret_cast<const bf16x8*>(base + (k & 1) * 16 * KROW + (k >> 1) * 64);
     };
     auto memory_operation = [&](int q) {
-      if (q < NKF - KF_AHEAD) return k_fragment(q + KF_AHEAD);
+      if (q < NKF - KF_AHEAD) return k_fragment(kf, kbase, q + KF_AHEAD);
       q -= NKF - KF_AHEAD;
       if (q < NP) return stash_piece(q, buf2);
       q -= NP;
       if (q < NP) return fetch_piece(q, k_in, v_in);
       q -= NP;
       if (q < DTMAX) { vf[q] = *reinterpret_cast<const bf16x8*>(vbase + q * 16 * TW_PF_VROW); return; }
-      lookup_piece(q - DTMAX, entry);
+      q -= DTMAX;
+      if (q < NP) return lookup_piece(q, entry);
+      k_fragment(ahead, kbase_next, q - NP);                  // (behind the barrier: the block after the next)
     };
     // (the empty statements hold an exponential in its slot: its input is taken there and no earlier, its
     // rounded pair of results is there and no later; the compiler gathered them where they cost most)
@@ -1144,7 +1151,7 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
       else mx[rt] = max2(mx[rt], hi4[3]);
     };
 #pragma unroll
-    for (int k = 0; k < KF_AHEAD; ++k) k_fragment(k);
+    for (int k = 0; k < KF_AHEAD; ++k) kf[k] = ahead[k];     // (read behind the barrier of the iteration before)
 #pragma unroll
     for (int j = 0; j < P_AHEAD; ++j) exponential(j);
     __builtin_amdgcn_sched_barrier(0);
@@ -1162,8 +1169,14 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         tw_mma16(l_mma[rt], ones, pb[rt]);                   // every output row: the sum over the block's keys
       }
 #pragma unroll
-      for (int q = slot * MPS; q < (slot + 1) * MPS; ++q)
+      for (int q = slot * MPS; q < (slot + 1) * MPS; ++q) {
         if (q < NMEM) memory_operation(q);
+        // The iteration's barrier stands in the middle of it: before it this wave's writes of block
+        // blk + 2 and its last reads of block blk (whose stage the next iteration overwrites), behind it
+        // the first reads of block blk + 2, which are in registers when the next iteration begins. A
+        // wave in another kind of iteration has its barrier at the end, after the same writes and reads.
+        if (q == VF_FIRST + DTMAX + NP - 1) __syncthreads();
+      }
 #pragma unroll
       for (int j = P_AHEAD; j < NPROB; ++j)
         if ((j - P_AHEAD) * P_SPAN / (NPROB - P_AHEAD) == slot) exponential(j);
@@ -1255,10 +1268,16 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     // (blk_end - 1 is the only block of the workgroup that may cross the end of the sequence)
     const bool all_whole = blk_end * 32 <= kv_len;
     const int ordered_end = all_whole ? both_end : min(both_end, blk_end - 5);
+    bf16x8 ahead[KF_AHEAD];                                  // the first K fragments of the block after blk
+    if (blk < ordered_end) {
+      const int buf1 = buf == TW_PF_STAGES - 1 ? 0 : buf + 1;
+#pragma unroll
+      for (int k = 0; k < KF_AHEAD; ++k)
+        ahead[k] = *reinterpret_cast<const bf16x8*>(k_frag[0] + buf1 * KSTAGE + (k & 1) * 16 * KROW + (k >> 1) * 64);
+    }
     for (; blk < ordered_end; ++blk) {
       const int buf1 = buf == TW_PF_STAGES - 1 ? 0 : buf + 1, buf2 = buf1 == TW_PF_STAGES - 1 ? 0 : buf1 + 1;
-      ordered_iteration(blk, buf, buf1, buf2, s_now, s_then);
-      __syncthreads();
+      ordered_iteration(blk, buf, buf1, buf2, s_now, s_then, ahead);
       buf = buf1;
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
