@@ -606,12 +606,17 @@ def test_attn_far_key_among_hundreds(ops, device):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("page,window", [(16, 0), (8, 0), (64, 0), (16, 70), (4, 33), (12, 0), (24, 70), (48, 0), (20, 33)])
-def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
+@pytest.mark.parametrize("page,window,n,q_len", [(16, 0, 300, 48), (8, 0, 300, 48), (64, 0, 300, 48), (16, 70, 300, 48),
+                                                 (4, 33, 300, 48), (12, 0, 300, 48), (24, 70, 300, 48), (48, 0, 300, 48),
+                                                 (20, 33, 300, 48),
+                                                 # many blocks a tile, so that the fast kernel's main loop runs, with
+                                                 # and without a window that begins inside a block
+                                                 (16, 0, 1000, 130), (16, 403, 1000, 130), (64, 530, 1000, 70)])
+def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window, n, q_len):
     """Each head's query points at ONE key that sits on an edge (of a page, of a 32-key block, of a split,
     of the window, of the sequence): a kernel that drops, doubles or misplaces that key is wrong by O(1),
     also in bfloat16, where random keys would hide it in the tolerance."""
-    d, n, q_len = 64, 300, 48
+    d = 64
     targets = [0, 1, 7, 8, 15, 16, 17, 31, 32, 33, 63, 64, 127, 128, 159, 160, 255, 256, n - q_len - 1, n - q_len,
                n - 2, n - 1]
     if window:
@@ -625,7 +630,7 @@ def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window):
         k[p, 0] = unit[h] * 30.0
     k, v = k.to(dtype).float(), v.to(dtype).float()
     q_one = (unit * 8.0).to(dtype)                                     # score of the target: 30, of the rest: ~0
-    keys, values, table = build_paged([k], [v], [n], page, 320 // page + 8, device, dtype, seed=21)
+    keys, values, table = build_paged([k], [v], [n], page, max(320, n + 20) // page + 8, device, dtype, seed=21)
     kv_len = torch.tensor([n], dtype=torch.int32, device=device)
     # decode: the last position asks
     want = plain.attention(q_one[None].float(), k, v, torch.tensor([n - 1]), window=window or None)
