@@ -1370,26 +1370,32 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(AttnArgs a) {
   }
 }
 
-// How the keys of a prefill tile are split over workgroups: returns the most chunks a tile can
-// have (1: no splitting) and the keys per chunk. With fewer tiles than the chip has room for,
-// long tiles are cut so that there are about a thousand units of work of similar size.
-// Rows of a workgroup's tile in the bfloat16 prefill kernel: 128 (32 per wave), or 64 (16 per wave)
-// when 128 would leave the chip with few workgroups: the kernel's time is a chain of latencies
-// (fragment reads, MFMAs, the softmax's dependent steps), and more waves hide more of it.
+// Rows of a workgroup's tile in the bfloat16 prefill kernel: 128 (32 per wave: half the LDS reads and a
+// fifth fewer instructions a row), or 64 (16 per wave) where 128 would leave the chip with too few workgroups.
 static int prefill_tile_rows(int n_seqs, int q_heads, int kv_heads, int max_q_len, int max_kv_len, int asked) {
   if (asked == 64 || asked == 128) return asked;
   const int G = kv_heads > 0 ? q_heads / kv_heads : 1;
-  const long tiles = (long)tw_div_up((long)max_q_len * G, 128) * kv_heads * n_seqs;
-  // A portion late in a long prompt (most keys come from the cache): every tile then reads about
-  // max_kv_len keys, the ramp and the uneven lengths of causal tiles count for little, and what a row
-  // costs decides: 128-row tiles need about 20 % fewer instructions a row. Measured (28 query heads over
-  // 4, head size 128): 2,048 tokens after 2,048 / 6,144 / 30,000 cached ones 222 -> 168, 344 -> 258 and
-  // 1,980 -> 1,530 us; 512 tokens at 8,192 and 32,768 keys 155 -> 138 and 541 -> 441 us; with fewer
-  // tokens or fewer keys than below the 64-row tiles are as fast or faster.
-  if (max_kv_len >= 2L * max_q_len && (max_q_len >= 2048 || (max_q_len >= 256 && max_kv_len >= 8192))) return 128;
-  return tiles < 640 ? 64 : 128;                    // (2,048 tokens of 28 heads: 64 is 16 % faster; 4,096: 10 % slower)
+  const long tiles128 = (long)tw_div_up((long)max_q_len * G, 128) * kv_heads * n_seqs;
+  const long tiles64 = (long)tw_div_up((long)max_q_len * G, 64) * kv_heads * n_seqs;
+  // Measured (28 query heads over 4, head size 128; us with 64-row / 128-row tiles).
+  // A workgroup a CU or more without cutting tiles into chunks: 128. Whole prompts of 1,536 / 2,048 / 3,072 /
+  // 4,096 tokens 42 / 40, 56 / 54, 110 / 88, 170 / 140; four of 512 25 / 22; 2,048 behind 1,024 cached 105 / 72.
+  if (tiles128 >= 256) return 128;
+  // A portion late in a long prompt (most keys come from the cache): every tile reads about max_kv_len
+  // keys and what a row costs decides, also where the tiles are then cut into chunks: 256 / 512 / 1,024
+  // tokens behind 8,192 cached 73 / 55, 122 / 98, 206 / 188.
+  if (max_kv_len >= 2L * max_q_len && max_q_len >= 256 && max_kv_len >= 8192) return 128;
+  // 64-row tiles fill the chip and 128-row tiles would have to be cut: 1,024 tokens alone 26 / 45, behind
+  // 1,024 or 2,048 cached 42 / 66 and 66 / 85.
+  if (tiles64 >= 256) return 64;
+  // Both are cut into chunks: with few keys the shorter tiles (128 to 512 tokens alone: 19 / 21, 18 / 19,
+  // 19 / 20), with many the cheaper rows (256 behind 2,048: 41 / 36; 128 behind 8,192: 41 / 38).
+  return max_kv_len >= 2048 ? 128 : 64;
 }
 
+// How the keys of a prefill tile are split over workgroups: returns the most chunks a tile can
+// have (1: no splitting) and the keys per chunk. With fewer tiles than the chip has room for,
+// long tiles are cut so that there are about a thousand units of work of similar size.
 // tile_rows: 0 (choose), 64 or 128; *tile_rows_out is the choice, to be given to tw_attn_prefill.
 extern "C" int tw_attn_prefill_split(int n_seqs, int q_heads, int kv_heads, int max_q_len, int max_kv_len,
                                      int tile_rows_in, int* kv_chunk, int* tile_rows_out) {
