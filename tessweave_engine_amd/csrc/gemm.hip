@@ -37,7 +37,7 @@ __device__ __forceinline__ size_t tw_shuffled_chunk(int n, int c, int k_steps, i
 // partial sums go to partial[split][M][N] and splitk_reduce_kernel (or the caller's next
 // kernel) adds them, always in the same order, so results do not depend on timing.
 // =====================================================================================
-#define TW_XROW(U) ((U) * 64 + 16)          /* LDS bytes per activation row of a stage, padded */
+#define TW_XROW(U) ((U) * 64 + 32)          /* LDS bytes per activation row of a stage, padded: 32 * an odd number (see tw_lds_swz4) */
 
 // PARTIAL: always write float32 partial sums partial[split][M][N] (splits >= 1), no epilogue.
 // SHUF: W is in the shuffled layout (ldw = its k_steps): every weight load is 1 KB of consecutive
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(TW_CU_WAVES * 64) void gemm_stream_cu_kernel(
   };
 
   // ---- this wave's share of the activation copies: blocks wave, wave + WAVES, ... of every stage ----
-  const int row16 = lane >> 2, cswz = (lane & 3) ^ ((lane >> 4) & 3);
+  const int row16 = lane >> 2, cswz = (lane & 3) ^ tw_lds_swz4(row16);
   const T* x_row[XD];
   int x_chunk[XD], x_dst[XD];
 #pragma unroll
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(TW_CU_WAVES * 64) void gemm_stream_cu_kernel(
     }
     // ---- a wave with a tile of 16 columns --------------------------------------------------------------
     const T* w_row = W + ((size_t)min(tile, last_block) * ldw * 64 + lane) * EPF + (size_t)step_begin * 64 * EPF;
-    const int slot = (r * 4 + (g ^ ((r >> 2) & 3))) * 16;
+    const int slot = (r * 4 + (g ^ tw_lds_swz4(r))) * 16;
     f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};

@@ -15,17 +15,30 @@ __device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* l
   constexpr int WCOLS = 32 * WN;                             // columns of a wave tile
   constexpr int EROW = WCOLS + 4;                            // floats per staged row, padded
   // (the launcher asks for max(pipeline stages, 4 waves x 32 rows x EROW floats) bytes of LDS)
-  float* stage = reinterpret_cast<float*>(lds) + wave * 32 * EROW;
+  float* stage = reinterpret_cast<float*>(lds) + wave * 32 * EROW;   // (the GLU form below may lay its rows out differently)
   constexpr int CPR = WCOLS / 8;                             // 8-column groups per row
   const bool vec_ok = (ldc % 8 == 0) && (residual == nullptr || ldr % 4 == 0) &&
                       ((uintptr_t)C % 16 == 0) && ((uintptr_t)residual % 16 == 0);
+  // The GLU form reads its staged rows in another pattern: a lane takes 8 gate and 8 up values, 16 columns
+  // apart, and the lanes of a row take column groups that are 256 bytes (all 64 banks) apart. With padded
+  // rows those reads met 4-way bank conflicts (a quarter of the LDS time of a whole gate_up GEMM). Where a
+  // wave tile's row is a multiple of 256 bytes the rows are not padded and the 16-byte pieces of row lr lie
+  // at piece ^ (0, 1, 4, 5)[lr % 4]: the 16 lanes that a 16-byte read serves in one pass (four rows, four
+  // column groups each) then find 16 different 16-byte columns.
+  constexpr bool SWIZZLED = GLU && WCOLS % 64 == 0;
+  constexpr int SROW = SWIZZLED ? WCOLS : EROW;
+  if (SWIZZLED) stage = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
+  auto swz = [](int row) { return SWIZZLED ? ((row & 1) | ((row & 2) << 1)) : 0; };
 #pragma unroll
   for (int i = 0; i < WM; ++i) {
     __syncthreads();                                          // the pipeline's (or the last round's) LDS reads are done
 #pragma unroll
     for (int j = 0; j < WN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) stage[(8 * (e / 4) + 4 * g + (e % 4)) * EROW + j * 32 + r] = acc[i][j][e];
+      for (int e = 0; e < 16; ++e) {
+        const int srow = 8 * (e / 4) + 4 * g + (e % 4);
+        stage[srow * SROW + (((j * 8 + (r >> 2)) ^ swz(srow)) << 2) + (r & 3)] = acc[i][j][e];
+      }
     __syncthreads();
     if (GLU) {
       // a wave tile's columns are [gate 16 | up 16] pairs; a lane forms 8 outputs of one row
@@ -36,12 +49,24 @@ __device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* l
         const int lc = (og >> 1) * 32 + (og & 1) * 8;         // gate columns lc.., up columns lc + 16..
         const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
         if (row >= M || col + 24 > N) continue;               // N is a multiple of 32: groups are whole
-        float v[8];
+        float v[8], gv[8], uv[8];
+        if (SWIZZLED) {
+          const float* base = stage + lr * SROW;
+          const int piece = lc >> 2, x = swz(lr);
+          const f32x4 g0 = *reinterpret_cast<const f32x4*>(base + ((piece ^ x) << 2));
+          const f32x4 g1 = *reinterpret_cast<const f32x4*>(base + (((piece + 1) ^ x) << 2));
+          const f32x4 u0 = *reinterpret_cast<const f32x4*>(base + (((piece + 4) ^ x) << 2));
+          const f32x4 u1 = *reinterpret_cast<const f32x4*>(base + (((piece + 5) ^ x) << 2));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { gv[e] = g0[e]; gv[4 + e] = g1[e]; uv[e] = u0[e]; uv[4 + e] = u1[e]; }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) { gv[e] = stage[lr * SROW + lc + e]; uv[e] = stage[lr * SROW + lc + 16 + e]; }
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          float gv = stage[lr * EROW + lc + e], uv = stage[lr * EROW + lc + 16 + e];
-          if (bias) { gv += bias[col + e]; uv += bias[col + 16 + e]; }
-          v[e] = tw_silu(gv) * uv;
+          if (bias) { gv[e] += bias[col + e]; uv[e] += bias[col + 16 + e]; }
+          v[e] = tw_silu(gv[e]) * uv[e];
         }
         OutT* dst = C + (size_t)row * ldc + (n0 + wn0) / 2 + (og >> 1) * 16 + (og & 1) * 8;
         if (ldc % 8 == 0 && (uintptr_t)C % 16 == 0) {
