@@ -171,7 +171,7 @@ struct RowTile {
 // =====================================================================================
 template <typename T, int DTMAX>
 __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
-  __shared__ float lds_o[3][16][DTMAX * 16];
+  __shared__ __attribute__((aligned(16))) float lds_o[3][16][DTMAX * 16 + 8];   // (rows of 32 bytes more than a multiple of 256: see tw_lds_swz4)
   __shared__ float lds_ml[3][16][2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -283,7 +283,7 @@ template <bool V> struct BoolTag { static constexpr bool value = V; };
 template <int DTMAX, bool EXACT>
 __global__ __launch_bounds__(256) void attn_decode_bf16_kernel(AttnArgs a) {
   constexpr int NSMAX = AttnShape<bf16_t, DTMAX>::NSMAX;
-  __shared__ float lds_o[3][16][DTMAX * 16];
+  __shared__ __attribute__((aligned(16))) float lds_o[3][16][DTMAX * 16 + 8];   // (rows of 32 bytes more than a multiple of 256: see tw_lds_swz4)
   __shared__ float lds_ml[3][16][2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
