@@ -25,6 +25,27 @@ __device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* l
   // wave tile's row is a multiple of 256 bytes the rows are not padded and the 16-byte pieces of row lr lie
   // at piece ^ (0, 1, 4, 5)[lr % 4]: the 16 lanes that a 16-byte read serves in one pass (four rows, four
   // column groups each) then find 16 different 16-byte columns.
+  // Bias: a lane's group of 8 columns in its round t of a pass through LDS is group (lane + 64 t) % CPR of
+  // the row, which repeats after NB rounds (1 where 64 is a multiple of the groups per row, 3 for 12 groups).
+  // Those NB groups' bias is read once, before the first barrier, instead of eight values at a time in front of
+  // every store (a fifth of a qkv projection's time at 2,048 rows went there).
+  constexpr int NB = 64 % CPR == 0 ? 1 : ((128 % CPR == 0) ? 2 : 3);
+  static_assert((64 * NB) % CPR == 0, "the column groups of a lane repeat after NB rounds");
+  float lane_bias[NB][8];
+  if (!GLU && bias) {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const int col = n0 + wn0 + ((lane + 64 * b) % CPR) * 8;
+      if (col + 8 <= N && (uintptr_t)bias % 16 == 0) {
+        const f32x4 b0 = *reinterpret_cast<const f32x4*>(bias + col), b1 = *reinterpret_cast<const f32x4*>(bias + col + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { lane_bias[b][e] = b0[e]; lane_bias[b][4 + e] = b1[e]; }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) lane_bias[b][e] = col + e < N ? bias[col + e] : 0.f;
+      }
+    }
+  }
   constexpr bool SWIZZLED = GLU && WCOLS % 64 == 0;
   constexpr int SROW = SWIZZLED ? WCOLS : EROW;
   if (SWIZZLED) stage = reinterpret_cast<float*>(lds) + wave * 32 * SROW;
@@ -87,7 +108,8 @@ __device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* l
       continue;
     }
 #pragma unroll
-    for (int q = lane; q < 32 * CPR; q += 64) {
+    for (int t = 0; t < 32 * CPR / 64; ++t) {
+      const int q = lane + 64 * t;
       const int lr = q / CPR, lc = (q % CPR) * 8;
       const int row = m0 + wm0 + i * 32 + lr, col = n0 + wn0 + lc;
       if (row >= M || col >= N) continue;
@@ -96,8 +118,7 @@ __device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* l
       for (int e = 0; e < 8; ++e) v[e] = stage[lr * EROW + lc + e];
       if (bias) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (col + e < N) v[e] += bias[col + e];
+        for (int e = 0; e < 8; ++e) v[e] += lane_bias[t % NB][e];
       }
       if (vec_ok && col + 8 <= N) {
         if (residual) {
