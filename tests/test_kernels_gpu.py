@@ -647,7 +647,10 @@ def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window, n, q_len):
     q = q_one[None].expand(q_len, heads, d).contiguous()
     want = plain.attention(q.float(), k, v, torch.arange(n - q_len, n), window=window or None)
     q_start = torch.tensor([0, q_len], dtype=torch.int32, device=device)
-    for generic, chunk, tile_rows in ((False, 0, 64), (False, 0, 128), (True, 0, 0), (False, 32, 128), (False, 96, 64)):
+    ways = [(False, 0, 64), (False, 0, 128), (True, 0, 0), (False, 32, 128), (False, 96, 64)]
+    if n >= 1000:                          # chunks long enough for the fast kernel's main loop, merged afterwards
+        ways += [(False, 512, 128), (False, 384, 64)]
+    for generic, chunk, tile_rows in ways:
         out = torch.full((q_len, heads * d), float("nan"), dtype=dtype, device=device)
         split = (math.ceil((n + 31) / chunk) + 1 if chunk else 1, chunk, tile_rows)
         ws = torch.full((ops.attn_prefill_workspace_floats(q_len, heads, d, split[0]),), float("nan"),
