@@ -958,14 +958,15 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
         m[rt] = m_new;
         m_use[rt] = use;
         m_thr[rt] = (m_new + TW_PF_SLACK) / c2;
-        // The output lives in accumulation registers, which only MFMAs and moves can name. Written as
-        // plain multiplications, the compiler moves all of it into vector registers at the top of EVERY
-        // iteration, for the sake of this branch that is hardly ever taken. As opaque code the moves
-        // stay in here.
+        // Where the output fits the vector registers (the kernels that work on two blocks at a time) it
+        // is scaled as it stands. In the kernels with the largest heads it lives in accumulation registers,
+        // which only MFMAs and moves can name: written as plain multiplications, the compiler moves all
+        // of it into vector registers at the top of EVERY iteration, for the sake of this branch that is
+        // hardly ever taken; as opaque code the moves stay in here.
 #pragma unroll
         for (int dt = 0; dt < DTMAX; ++dt) {
           if constexpr (PIPELINED) {
-            acc[rt][dt] *= alpha;                            // (these kernels' accumulators are in vector registers)
+            acc[rt][dt] *= alpha;
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
