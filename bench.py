@@ -74,6 +74,9 @@ def parse():
                    help="instead: continuous batching of --requests requests (prompts of 128..4096 tokens, 256 "
                         "generated each, Poisson arrivals at --rate a second, prompt portions of 512)")
     p.add_argument("--requests", type=int, default=64)
+    p.add_argument("--prefill-chunk", type=int, default=512,
+                   help="with --serve: the largest prompt portion in one step (larger: more prompt tokens a second and "
+                        "a shorter time to the first token, longer steps for the requests that are decoding)")
     p.add_argument("--rate", type=float, default=16.0, help="mean arrivals a second (0: all at once)")
     return p.parse_args()
 
@@ -132,7 +135,7 @@ def serve_run(model, torch, args):
     from tessweave_engine_amd.config import EngineConfig
     from tessweave_engine_amd.engine import Engine
 
-    page, chunk, outputs, longest = 16, 512, 256, 4096
+    page, chunk, outputs, longest = 16, args.prefill_chunk, 256, 4096
     n, active = args.requests, min(args.requests, 64)
     config = EngineConfig(block_size=page, kv_blocks=active * ((longest + outputs) // page + 1),
                           max_context=longest + outputs, max_active=active, max_queue=n, prefill_chunk=chunk,
