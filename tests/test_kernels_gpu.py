@@ -660,6 +660,50 @@ def test_attn_sharp_keys_at_edges(ops, device, dtype, page, window, n, q_len):
         torch.testing.assert_close(out.float().cpu().reshape(q_len, heads, d), want, **ATTN_TOL[dtype])
 
 
+def test_attn_prefill_random_shapes_with_long_key_ranges(ops, device):
+    """Two dozen random launches of the bfloat16 prompt attention (head sizes, groups, page sizes, one to three
+    sequences of up to 2,500 keys, whole prompts and portions, windows, both tile sizes, tiles cut into chunks
+    where the launcher would) against the plain implementation: the fast kernel's main loop runs from six
+    32-key blocks a tile on, which the small cases above hardly reach."""
+    import random
+    rng = random.Random(7)
+    dtype = torch.bfloat16
+    for case in range(24):
+        d = rng.choice([64, 128, 128, 128, 96, 256])
+        kvh = rng.choice([1, 2, 4])
+        heads = kvh * rng.choice([1, 2, 4, 7])
+        page = rng.choice([8, 16, 16, 32, 64, 12, 48])
+        lengths, qlens = [], []
+        for _ in range(rng.choice([1, 1, 2, 3])):
+            n = rng.choice([rng.randint(200, 700), rng.randint(700, 2500), rng.randint(33, 200)])
+            lengths.append(n)
+            qlens.append(rng.choice([n, rng.randint(1, min(n, 300)), rng.randint(1, n)]))
+        window = rng.choice([0, 0, 0, rng.randint(40, 900)])
+        gen = torch.Generator().manual_seed(case)
+        k = [(torch.randn(n, kvh, d, generator=gen) * 0.7).to(dtype).float() for n in lengths]
+        v = [torch.randn(n, kvh, d, generator=gen).to(dtype).float() for n in lengths]
+        keys, values, table = build_paged(k, v, lengths, page, sum(math.ceil(n / page) for n in lengths) + 5, device,
+                                          dtype, seed=case)
+        total_q = sum(qlens)
+        q = (torch.randn(total_q, heads, d, generator=gen) * 1.5).to(dtype)
+        want, q_start, row = [], [0], 0
+        for n, ql, kk, vv in zip(lengths, qlens, k, v):
+            want.append(plain.attention(q[row:row + ql].float(), kk, vv, torch.arange(n - ql, n), window=window or None))
+            row += ql
+            q_start.append(row)
+        buf = torch.zeros(total_q, (heads + 2 * kvh) * d, dtype=dtype, device=device)
+        buf[:, :heads * d] = q.reshape(total_q, -1).to(device)
+        out = torch.full((total_q, heads * d), float("nan"), dtype=dtype, device=device)
+        split = ops.attn_prefill_split(len(lengths), heads, kvh, max(qlens), max(lengths), tile_rows=rng.choice([0, 0, 64, 128]))
+        ws = torch.full((max(1, ops.attn_prefill_workspace_floats(total_q, heads, d, split[0])),), float("nan"), device=device)
+        ops.attn_prefill(buf, keys, values, table, torch.tensor(q_start, dtype=torch.int32, device=device),
+                         torch.tensor(lengths, dtype=torch.int32, device=device), 0, len(lengths), max(qlens), out, heads,
+                         kvh, d, d ** -0.5, window=window, split=split, workspace=ws)
+        torch.testing.assert_close(out.float().cpu().reshape(total_q, heads, d), torch.cat(want), **ATTN_TOL[dtype],
+                                   msg=lambda m: f"case {case}: d {d} heads {heads}/{kvh} page {page} lengths {lengths} "
+                                                 f"q {qlens} window {window} split {split}: {m}")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attn_soft_capped_scores(ops, device, dtype):
     """softcap * tanh(score / softcap) before the softmax, decode and prompt portions, against the formula in
