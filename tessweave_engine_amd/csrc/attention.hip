@@ -1559,6 +1559,7 @@ static int prefill_launch(AttnArgs a, int n_seqs, int max_q_len, int generic, hi
     if (a.head_dim < 64) return prefill_bf16_launch<4, false>(a, n_seqs, max_q_len, stream);
     if (a.head_dim == 128) return prefill_bf16_launch<8, true>(a, n_seqs, max_q_len, stream);
     if (a.head_dim < 128) return prefill_bf16_launch<8, false>(a, n_seqs, max_q_len, stream);
+    if (a.head_dim == 256) return prefill_bf16_launch<16, true>(a, n_seqs, max_q_len, stream);
     return prefill_bf16_launch<16, false>(a, n_seqs, max_q_len, stream);
   }
   const int G = a.q_heads / a.kv_heads;
