@@ -1501,6 +1501,8 @@ static int decode_launch(AttnArgs a, int n_seqs, int generic, hipStream_t stream
       attn_decode_bf16_kernel<8, true><<<grid, 256, 0, stream>>>(a);
     else if (a.head_dim < 128)
       attn_decode_bf16_kernel<8, false><<<grid, 256, 0, stream>>>(a);
+    else if (a.head_dim == 256)
+      attn_decode_bf16_kernel<16, true><<<grid, 256, 0, stream>>>(a);
     else
       attn_decode_bf16_kernel<16, false><<<grid, 256, 0, stream>>>(a);
   } else if (a.head_dim <= 64)
