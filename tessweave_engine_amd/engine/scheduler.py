@@ -262,7 +262,9 @@ class Engine:
                 else:
                     tokens = r.tokens[begin:begin + p.count]
                 entries.append(StepEntry(r.seq, tokens, [p.count - 1] if p.samples else []))
-            logits = self.stepper.step(entries)
+            # (with lookahead everything of a turn is issued on the step's own stream: nothing waits for another stream)
+            with (self._sampling_stream() if self.lookahead else contextlib.nullcontext()):
+                logits = self.stepper.step(entries)
             self._publish_prompt_blocks(portions)
             sampled = [p for p in portions if p.samples]
             arguments = (logits, [p.request.temperature for p in sampled], [p.request.seed for p in sampled],
