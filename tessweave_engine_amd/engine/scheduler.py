@@ -262,8 +262,8 @@ class Engine:
                 else:
                     tokens = r.tokens[begin:begin + p.count]
                 entries.append(StepEntry(r.seq, tokens, [p.count - 1] if p.samples else []))
-            # (with lookahead everything of a turn is issued on the step's own stream: nothing waits for another stream)
-            with (self._sampling_stream() if self.lookahead else contextlib.nullcontext()):
+            # (everything of a turn is issued on the step's own stream: nothing waits for another stream)
+            with self._sampling_stream():
                 logits = self.stepper.step(entries)
             self._publish_prompt_blocks(portions)
             sampled = [p for p in portions if p.samples]
@@ -278,7 +278,8 @@ class Engine:
                     pending = self.sampler.sample_async(*arguments)
                 self._inflight = (pending, [(p.request, i) for i, p in enumerate(sampled)])
             else:
-                ids = self.sampler.sample(*arguments)
+                with self._sampling_stream():
+                    ids = self.sampler.sample(*arguments)
                 self._inflight = (ids, [(p.request, i) for i, p in enumerate(sampled)])
             for i, p in enumerate(sampled):
                 p.request.issued += 1
