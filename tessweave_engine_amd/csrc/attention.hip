@@ -766,8 +766,8 @@ __global__ __launch_bounds__(256) void attn_prefill_bf16_kernel(AttnArgs a) {
     k_slot[i] = P >= 32 ? 0 : (key_c >> pshift);           // which of the block's pages
     k_goff[i] = (P >= 32 ? key_c : (key_c & pmask)) * D + chunk_c * 8;
     // key k lies in LDS row (k / 8 % 4) * 4 + k % 4 + 16 * (k / 4 % 2): the 16 keys whose scores one MFMA
-    // forms (k % 8 < 4, or >= 4) are 16 consecutive rows, which with the odd row length (in 16-byte units)
-    // a fragment read finds in 16 different 16-byte columns of the banks
+    // forms (k % 8 < 4, or >= 4) are 16 consecutive rows, which with the row length KROW a fragment read
+    // finds in 16 different 16-byte columns of the banks (see tw_lds_swz4)
     k_loff[i] = (((key >> 3) & 3) * 4 + (key & 3) + 16 * ((key >> 2) & 1)) * KROW + chunk * 16;
   }
 #pragma unroll
